@@ -1,0 +1,239 @@
+#!/usr/bin/env python3
+"""Benchmark of the BGEMM / BWTA hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--all]
+
+A step is one pass of the hot path over one batch of synthetic input: one 8192^3
+{-1,1}x{-1,1} BGEMM on prepacked operands (BASELINE config 5, the compute-bound case the
+metric's target is quoted on), int32 output, operands resident in HBM before the timed
+region.  One JSON line goes to stdout; `value` is effective binary TOPS = 2*M*N*K / t
+(the reference drivers' own op count, lowbit_kernel/csrc/benchmark.cu:291).  With --all the
+line also carries the other BASELINE configurations (MLP forward, batched attention A x V,
+decode-shape BWTA) under "all_configs".
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "bgemm-cuda_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+INT8_MFMA_PEAK_TOPS = 5000.0      # MI355X dense int8 MFMA, published
+HBM_PEAK_GBS = 8000.0             # MI355X HBM3E, published
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def time_gpu(fn, warmup, steps):
+    """Average milliseconds per call of fn(i), timed with events on the launch stream."""
+    import torch
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(steps):
+        fn(i)
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps
+
+
+def pm1_f16(shape, seed, device):
+    import torch
+    g = torch.Generator(device=device).manual_seed(seed)
+    bits = torch.randint(0, 2, shape, generator=g, device=device, dtype=torch.int8)
+    return (1 - 2 * bits).to(torch.half)
+
+
+def check_sampled(out, w16, x16, n_rows=64, n_cols=64):
+    """Spot parity check of an [N,M] XOR result against the fp32 closed form on sampled rows."""
+    import torch
+    N, M = out.shape
+    g = torch.Generator().manual_seed(7)
+    rs = torch.randperm(M, generator=g)[:n_rows].to(out.device)
+    cs = torch.randperm(N, generator=g)[:n_cols].to(out.device)
+    want = (x16[cs].float().cpu() @ w16[rs].float().cpu().T).to(torch.int32)
+    return bool(torch.equal(out[cs][:, rs].cpu(), want))
+
+
+def bench_c5(steps, warmup, M=8192, N=8192, K=8192, splitK=1, variant=0):
+    import torch
+    import lowbit_kernel as lk
+    dev = torch.device("cuda:0")
+    w16, x16 = pm1_f16((M, K), 5001, dev), pm1_f16((N, K), 5002, dev)
+    wp, xp = lk.pack_sign(w16), lk.pack_sign(x16)
+    out = torch.empty((1, N, M), dtype=torch.int32, device=dev)
+    fn = lambda i: lk.bgemm_packed_forward(wp, xp, lk.MODE_XOR, torch.int32, splitK, variant, out=out)
+    ms = time_gpu(fn, warmup, steps)
+    ok = check_sampled(out[0], w16, x16)
+    ops = 2.0 * M * N * K
+    bytes_alg = M * K / 8 + N * K / 8 + 4.0 * M * N
+    pack_ms = time_gpu(lambda i: lk.pack_sign(x16), 2, 10)
+    return {"name": "C5 BGEMM %dx%dx%d xor int32 splitK=%d" % (M, N, K, splitK), "ms": ms,
+            "tops": ops / ms / 1e9, "gbs": bytes_alg / ms / 1e6, "ops": ops, "bytes": bytes_alg,
+            "bit_exact": ok, "act_pack_ms": pack_ms}, (w16, x16)
+
+
+def cpu_baseline_c5(w16, x16, budget_s=12.0):
+    """Reference CPU path (torch matmul on +-1 fp32 tensors) on a bounded column slice."""
+    import torch
+    from oracle import oracle
+    torch.set_num_threads(max(1, min(os.cpu_count() or 1, 16)))
+    M, K = w16.shape
+    wf = w16.float().cpu()
+    n = 64
+    xf = x16[:n].float().cpu()
+    t0 = time.perf_counter()
+    oracle.cpu_path_linear(xf, wf)
+    dt = max(time.perf_counter() - t0, 1e-4)
+    n = int(min(x16.shape[0], max(64, n * budget_s / dt / 3)))
+    xf = x16[:n].float().cpu()
+    oracle.cpu_path_linear(xf, wf)                       # warm-up at the timed size
+    reps, t0 = 0, time.perf_counter()
+    while reps < 2 or time.perf_counter() - t0 < budget_s / 2:
+        oracle.cpu_path_linear(xf, wf)
+        reps += 1
+    dt = (time.perf_counter() - t0) / reps
+    return {"value": 2.0 * M * n * K / dt / 1e12, "unit": "TOPS", "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": "torch.matmul fp32 on +-1 tensors, W[%d,%d] x X[%d,%d] (%d of %d activation rows), %d reps"
+                      % (M, K, n, K, n, x16.shape[0], reps)}
+
+
+def bench_c4(steps, warmup, N, splitK, variant=0, copies=64):
+    """Decode-shape BWTA linear: W[11008,4096] prepacked, ternary activations, weights rotated
+    over `copies` buffers (> 256 MB in total) so no launch finds its weights in cache."""
+    import torch
+    import lowbit_kernel as lk
+    dev = torch.device("cuda:0")
+    M, K = 11008, 4096
+    g = torch.Generator(device=dev).manual_seed(4000 + N)
+    t = torch.randint(0, 4, (N, K), generator=g, device=dev)
+    x16 = torch.where(t == 0, -1.0, torch.where(t == 3, 1.0, 0.0)).to(torch.half)      # p(0) = 0.5
+    xt = lk.pack_ternary(x16)
+    w16 = pm1_f16((M, K), 4001, dev)
+    base = lk.pack_sign(w16)
+    wps = [lk.PackedBits(base.data.clone(), None, 1, M, K) for _ in range(copies)]
+    out = torch.empty((1, N, M), dtype=torch.int32, device=dev)
+    fn = lambda i: lk.bgemm_packed_forward(wps[i % copies], xt, lk.MODE_BWTA, torch.int32, splitK, variant, out=out)
+    ms = time_gpu(fn, warmup, steps)
+    want = (torch.sign(x16.float()).cpu() @ w16.float().cpu().T).to(torch.int32)
+    ok = bool(torch.equal(out[0].cpu(), want))
+    ops = 2.0 * M * N * K
+    bytes_alg = M * K / 8 + 2 * N * K / 8 + 4.0 * M * N
+    return {"name": "C4 BWTA W[11008,4096] N=%d splitK=%d" % (N, splitK), "ms": ms, "tops": ops / ms / 1e9,
+            "gbs": bytes_alg / ms / 1e6, "ops": ops, "bytes": bytes_alg, "bit_exact": ok}
+
+
+def bench_c3(steps, warmup, variant=0):
+    """192 x ([512,512] {0,1} x [512,64] {-1,1}) -> int32 [192,512,64]."""
+    import torch
+    import lowbit_kernel as lk
+    dev = torch.device("cuda:0")
+    B, S, D = 192, 512, 64
+    attn16 = pm1_f16((B, S, S), 3001, dev)                 # sign bit clear = 1
+    v16 = pm1_f16((B, S, D), 3002, dev)
+    ap, vp = lk.pack_sign(attn16), lk.pack_sign(v16.transpose(1, 2).contiguous())
+    out = torch.empty((B, S, D), dtype=torch.int32, device=dev)
+    fn = lambda i: lk.bgemm_packed_forward(vp, ap, lk.MODE_ATTN_X, torch.int32, 1, variant, out=out)
+    ms = time_gpu(fn, warmup, steps)
+    want = torch.bmm((attn16[:4] > 0).float(), v16[:4].float()).to(torch.int32)
+    ok = bool(torch.equal(out[:4], want))
+    ops = 2.0 * B * S * S * D
+    bytes_alg = B * (S * S / 8 + S * D / 8 + 4.0 * S * D)
+    return {"name": "C3 attention AxV 192x[512,512]x[512,64]", "ms": ms, "tops": ops / ms / 1e9,
+            "gbs": bytes_alg / ms / 1e6, "ops": ops, "bytes": bytes_alg, "bit_exact": ok}
+
+
+def bench_c2(steps, warmup):
+    """3-layer binarised MLP forward 784->4096->4096->10, batch 128, through the fp16 drop-in call."""
+    import torch
+    import lowbit_kernel as lk
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(2001)
+    dims = [784, 4096, 4096, 10]
+    x = torch.randn(128, 784, generator=g, device=dev).half()
+    Ws = [torch.randn(dims[i + 1], dims[i], generator=g, device=dev).half() for i in range(3)]
+    sws = [(W.float().norm(1, 1) / W.numel()).half() for W in Ws]
+    sa = torch.tensor(1.0, device=dev).half()
+
+    def fwd(i):
+        h = x
+        for W, sw in zip(Ws, sws):
+            h = lk.bgemm_linear_forward_cuda(h, W, 1, 1) * sw * sa
+        return h
+    ms = time_gpu(fwd, warmup, steps)
+    ops = 2.0 * 128 * (784 * 4096 + 4096 * 4096 + 4096 * 10)
+    return {"name": "C2 MLP 784-4096-4096-10 batch 128 (fp16 in/out, packs per call)", "ms": ms,
+            "tops": ops / ms / 1e9, "ops": ops}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--all", action="store_true", help="also time the other BASELINE configurations")
+    ap.add_argument("--variant", type=int, default=0, help="0 auto, 1 VALU, 2 MFMA")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build targets one GPU (its boxes have one); run with --gpus 1")
+
+    import torch
+    import _lib
+    _lib.lib()          # fail loudly if the HIP library is missing
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+
+    c5, (w16, x16) = bench_c5(args.steps, args.warmup, variant=args.variant)
+    log("C5:", json.dumps(c5))
+    cpu = None if args.no_cpu else cpu_baseline_c5(w16, x16)
+    del w16, x16
+    extra = []
+    if args.all:
+        for N in (1, 4, 16):
+            for sk in (1, 8):
+                extra.append(bench_c4(2000, 200, N, sk))
+                log(json.dumps(extra[-1]))
+        extra.append(bench_c3(200, 20))
+        log(json.dumps(extra[-1]))
+        extra.append(bench_c2(200, 20))
+        log(json.dumps(extra[-1]))
+        for (K, N) in [(4096, 256), (4096, 2048), (16384, 256), (16384, 2048)]:
+            for sk in (1, 2, 4):
+                r, _ = bench_c5(20, 3, 8192, N, K, sk)
+                extra.append(r)
+                log(json.dumps(r))
+        for r in extra:
+            r["frac_int8_mfma"] = r["tops"] / INT8_MFMA_PEAK_TOPS
+            if "gbs" in r:
+                r["frac_hbm"] = r["gbs"] / HBM_PEAK_GBS
+
+    line = {
+        "metric": "effective binary TOPS (2*M*N*K/t), bit-exact int32",
+        "value": c5["tops"], "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": c5["ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8 MFMA on 1-bit operands, int32 accumulate", "data": "synthetic",
+        "config": {"workload": "BASELINE config 5: BGEMM M=N=K=8192, {-1,+1}x{-1,+1}, weights and activations "
+                               "prepacked (tiled bit layout), int32 output, splitK=1",
+                   "bit_exact_sampled": c5["bit_exact"], "hbm_gbs_algorithmic": c5["gbs"],
+                   "activation_pack_ms": c5["act_pack_ms"]},
+        "roofline": {"bound": "mfma", "achieved": c5["tops"], "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOP/s",
+                     "frac": c5["tops"] / INT8_MFMA_PEAK_TOPS, "traffic": None},
+        "cpu_baseline": cpu,
+    }
+    if extra:
+        line["all_configs"] = extra
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,66 @@
+"""ctypes binding of libbgemm_mi355x.so (the C ABI declared in include/bgemm_mi355x.h).
+
+The library must have been built (``python _build.py`` or ``__graft_entry__.build()``);
+there is no CPU fallback: a missing library raises ImportError.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+SO_PATH = os.path.join(_HERE, "libbgemm_mi355x.so")
+
+OK, EINVAL, ENULL, EWORKSPACE, ELAUNCH, EALIGN = 0, -1, -2, -3, -4, -5
+MODE_AND, MODE_XOR, MODE_ATTN, MODE_BWTA, MODE_ATTN_X = 0, 1, 2, 3, 4
+OUT_I32, OUT_F16 = 0, 1
+VARIANT_AUTO, VARIANT_VALU, VARIANT_MFMA = 0, 1, 2
+
+_i64, _p, _int, _sz = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+
+# symbol -> (restype, argtypes); mirrors include/bgemm_mi355x.h one to one
+SIGNATURES = {
+    "bgemm_last_error": (ctypes.c_char_p, []),
+    "bgemm_abi_version": (_int, []),
+    "bgemm_tiled_words": (_i64, [_i64, _i64]),
+    "bgemm_pack_sign_f16": (_int, [_p, _i64, _i64, _i64, _p, _p]),
+    "bgemm_pack_sign_f16_logical": (_int, [_p, _i64, _i64, _i64, _p, _p]),
+    "bgemm_pack_ternary_f16": (_int, [_p, _i64, _i64, _i64, _p, _p, _p]),
+    "bgemm_tile_from_logical": (_int, [_p, _i64, _i64, _p, _p]),
+    "bgemm_logical_from_tiled": (_int, [_p, _i64, _i64, _p, _p]),
+    "bgemm_packed_workspace_bytes": (_sz, [_int, _i64, _i64, _i64, _i64, _int, _int]),
+    "bgemm_packed_forward": (_int, [_int, _p, _p, _p, _p, _int, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
+                                    _int, _int, _p, _sz, _p]),
+    "bgemm_f16_workspace_bytes": (_sz, [_i64, _i64, _i64, _int]),
+    "bgemm_f16_workspace_zero_bytes": (_sz, [_i64, _i64, _i64, _int]),
+    "bgemm_f16_forward": (_int, [_p, _p, _p, _i64, _i64, _i64, _p, _sz, _int, _int, _p]),
+}
+
+_lib = None
+
+
+def lib():
+    """Loads the shared library once and types every entry point."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(SO_PATH):
+            raise ImportError("%s is missing: build it with `python %s`" %
+                              (SO_PATH, os.path.join(_HERE, "_build.py")))
+        L = ctypes.CDLL(SO_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(L, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = L
+    return _lib
+
+
+class BgemmError(RuntimeError):
+    pass
+
+
+def check(rc):
+    """Turns a negative status into the Python exception the reference's asserts map to."""
+    if rc == OK:
+        return
+    msg = lib().bgemm_last_error().decode() or "error %d" % rc
+    if rc in (EINVAL, ENULL, EALIGN, EWORKSPACE):
+        raise ValueError(msg)
+    raise BgemmError(msg)

@@ -1,0 +1,252 @@
+"""Binary Linear / matmul layers over the MI355X BGEMM library.
+
+Host-side mirror of the reference's layer file (tests/python/bgemm_linear.py): the same
+class and function names, argument meaning and forward arithmetic, calling
+``lowbit_kernel.bgemm_linear_forward_cuda`` exactly where the reference does.  Supersets:
+any batch size (the reference asserts ``x.shape[0] % 32 == 0``, bgemm_linear.py:475),
+inputs with leading batch dimensions, non-contiguous operands, and an inference cache of
+the bit-packed weight.
+"""
+import math
+
+import torch
+import torch.nn as nn
+
+import lowbit_kernel
+
+__all__ = ['BNNLinear', 'BGEMMLinear', 'BGEMMLinear_elastic_signed', 'bgemm_matmul', 'bgemm_attn_matmul',
+           'BGEMMLinear_bireal', 'NNLinear_elastic_signed', 'bgemm_linear', 'bgemm_linear_bireal',
+           'bgemm_linear_elastic_signed', 'nn_linear_elastic_signed', 'BinActive', 'ternary']
+
+
+def _instr(instruction):
+    return lowbit_kernel.AND_POP if instruction == 'and' else lowbit_kernel.XOR_POP
+
+
+def _kernel_2d(x, w, instr):
+    """fp16 [..., K] x fp16 [M, K] -> fp16 [..., M] through the drop-in entry point."""
+    lead = x.shape[:-1]
+    out = lowbit_kernel.bgemm_linear_forward_cuda(x.reshape(-1, x.shape[-1]), w, 1, instr)
+    return out.reshape(*lead, w.shape[0])
+
+
+def _linear_grads(grad_out, x_sign, w_sign):
+    """Straight-through gradients of out = x_sign @ w_sign.T (bgemm_linear.py:149-165)."""
+    g = grad_out.to(x_sign.dtype)
+    grad_x = g @ w_sign
+    grad_w = g.reshape(-1, g.shape[-1]).T @ x_sign.reshape(-1, x_sign.shape[-1])
+    return grad_x, grad_w
+
+
+class bgemm_matmul(torch.autograd.Function):
+    """matA [.., N, K] @ matB [K, M] with both operands binarised by sign (bgemm_linear.py:9-42)."""
+
+    @staticmethod
+    def forward(ctx, matA, matB, instruction='xor'):
+        matA, matB = matA.to(torch.half), matB.to(torch.half)
+        ctx.save_for_backward(matA, matB)
+        return _kernel_2d(matA, matB.transpose(-1, -2).contiguous(), _instr(instruction))
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        matA, matB = ctx.saved_tensors
+        grad_a, grad_bt = _linear_grads(grad_output, matA.sign(), matB.sign().transpose(-1, -2))
+        return grad_a, grad_bt.transpose(-1, -2), None
+
+
+class bgemm_attn_matmul(torch.autograd.Function):
+    """attn [S_q, S_k] ({0,1}: 1 where the sign bit is clear) @ value [S_k, d] ({-1,1})
+    (bgemm_linear.py:45-86).  The kernel sees attn as the weight-side operand with INSTR=2."""
+
+    @staticmethod
+    def forward(ctx, input1, input2, instruction="attn_mm"):
+        input1, input2 = input1.to(torch.half), input2.to(torch.half)
+        ctx.save_for_backward(input1, input2)
+        vt = input2.transpose(-1, -2).contiguous()
+        return lowbit_kernel.bgemm_linear_forward_cuda(vt, input1, 1, lowbit_kernel.ATTN_MM).T
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        attn, value = ctx.saved_tensors
+        a01 = (attn.sign() + 1) / 2
+        a01 = torch.where(a01 == 0, torch.ones_like(a01), a01)     # as the reference does (:70-71)
+        v = value.sign()
+        g = grad_output.to(v.dtype)
+        return (g @ v.T) / 2, a01.T @ g, None
+
+
+class bgemm_linear(torch.autograd.Function):
+    """out = sign(input) @ sign(weight).T on the binary kernel (bgemm_linear.py:131-165)."""
+
+    @staticmethod
+    def forward(ctx, input, weight, instruction='xor'):
+        input, weight = input.to(torch.half), weight.to(torch.half)
+        ctx.save_for_backward(input, weight)
+        return _kernel_2d(input, weight, _instr(instruction))
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        x, w = ctx.saved_tensors
+        grad_x, grad_w = _linear_grads(grad_output, x.sign(), w.sign())
+        return grad_x, grad_w, None
+
+
+class bgemm_linear_bireal(torch.autograd.Function):
+    """As bgemm_linear with the Bi-Real surrogate 2 - 2|x| on the input gradient (:168-219)."""
+
+    @staticmethod
+    def forward(ctx, input, weight, instruction='xor'):
+        input, weight = input.to(torch.half), weight.to(torch.half)
+        ctx.save_for_backward(input, weight)
+        return _kernel_2d(input, weight, _instr(instruction))
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        x, w = ctx.saved_tensors
+        grad_x, grad_w = _linear_grads(grad_output, x.sign(), w.sign())
+        return grad_x * (2 - 2 * x.abs().clamp(max=1)), grad_w, None
+
+
+def ternary(x, is_act=True):
+    """The reference's ternariser is plain sign (bgemm_linear.py:222-241)."""
+    return x.sign()
+
+
+def calculate_gradient_signed(qx, grad, grad_scale, is_act):
+    """Scale gradient of the elastic quantiser (bgemm_linear.py:519-535)."""
+    if is_act:
+        small, big = (qx < -1).float(), (qx > 1).float()
+        middle = 1.0 - small - big
+        inner = big - small + middle * (ternary(qx, True) - qx)
+    else:
+        inner = ternary(qx, False)
+    return grad, (inner * grad * grad_scale).sum(dim=-1).unsqueeze(dim=0)
+
+
+def _elastic_prepare(input, weight, sa):
+    x = input - input.mean().item()
+    w = weight - weight.mean().item()
+    return x / sa, w
+
+
+def _elastic_backward(ctx, grad_output, surrogate, clip):
+    x, w = ctx.saved_tensors
+    grad_x, grad_w = _linear_grads(grad_output, ternary(x, True), ternary(w, False))
+    grad_x, grad_sa = calculate_gradient_signed(x, grad_x, ctx.other, True)
+    _, grad_sw = calculate_gradient_signed(w, grad_w, ctx.other, False)
+    grad_x = grad_x * surrogate(x.abs().clamp(max=clip))
+    grad_w = grad_w * surrogate(w.abs().clamp(max=clip))
+    return grad_x, grad_w, grad_sa, grad_sw, None, None
+
+
+class nn_linear_elastic_signed(torch.autograd.Function):
+    """The CPU-runnable path: ternary(x) @ ternary(w).T in torch (bgemm_linear.py:243-347)."""
+
+    @staticmethod
+    def forward(ctx, input, weight, sa, sw, grad_scale, instruction="xor"):
+        x, w = _elastic_prepare(input, weight, sa)
+        ctx.other = grad_scale
+        ctx.save_for_backward(x, w)
+        xt, wt = ternary(x.to(torch.half), True), ternary(w.to(torch.half), False)
+        return (xt @ wt.T) * sa * sw
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        return _elastic_backward(ctx, grad_output, lambda t: 2 * torch.exp(-t ** 2), 1)
+
+
+class bgemm_linear_elastic_signed(torch.autograd.Function):
+    """Elastic-scale binary linear on the kernel (bgemm_linear.py:350-457)."""
+
+    @staticmethod
+    def forward(ctx, input, weight, sa, sw, grad_scale, instruction="xor"):
+        x, w = _elastic_prepare(input, weight, sa)
+        ctx.other = grad_scale
+        ctx.save_for_backward(x, w)
+        out = _kernel_2d(x.to(torch.half), w.to(torch.half), _instr(instruction))
+        return out * sa * sw
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        return _elastic_backward(ctx, grad_output, lambda t: 2 / torch.cosh(t) ** 2, 4)
+
+
+class BinActive(torch.autograd.Function):
+    """sign with 0 -> +1, identity gradient (bgemm_linear.py:599-616)."""
+
+    @staticmethod
+    def forward(ctx, input):
+        s = input.sign()
+        return torch.where(s == 0, torch.ones_like(s), s)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        return grad_output.clone()
+
+
+class _ScaledBinaryLinear(nn.Linear):
+    """Shared state of the binary Linear modules: lazily initialised scales and zero points
+    (bgemm_linear.py:466-472): sw = |w|_1 per output row / numel, sa = 2 mean|x|."""
+
+    def __init__(self, in_channels, out_channels, bias=False):
+        super().__init__(in_channels, out_channels, bias)
+        self.initialized = False
+
+    def _initialize(self, x, w):
+        assert not self.initialized, 'already initialized.'
+        self.sw = nn.Parameter(w.norm(1, 1).div(w.nelement()), requires_grad=True)
+        self.sa = nn.Parameter(2 * x.abs().mean(), requires_grad=True)
+        self.grad_scale = 1.0 / math.sqrt(x.numel())
+        self.zpw = torch.mean(w).detach()
+        self.zpa = torch.mean(x).detach()
+        self.initialized = True
+
+    def _add_bias(self, out):
+        if self.bias is not None:
+            out += self.bias.view(1, -1).expand_as(out)
+        return out
+
+
+class BGEMMLinear(_ScaledBinaryLinear):
+    """out = bgemm(x - zpa, w - zpw) * sw * sa (+ bias)  (bgemm_linear.py:460-486)."""
+    _fn = bgemm_linear
+
+    def forward(self, x):
+        if not self.initialized:
+            self._initialize(x, self.weight)
+        out = self._fn.apply(x - self.zpa, self.weight - self.zpw) * self.sw * self.sa
+        return self._add_bias(out)
+
+
+class BGEMMLinear_bireal(BGEMMLinear):
+    """BGEMMLinear with the Bi-Real backward (bgemm_linear.py:489-516)."""
+    _fn = bgemm_linear_bireal
+
+
+class BGEMMLinear_elastic_signed(_ScaledBinaryLinear):
+    """Learned-scale binary linear (bgemm_linear.py:538-564)."""
+    _fn = bgemm_linear_elastic_signed
+
+    def __init__(self, in_channels, out_channels, bias=True):
+        super().__init__(in_channels, out_channels, bias)
+
+    def forward(self, x):
+        if not self.initialized:
+            self._initialize(x, self.weight)
+        return self._add_bias(self._fn.apply(x, self.weight, self.sa, self.sw, self.grad_scale))
+
+
+class NNLinear_elastic_signed(BGEMMLinear_elastic_signed):
+    """Same layer on the torch CPU/GPU matmul path (bgemm_linear.py:569-595)."""
+    _fn = nn_linear_elastic_signed
+
+
+class BNNLinear(_ScaledBinaryLinear):
+    """Dense torch baseline: F.linear(BinActive(x - zpa), BinActive(w - zpw)) * sw * sa (:619-645)."""
+
+    def forward(self, x):
+        if not self.initialized:
+            self._initialize(x, self.weight)
+        bw = BinActive.apply(self.weight - self.zpw)
+        bx = BinActive.apply(x - self.zpa)
+        return nn.functional.linear(bx, bw, self.bias) * self.sw * self.sa

@@ -1,0 +1,157 @@
+// C ABI: argument checking, workspace carving, variant dispatch.
+#include "common.h"
+#include <string.h>
+
+namespace bgemm {
+
+static thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof g_err, fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int check_launch(const char* what)
+{
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(BGEMM_ELAUNCH, "%s: %s", what, hipGetErrorString(e));
+    return BGEMM_OK;
+}
+
+static size_t round256(size_t x) { return (x + 255) / 256 * 256; }
+
+// Split-K state: int32 running sums [batch][N][M], then one arrival counter per output tile
+// of the finest tiling any kernel uses (32 x 64 outputs).
+static size_t splitk_acc_bytes(int64_t batch, int64_t M, int64_t N) { return round256((size_t)batch * N * M * 4); }
+static size_t splitk_cnt_bytes(int64_t batch, int64_t M, int64_t N)
+{
+    return round256((size_t)batch * cdiv(N, 32) * cdiv(M, 64) * 4);
+}
+
+static int pick_variant(const GemmArgs& a)
+{
+    (void)a;
+    return BGEMM_VARIANT_MFMA;
+}
+
+}  // namespace bgemm
+
+using namespace bgemm;
+
+extern "C" const char* bgemm_last_error(void) { return g_err; }
+extern "C" int bgemm_abi_version(void) { return 1; }
+
+extern "C" size_t bgemm_packed_workspace_bytes(int mode, int64_t batch, int64_t M, int64_t N, int64_t K,
+                                               int splitK, int variant)
+{
+    (void)mode; (void)K; (void)variant;
+    if (splitK <= 1 || batch <= 0 || M <= 0 || N <= 0) return 0;
+    return splitk_acc_bytes(batch, M, N) + splitk_cnt_bytes(batch, M, N);
+}
+
+extern "C" int bgemm_packed_forward(int mode, const void* W_tiled, const void* X_tiled, const void* X2_tiled,
+                                    void* out, int out_dtype, int64_t batch, int64_t M, int64_t N, int64_t K,
+                                    int64_t strideW, int64_t strideX, int64_t strideC,
+                                    int splitK, int variant, void* ws, size_t ws_bytes, void* stream)
+{
+    g_err[0] = 0;
+    GemmArgs a;
+    memset(&a, 0, sizeof a);
+    if (!mode_coef(mode, &a.mc)) return fail(BGEMM_EINVAL, "bgemm_packed_forward: unknown mode %d", mode);
+    if (out_dtype != BGEMM_OUT_I32 && out_dtype != BGEMM_OUT_F16)
+        return fail(BGEMM_EINVAL, "bgemm_packed_forward: unknown output dtype %d", out_dtype);
+    if (variant < BGEMM_VARIANT_AUTO || variant > BGEMM_VARIANT_MFMA)
+        return fail(BGEMM_EINVAL, "bgemm_packed_forward: unknown variant %d", variant);
+    if (batch < 0 || M < 0 || N < 0 || K < 0 || splitK < 1 || splitK > 65535)
+        return fail(BGEMM_EINVAL, "bgemm_packed_forward: bad shape batch=%lld M=%lld N=%lld K=%lld splitK=%d",
+                    (long long)batch, (long long)M, (long long)N, (long long)K, splitK);
+    if (K >= (1LL << 24))   // keeps |C| below 2^24: exact in the fp32 step of the fp16 store
+        return fail(BGEMM_EINVAL, "bgemm_packed_forward: K=%lld exceeds 2^24-1", (long long)K);
+    if (batch > 0x7fffffff || M > 0x7fffffff || N > 0x7fffffff)
+        return fail(BGEMM_EINVAL, "bgemm_packed_forward: dimension too large");
+    if (strideW < 0 || strideX < 0 || strideC < 0 || (strideW & 3) || (strideX & 3))
+        return fail(BGEMM_EINVAL, "bgemm_packed_forward: operand strides must be non-negative multiples of 4 words");
+    if (batch == 0 || M == 0 || N == 0) return BGEMM_OK;
+    if (!out) return fail(BGEMM_ENULL, "bgemm_packed_forward: out is NULL");
+    if (K == 0) {   // empty sum: every mode gives 0
+        const size_t esz = out_dtype == BGEMM_OUT_F16 ? 2 : 4;
+        for (int64_t b = 0; b < batch; b++) {
+            hipError_t e = hipMemsetAsync((char*)out + (size_t)b * strideC * esz, 0, (size_t)N * M * esz, (hipStream_t)stream);
+            if (e != hipSuccess) return fail(BGEMM_ELAUNCH, "bgemm_packed_forward: memset: %s", hipGetErrorString(e));
+        }
+        return BGEMM_OK;
+    }
+    if (!W_tiled || !X_tiled || (a.mc.planes == 2 && !X2_tiled))
+        return fail(BGEMM_ENULL, "bgemm_packed_forward: operand pointer is NULL");
+    if (((uintptr_t)W_tiled & 15) || ((uintptr_t)X_tiled & 15) || ((uintptr_t)X2_tiled & 15))
+        return fail(BGEMM_EALIGN, "bgemm_packed_forward: operands must be 16-byte aligned");
+    if (batch > 1 && strideC < M * N)
+        return fail(BGEMM_EINVAL, "bgemm_packed_forward: strideC=%lld smaller than N*M", (long long)strideC);
+
+    a.W = (const uint4*)W_tiled; a.X = (const uint4*)X_tiled; a.X2 = (const uint4*)X2_tiled;
+    a.out = out; a.out_f16 = out_dtype == BGEMM_OUT_F16;
+    a.M = M; a.N = N; a.K = K;
+    a.MT = (int)row_tiles(M); a.NT = (int)row_tiles(N); a.KT = (int)k_tiles(K);
+    a.strideW = strideW / 4; a.strideX = strideX / 4; a.strideC = strideC;
+    a.batch = (int)batch; a.splitK = splitK;
+    if (splitK > 1) {
+        const size_t need = bgemm_packed_workspace_bytes(mode, batch, M, N, K, splitK, variant);
+        if (!ws) return fail(BGEMM_EWORKSPACE, "bgemm_packed_forward: splitK=%d needs a workspace of %zu bytes", splitK, need);
+        if (ws_bytes < need) return fail(BGEMM_EWORKSPACE, "bgemm_packed_forward: workspace %zu < %zu bytes", ws_bytes, need);
+        if ((uintptr_t)ws & 15) return fail(BGEMM_EALIGN, "bgemm_packed_forward: workspace must be 16-byte aligned");
+        a.ws_acc = (int32_t*)ws;
+        a.ws_cnt = (uint32_t*)((char*)ws + splitk_acc_bytes(batch, M, N));
+    }
+    int v = variant == BGEMM_VARIANT_AUTO ? pick_variant(a) : variant;
+    if (v == BGEMM_VARIANT_VALU) return launch_gemm_valu(a, (hipStream_t)stream);
+    return launch_gemm_mfma(a, (hipStream_t)stream);
+}
+
+// ---- fp16-operand call: pack both operands into the workspace, then the packed GEMM ----
+// Workspace layout: [split-K state (zero contract)] [W tiled] [X tiled]
+extern "C" size_t bgemm_f16_workspace_zero_bytes(int64_t M, int64_t N, int64_t K, int splitK)
+{
+    return bgemm_packed_workspace_bytes(BGEMM_MODE_XOR, 1, M, N, K, splitK, BGEMM_VARIANT_AUTO);
+}
+
+extern "C" size_t bgemm_f16_workspace_bytes(int64_t M, int64_t N, int64_t K, int splitK)
+{
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    return bgemm_f16_workspace_zero_bytes(M, N, K, splitK) + round256((size_t)bgemm_tiled_words(M, K) * 4) +
+           round256((size_t)bgemm_tiled_words(N, K) * 4);
+}
+
+extern "C" int bgemm_f16_forward(const void* W, const void* X, void* C, int64_t M, int64_t N, int64_t K,
+                                 void* ws, size_t ws_bytes, int splitK, int INSTR, void* stream)
+{
+    g_err[0] = 0;
+    if (INSTR < BGEMM_MODE_AND || INSTR > BGEMM_MODE_ATTN)
+        return fail(BGEMM_EINVAL, "bgemm_f16_forward: INSTR must be 0 (and), 1 (xor) or 2 (attn), got %d", INSTR);
+    if (M < 0 || N < 0 || K < 0 || splitK < 1)
+        return fail(BGEMM_EINVAL, "bgemm_f16_forward: bad shape M=%lld N=%lld K=%lld splitK=%d", (long long)M,
+                    (long long)N, (long long)K, splitK);
+    if (M == 0 || N == 0) return BGEMM_OK;
+    if (!C) return fail(BGEMM_ENULL, "bgemm_f16_forward: C is NULL");
+    if (K == 0)
+        return bgemm_packed_forward(INSTR, nullptr, nullptr, nullptr, C, BGEMM_OUT_F16, 1, M, N, 0, 0, 0, 0, 1,
+                                    BGEMM_VARIANT_AUTO, nullptr, 0, stream);
+    if (!W || !X) return fail(BGEMM_ENULL, "bgemm_f16_forward: operand pointer is NULL");
+    const size_t need = bgemm_f16_workspace_bytes(M, N, K, splitK);
+    if (!ws || ws_bytes < need)
+        return fail(BGEMM_EWORKSPACE, "bgemm_f16_forward: workspace of %zu bytes required, %zu given", need,
+                    ws ? ws_bytes : (size_t)0);
+    if ((uintptr_t)ws & 255) return fail(BGEMM_EALIGN, "bgemm_f16_forward: workspace must be 256-byte aligned");
+    const size_t zb = bgemm_f16_workspace_zero_bytes(M, N, K, splitK);
+    char* wt = (char*)ws + zb;
+    char* xt = wt + round256((size_t)bgemm_tiled_words(M, K) * 4);
+    int rc = bgemm_pack_sign_f16(W, M, K, K, wt, stream);
+    if (rc) return rc;
+    rc = bgemm_pack_sign_f16(X, N, K, K, xt, stream);
+    if (rc) return rc;
+    return bgemm_packed_forward(INSTR, wt, xt, nullptr, C, BGEMM_OUT_F16, 1, M, N, K, 0, 0, 0, splitK,
+                                BGEMM_VARIANT_AUTO, ws, zb, stream);
+}

@@ -1,0 +1,80 @@
+// Shared definitions for the gfx950 BGEMM library (host + device).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "../../include/bgemm_mi355x.h"
+
+namespace bgemm {
+
+// Tiled operand geometry: a tile is 32 rows x 256 K-bits = 64 slots of 16 bytes.
+constexpr int TILE_ROWS = 32;
+constexpr int TILE_KBITS = 256;
+constexpr int TILE_U4 = 64;      // uint4 slots per tile
+constexpr int TILE_WORDS = 256;  // uint32 words per tile
+
+static inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+static inline int64_t row_tiles(int64_t rows) { return cdiv(rows, TILE_ROWS); }
+static inline int64_t k_tiles(int64_t K) { return cdiv(K, TILE_KBITS); }
+
+// Records a message for bgemm_last_error() and returns `code`.
+int fail(int code, const char* fmt, ...);
+// Maps a pending HIP error after a launch to BGEMM_ELAUNCH.
+int check_launch(const char* what);
+
+// Integer epilogue applied to the AND-dot D of a K range holding `bits` valid positions:
+//   C = c0*bits + ca*pa[m] + cb*pb[n] + cd*D (+ cb2*pb2[n] + cd2*D2 for the second plane)
+// pa / pb = popcounts of the weight-side / activation-side rows over the same range.
+struct ModeCoef { int c0, ca, cb, cd, cb2, cd2, planes; };
+
+static inline bool mode_coef(int mode, ModeCoef* mc)
+{
+    switch (mode) {
+    case BGEMM_MODE_AND:    *mc = {0,  0,  0, 1, 0, 0, 1}; return true;
+    case BGEMM_MODE_XOR:    *mc = {1, -2, -2, 4, 0, 0, 1}; return true;   // K - 2 popc(a^b)
+    case BGEMM_MODE_ATTN:   *mc = {1, -1, -2, 2, 0, 0, 1}; return true;   // sum (1-a)(1-2b)
+    case BGEMM_MODE_ATTN_X: *mc = {1, -2, -1, 2, 0, 0, 1}; return true;   // sum (1-b)(1-2a)
+    case BGEMM_MODE_BWTA:   *mc = {0,  0,  1, -2, -2, 4, 2}; return true; // pz - 2pzs - 2D(a,z) + 4D(a,zs)
+    default: return false;
+    }
+}
+
+struct GemmArgs {
+    const uint4* W; const uint4* X; const uint4* X2;
+    void* out; int out_f16;
+    int64_t M, N, K;
+    int MT, NT, KT;
+    int64_t strideW, strideX, strideC;   // uint4 units for W/X, elements for C
+    int batch, splitK;
+    ModeCoef mc;
+    int32_t* ws_acc;      // split-K running sums, [batch][N][M], zero between calls
+    uint32_t* ws_cnt;     // split-K arrival counters, one per output tile, zero between calls
+};
+
+// Contiguous split-K ranges over k-tiles: the first (KT - avg*splitK) splits get one extra.
+__host__ __device__ static inline void split_range(int KT, int splitK, int s, int* k0, int* k1)
+{
+    const int avg = KT / splitK, extra = KT - avg * splitK;
+    const int n = avg + (s < extra ? 1 : 0);
+    const int st = avg * s + (s < extra ? s : extra);
+    *k0 = st; *k1 = st + n;
+}
+
+// Final store of one output element: int32 as is, or fp16 = the integer rounded to nearest
+// even (exact through fp32 because |v| < 2^24).
+__device__ __forceinline__ void store_out(void* out, int out_f16, int64_t idx, int v)
+{
+    if (out_f16) reinterpret_cast<__half*>(out)[idx] = __float2half_rn((float)v);
+    else reinterpret_cast<int*>(out)[idx] = v;
+}
+
+// Kernel families (each in its own translation unit).
+int launch_gemm_mfma(const GemmArgs& a, hipStream_t st);
+int launch_gemm_valu(const GemmArgs& a, hipStream_t st);
+size_t gemm_mfma_ws_bytes(int64_t batch, int64_t M, int64_t N, int64_t K, int splitK, int planes);
+bool gemm_valu_supported(const GemmArgs& a);
+
+}  // namespace bgemm

@@ -1,0 +1,162 @@
+// Design (a): AND + popcount on the vector ALU (v_and_b32 + v_bcnt_u32_b32).
+//
+// A general register-tiled kernel: a 256-thread block owns 64 x 64 outputs, stages one
+// 256-bit K-tile of both operands through LDS in the tiled order (so the 16-byte LDS
+// reads of neighbouring lanes are contiguous) and every thread accumulates a 4 x 4
+// patch.  Like the MFMA kernel it computes the AND-dot and applies the mode's integer
+// epilogue from the row popcounts, which the loading threads collect for free.
+#include "common.h"
+
+namespace bgemm {
+
+__device__ __forceinline__ int popc4v(const uint4 w)
+{
+    return __popc(w.x) + __popc(w.y) + __popc(w.z) + __popc(w.w);
+}
+
+__device__ __forceinline__ int and_popc(const uint4 a, const uint4 b, int acc)
+{
+    acc += __popc(a.x & b.x); acc += __popc(a.y & b.y);
+    acc += __popc(a.z & b.z); acc += __popc(a.w & b.w);
+    return acc;
+}
+
+template <int PL>
+__global__ __launch_bounds__(256) void gemm_valu_kernel(const GemmArgs a, const int tiles_n, const int tiles_m)
+{
+    __shared__ uint4 sX[PL][2][128];     // [plane][buffer][row tile (2) x slot (64)]
+    __shared__ uint4 sW[2][128];
+    __shared__ int sPopX[PL][64], sPopW[64];
+    __shared__ int s_last;
+
+    const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+    const int per_gemm = tiles_n * tiles_m;
+    const unsigned bid = blockIdx.x;
+    const int tile_id = bid % per_gemm, bs = bid / per_gemm;
+    const int split = bs % a.splitK, b = bs / a.splitK;
+    const int tn = tile_id / tiles_m, tm = tile_id % tiles_m;
+    int kt0, kt1;
+    split_range(a.KT, a.splitK, split, &kt0, &kt1);
+
+    // loader role: threads 0..127 fetch the activation tile slots, 128..255 the weight ones
+    const bool loadsX = tid < 128;
+    const int lslot = tid & 127, lrt = lslot >> 6;
+    const uint4* lsrc; const uint4* lsrc2 = nullptr;
+    if (loadsX) {
+        const int64_t rt = min((int64_t)tn * 2 + lrt, (int64_t)a.NT - 1);
+        lsrc = a.X + (int64_t)b * a.strideX + rt * a.KT * TILE_U4 + (lslot & 63);
+        if (PL == 2) lsrc2 = a.X2 + (int64_t)b * a.strideX + rt * a.KT * TILE_U4 + (lslot & 63);
+    } else {
+        const int64_t rt = min((int64_t)tm * 2 + lrt, (int64_t)a.MT - 1);
+        lsrc = a.W + (int64_t)b * a.strideW + rt * a.KT * TILE_U4 + (lslot & 63);
+    }
+    if (tid < 64) { sPopW[tid] = 0; for (int p = 0; p < PL; p++) sPopX[p][tid] = 0; }
+    __syncthreads();
+
+    int acc[PL][4][4];
+#pragma unroll
+    for (int p = 0; p < PL; p++)
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) acc[p][i][j] = 0;
+    int mypop = 0, mypop2 = 0;
+
+    // LDS slot of row `row` (0..63) for K half h: tiled order inside each 32-row tile
+    auto slot_of = [](int row, int h) { return (row >> 5) * 64 + h * 32 + (row & 31); };
+
+    uint4 g0 = make_uint4(0, 0, 0, 0), g1 = g0;
+    if (kt0 < kt1) { g0 = lsrc[(int64_t)kt0 * TILE_U4]; if (PL == 2 && loadsX) g1 = lsrc2[(int64_t)kt0 * TILE_U4]; }
+    for (int kt = kt0; kt < kt1; kt++) {
+        const int buf = (kt - kt0) & 1;
+        if (loadsX) { sX[0][buf][lslot] = g0; if (PL == 2) sX[PL - 1][buf][lslot] = g1; }
+        else sW[buf][lslot] = g0;
+        mypop += popc4v(g0);
+        if (PL == 2) mypop2 += popc4v(g1);
+        if (kt + 1 < kt1) {
+            g0 = lsrc[(int64_t)(kt + 1) * TILE_U4];
+            if (PL == 2 && loadsX) g1 = lsrc2[(int64_t)(kt + 1) * TILE_U4];
+        }
+        __syncthreads();   // one barrier per K-tile: the two LDS buffers alternate
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            uint4 w[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) w[j] = sW[buf][slot_of(tx + 16 * j, h)];
+#pragma unroll
+            for (int p = 0; p < PL; p++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const uint4 x = sX[p][buf][slot_of(ty + 16 * i, h)];
+#pragma unroll
+                    for (int j = 0; j < 4; j++) acc[p][i][j] = and_popc(x, w[j], acc[p][i][j]);
+                }
+        }
+    }
+    // row popcounts: each loader owns (row, half) of one operand
+    {
+        const int row = lrt * 32 + (lslot & 31);
+        if (loadsX) { atomicAdd(&sPopX[0][row], mypop); if (PL == 2) atomicAdd(&sPopX[PL - 1][row], mypop2); }
+        else atomicAdd(&sPopW[row], mypop);
+    }
+    __syncthreads();
+
+    const int64_t kbit0 = (int64_t)kt0 * TILE_KBITS;
+    int64_t kbit1 = (int64_t)kt1 * TILE_KBITS;
+    if (kbit1 > a.K) kbit1 = a.K;
+    const int bits = kbit1 > kbit0 ? (int)(kbit1 - kbit0) : 0;
+    const ModeCoef mc = a.mc;
+    const bool direct = a.splitK == 1;
+    int* accum = direct ? nullptr : a.ws_acc + (int64_t)b * a.N * a.M;
+    const int64_t out_off = (int64_t)b * a.strideC;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int nl = ty + 16 * i;
+        const int64_t n = (int64_t)tn * 64 + nl;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int ml = tx + 16 * j;
+            const int64_t m = (int64_t)tm * 64 + ml;
+            int val = mc.c0 * bits + mc.ca * sPopW[ml] + mc.cb * sPopX[0][nl] + mc.cd * acc[0][i][j];
+            if (PL == 2) val += mc.cb2 * sPopX[PL - 1][nl] + mc.cd2 * acc[PL - 1][i][j];
+            if (n < a.N && m < a.M) {
+                if (direct) store_out(a.out, a.out_f16, out_off + n * a.M + m, val);
+                else atomicAdd(accum + n * a.M + m, val);
+            }
+        }
+    }
+    if (direct) return;
+    __threadfence();
+    __syncthreads();
+    if (tid == 0) {
+        const unsigned t = atomicAdd(a.ws_cnt + (int64_t)b * per_gemm + tile_id, 1u);
+        s_last = (t == (unsigned)a.splitK - 1u);
+    }
+    __syncthreads();
+    if (!s_last) return;
+    __threadfence();
+    for (int e = tid; e < 64 * 64; e += 256) {
+        const int64_t n = (int64_t)tn * 64 + e / 64, m = (int64_t)tm * 64 + e % 64;
+        if (n < a.N && m < a.M) {
+            const int v = atomicExch(accum + n * a.M + m, 0);
+            store_out(a.out, a.out_f16, out_off + n * a.M + m, v);
+        }
+    }
+    if (tid == 0) atomicExch(a.ws_cnt + (int64_t)b * per_gemm + tile_id, 0u);
+}
+
+bool gemm_valu_supported(const GemmArgs&) { return true; }
+
+int launch_gemm_valu(const GemmArgs& a, hipStream_t st)
+{
+    const int tiles_n = (int)cdiv(a.N, 64), tiles_m = (int)cdiv(a.M, 64);
+    const int64_t grid = (int64_t)a.batch * a.splitK * tiles_n * tiles_m;
+    if (grid <= 0 || grid > 0x7fffffffLL) return fail(BGEMM_EINVAL, "gemm_valu: grid of %lld blocks", (long long)grid);
+    if (a.mc.planes == 2)
+        hipLaunchKernelGGL((gemm_valu_kernel<2>), dim3((unsigned)grid), dim3(256), 0, st, a, tiles_n, tiles_m);
+    else
+        hipLaunchKernelGGL((gemm_valu_kernel<1>), dim3((unsigned)grid), dim3(256), 0, st, a, tiles_n, tiles_m);
+    return check_launch("gemm_valu");
+}
+
+}  // namespace bgemm

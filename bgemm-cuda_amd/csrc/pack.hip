@@ -1,0 +1,151 @@
+// fp16 -> bit-plane packing and logical <-> tiled re-layout.  HBM-bound byte work:
+// one 16-byte load per lane, eight sign (and nonzero) bits extracted per lane, four
+// lanes merged into a 32-bit word, 16-byte-contiguous stores into the tiled layout.
+#include "common.h"
+
+namespace bgemm {
+
+// Word offset of logical word jw of `row` inside a tiled operand with KT k-tiles.
+__host__ __device__ static inline int64_t tiled_word_offset(int64_t row, int64_t jw, int64_t KT)
+{
+    const int64_t rt = row >> 5, r = row & 31, kt = jw >> 3, h = (jw >> 2) & 1, q = jw & 3;
+    return ((rt * KT + kt) * TILE_U4 + h * 32 + r) * 4 + q;
+}
+
+// One wave packs 512 consecutive K elements of one row (16 words).
+// mode bit0: also write the (sign & nonzero) plane and make plane 0 the nonzero plane.
+// mode bit1: write the logical layout instead of the tiled one.
+__global__ __launch_bounds__(256) void pack_f16_kernel(
+    const uint16_t* __restrict__ src, int64_t rows, int64_t K, int64_t ld,
+    uint32_t* __restrict__ dst0, uint32_t* __restrict__ dst1, int mode,
+    int64_t rows_out, int64_t nseg, int64_t KT, int64_t Kw)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t gw = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t row = gw / nseg, seg = gw - row * nseg;
+    if (row >= rows_out) return;          // whole wave leaves together
+    const int64_t k0 = seg * 512 + 8 * lane;
+
+    uint16_t h[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) h[e] = 0;
+    if (row < rows && k0 < K) {
+        const uint16_t* p = src + row * ld + k0;
+        if (k0 + 8 <= K && (((uintptr_t)p) & 15) == 0) {
+            const uint4 v = *reinterpret_cast<const uint4*>(p);
+            h[0] = v.x & 0xffff; h[1] = v.x >> 16; h[2] = v.y & 0xffff; h[3] = v.y >> 16;
+            h[4] = v.z & 0xffff; h[5] = v.z >> 16; h[6] = v.w & 0xffff; h[7] = v.w >> 16;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; e++) if (k0 + e < K) h[e] = p[e];
+        }
+    }
+    uint32_t sg = 0, nz = 0;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        sg |= (uint32_t)(h[e] >> 15) << (7 - e);
+        nz |= (uint32_t)((h[e] & 0x7fff) != 0) << (7 - e);
+    }
+    const bool ternary = mode & 1;
+    uint32_t p0 = ternary ? nz : sg, p1 = sg & nz;
+    const int sh = 8 * (3 - (lane & 3));
+    p0 <<= sh; p1 <<= sh;
+    p0 |= __shfl_xor(p0, 1); p0 |= __shfl_xor(p0, 2);
+    if (ternary) { p1 |= __shfl_xor(p1, 1); p1 |= __shfl_xor(p1, 2); }
+    if (lane & 3) return;
+    const int64_t jw = seg * 16 + (lane >> 2);
+    if (mode & 2) {
+        if (row < rows && jw < Kw) { dst0[row * Kw + jw] = p0; if (ternary) dst1[row * Kw + jw] = p1; }
+    } else if (jw < KT * 8) {
+        const int64_t o = tiled_word_offset(row, jw, KT);
+        dst0[o] = p0;
+        if (ternary) dst1[o] = p1;
+    }
+}
+
+// dir 0: logical -> tiled (zero padding), dir 1: tiled -> logical.  One thread per tiled word.
+__global__ __launch_bounds__(256) void relayout_kernel(
+    const uint32_t* __restrict__ src, uint32_t* __restrict__ dst, int64_t rows, int64_t Kw,
+    int64_t KT, int64_t total, int dir)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    // decode tiled word index i -> (row, jw)
+    const int64_t q = i & 3, slot = (i >> 2) & 63, tile = i >> 8;
+    const int64_t kt = tile % KT, rt = tile / KT;
+    const int64_t row = rt * 32 + (slot & 31), jw = kt * 8 + (slot >> 5) * 4 + q;
+    const bool real = row < rows && jw < Kw;
+    if (dir == 0) dst[i] = real ? src[row * Kw + jw] : 0u;
+    else if (real) dst[row * Kw + jw] = src[i];
+}
+
+static int pack_common(const void* src, int64_t rows, int64_t K, int64_t ld, void* d0, void* d1,
+                       int mode, hipStream_t st, const char* who)
+{
+    if (rows < 0 || K < 0 || ld < K) return fail(BGEMM_EINVAL, "%s: bad shape rows=%lld K=%lld ld=%lld", who,
+                                                 (long long)rows, (long long)K, (long long)ld);
+    if (rows == 0 || K == 0) return BGEMM_OK;
+    if (!src || !d0 || ((mode & 1) && !d1)) return fail(BGEMM_ENULL, "%s: null pointer", who);
+    if (((uintptr_t)d0 & 15) || ((uintptr_t)d1 & 15)) return fail(BGEMM_EALIGN, "%s: destination not 16-byte aligned", who);
+    const int64_t KT = k_tiles(K), Kw = cdiv(K, 32);
+    const int64_t rows_out = (mode & 2) ? rows : row_tiles(rows) * TILE_ROWS;
+    const int64_t nseg = cdiv(KT * TILE_KBITS, 512);
+    const int64_t waves = rows_out * nseg, blocks = cdiv(waves, 4);
+    if (blocks > 0x7fffffffLL) return fail(BGEMM_EINVAL, "%s: operand too large", who);
+    hipLaunchKernelGGL(pack_f16_kernel, dim3((unsigned)blocks), dim3(256), 0, st,
+                       (const uint16_t*)src, rows, K, ld, (uint32_t*)d0, (uint32_t*)d1, mode,
+                       rows_out, nseg, KT, Kw);
+    return check_launch(who);
+}
+
+}  // namespace bgemm
+
+using namespace bgemm;
+
+extern "C" int64_t bgemm_tiled_words(int64_t rows, int64_t K)
+{
+    if (rows <= 0 || K <= 0) return 0;
+    return row_tiles(rows) * k_tiles(K) * TILE_WORDS;
+}
+
+extern "C" int bgemm_pack_sign_f16(const void* src, int64_t rows, int64_t K, int64_t ld,
+                                   void* dst_tiled, void* stream)
+{
+    return pack_common(src, rows, K, ld, dst_tiled, nullptr, 0, (hipStream_t)stream, "bgemm_pack_sign_f16");
+}
+
+extern "C" int bgemm_pack_sign_f16_logical(const void* src, int64_t rows, int64_t K, int64_t ld,
+                                           uint32_t* dst_logical, void* stream)
+{
+    return pack_common(src, rows, K, ld, dst_logical, nullptr, 2, (hipStream_t)stream, "bgemm_pack_sign_f16_logical");
+}
+
+extern "C" int bgemm_pack_ternary_f16(const void* src, int64_t rows, int64_t K, int64_t ld,
+                                      void* nz_tiled, void* sg_tiled, void* stream)
+{
+    return pack_common(src, rows, K, ld, nz_tiled, sg_tiled, 1, (hipStream_t)stream, "bgemm_pack_ternary_f16");
+}
+
+static int relayout(const void* src, void* dst, int64_t rows, int64_t K, int dir, void* stream, const char* who)
+{
+    if (rows < 0 || K < 0) return fail(BGEMM_EINVAL, "%s: bad shape", who);
+    if (rows == 0 || K == 0) return BGEMM_OK;
+    if (!src || !dst) return fail(BGEMM_ENULL, "%s: null pointer", who);
+    const int64_t total = bgemm_tiled_words(rows, K), blocks = cdiv(total, 256);
+    if (blocks > 0x7fffffffLL) return fail(BGEMM_EINVAL, "%s: operand too large", who);
+    hipLaunchKernelGGL(relayout_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       (const uint32_t*)src, (uint32_t*)dst, rows, cdiv(K, 32), k_tiles(K), total, dir);
+    return check_launch(who);
+}
+
+extern "C" int bgemm_tile_from_logical(const uint32_t* logical, int64_t rows, int64_t K,
+                                       void* dst_tiled, void* stream)
+{
+    return relayout(logical, dst_tiled, rows, K, 0, stream, "bgemm_tile_from_logical");
+}
+
+extern "C" int bgemm_logical_from_tiled(const void* tiled, int64_t rows, int64_t K,
+                                        uint32_t* dst_logical, void* stream)
+{
+    return relayout(tiled, dst_logical, rows, K, 1, stream, "bgemm_logical_from_tiled");
+}

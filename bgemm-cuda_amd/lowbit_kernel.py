@@ -1,0 +1,210 @@
+"""Drop-in for the reference's ``lowbit_kernel`` extension module (BGEMM part).
+
+``bgemm_linear_forward_cuda(in_feats, weights, splitK=1, INSTR=1)`` has the reference's
+name, argument order, defaults and return value (lowbit_kernel/csrc/pybind.cpp:12,
+fp6_linear.cu:561-616): fp16 ``[N,K]`` x fp16 ``[M,K]`` -> fp16 ``[N,M]``.  Everything
+else here is the packed-operand surface the reference only stubbed
+(binary_weight_prepacking_cuda, fp6_linear.cu:519-542).
+
+All work is enqueued on the current torch stream through the C ABI in
+include/bgemm_mi355x.h; torch supplies device memory and streams only.
+"""
+import torch
+
+import _lib as _b
+from _lib import (MODE_AND, MODE_XOR, MODE_ATTN, MODE_BWTA, MODE_ATTN_X, OUT_I32, OUT_F16,
+                  VARIANT_AUTO, VARIANT_VALU, VARIANT_MFMA)
+
+AND_POP, XOR_POP, ATTN_MM = 0, 1, 2   # lowbit_kernel/csrc/include/configs.h:70-72
+
+__all__ = ["bgemm_linear_forward_cuda", "binary_weight_prepacking", "pack_sign", "pack_ternary",
+           "bgemm_packed_forward", "PackedBits", "AND_POP", "XOR_POP", "ATTN_MM"]
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _need_cuda(t, name):
+    if not isinstance(t, torch.Tensor):
+        raise TypeError("%s must be a torch.Tensor" % name)
+    if not t.is_cuda:
+        raise ValueError("%s must live on the GPU" % name)
+
+
+# Split-K state must be zero before first use and is left zero by every call, so one
+# zero-filled buffer per (device, stream) is grown on demand and reused.
+_zero_ws = {}
+
+
+def _zeroed_workspace(nbytes, device):
+    key = (device.index, _stream())
+    buf = _zero_ws.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _zero_ws[key] = buf
+    return buf
+
+
+class PackedBits:
+    """A bit-packed operand in the tiled layout (32 rows x 256 K-bits per 1 KiB tile).
+
+    ``data`` is an int32 tensor ``[batch, words]``; ``data2`` is the second plane of a ternary
+    operand (sign & nonzero) or None.
+    """
+
+    def __init__(self, data, data2, batch, rows, K):
+        self.data, self.data2, self.batch, self.rows, self.K = data, data2, batch, rows, K
+
+    @property
+    def ternary(self):
+        return self.data2 is not None
+
+    @property
+    def words(self):
+        return self.data.shape[1]
+
+    def nbytes(self):
+        return self.data.numel() * 4 * (2 if self.ternary else 1)
+
+
+def _pack(x, ternary):
+    _need_cuda(x, "input")
+    if x.dim() not in (2, 3):
+        raise ValueError("expected a 2-D or 3-D tensor, got %d-D" % x.dim())
+    x = x.to(torch.half).contiguous()
+    batch = 1 if x.dim() == 2 else x.shape[0]
+    rows, K = x.shape[-2], x.shape[-1]
+    L = _b.lib()
+    words = L.bgemm_tiled_words(rows, K)
+    d0 = torch.empty((batch, words), dtype=torch.int32, device=x.device)
+    d1 = torch.empty_like(d0) if ternary else None
+    with torch.cuda.device(x.device):
+        st = _stream()
+        if batch > 1 and rows % 32 == 0:
+            # whole tiles per matrix: the batch is one tall matrix in the tiled layout
+            groups = [(x.data_ptr(), batch * rows, d0.data_ptr(), d1.data_ptr() if ternary else None)]
+        else:
+            groups = [(x[i].data_ptr() if x.dim() == 3 else x.data_ptr(), rows, d0[i].data_ptr(),
+                       d1[i].data_ptr() if ternary else None) for i in range(batch)]
+        for src, r, p0, p1 in groups:
+            if ternary:
+                _b.check(L.bgemm_pack_ternary_f16(src, r, K, K, p0, p1, st))
+            else:
+                _b.check(L.bgemm_pack_sign_f16(src, r, K, K, p0, st))
+    return PackedBits(d0, d1, batch, rows, K)
+
+
+def pack_sign(x):
+    """fp16 (or castable) ``[R,K]`` / ``[B,R,K]`` -> tiled sign bits (bit = 1 for negative, -0.0 included)."""
+    return _pack(x, False)
+
+
+def pack_ternary(x):
+    """``[R,K]`` / ``[B,R,K]`` -> tiled (nonzero, sign&nonzero) planes of sign(x) in {-1,0,+1}."""
+    return _pack(x, True)
+
+
+def binary_weight_prepacking(weights):
+    """half ``[OC,IC]`` -> int32 ``[OC, ceil(IC/32)]`` in the reference's logical format
+    (bit 31-i of word j = sign bit of element 32j+i; weight_prepacking.h:181-230).  This is what
+    binary_weight_prepacking_cuda (fp6_linear.cu:519-542) declares but leaves uninitialised."""
+    _need_cuda(weights, "weights")
+    if weights.dim() != 2:
+        raise ValueError("weights must be 2-D")
+    w = weights.to(torch.half).contiguous()
+    OC, IC = w.shape
+    out = torch.empty((OC, (IC + 31) // 32), dtype=torch.int32, device=w.device)
+    with torch.cuda.device(w.device):
+        _b.check(_b.lib().bgemm_pack_sign_f16_logical(w.data_ptr(), OC, IC, IC, out.data_ptr(), _stream()))
+    return out
+
+
+def tile_from_logical(logical, K):
+    """int32 ``[R, ceil(K/32)]`` logical words -> PackedBits in the tiled layout."""
+    _need_cuda(logical, "logical")
+    logical = logical.contiguous()
+    R = logical.shape[0]
+    L = _b.lib()
+    d0 = torch.empty((1, L.bgemm_tiled_words(R, K)), dtype=torch.int32, device=logical.device)
+    with torch.cuda.device(logical.device):
+        _b.check(L.bgemm_tile_from_logical(logical.data_ptr(), R, K, d0.data_ptr(), _stream()))
+    return PackedBits(d0, None, 1, R, K)
+
+
+def logical_from_tiled(packed, plane=0):
+    """PackedBits (batch 1) -> int32 ``[R, ceil(K/32)]`` in the logical format."""
+    src = packed.data if plane == 0 else packed.data2
+    out = torch.empty((packed.rows, (packed.K + 31) // 32), dtype=torch.int32, device=src.device)
+    with torch.cuda.device(src.device):
+        _b.check(_b.lib().bgemm_logical_from_tiled(src.data_ptr(), packed.rows, packed.K, out.data_ptr(), _stream()))
+    return out
+
+
+def bgemm_packed_forward(w, x, mode=MODE_XOR, out_dtype=torch.int32, splitK=1, variant=VARIANT_AUTO, out=None):
+    """GEMM on packed operands: ``out[b,n,m]`` for weight-side ``w`` (M rows) and activation-side
+    ``x`` (N rows).  A batch of 1 on either side is shared across the other side's batch."""
+    if w.K != x.K:
+        raise ValueError("K mismatch: %d vs %d" % (w.K, x.K))
+    if (mode == MODE_BWTA) != x.ternary:
+        raise ValueError("MODE_BWTA needs a ternary activation operand, the other modes a binary one")
+    if w.ternary:
+        raise ValueError("the weight side is binary")
+    batch = max(w.batch, x.batch)
+    if w.batch not in (1, batch) or x.batch not in (1, batch):
+        raise ValueError("batch mismatch: %d vs %d" % (w.batch, x.batch))
+    if out_dtype not in (torch.int32, torch.half):
+        raise ValueError("out_dtype must be torch.int32 or torch.half")
+    M, N, K = w.rows, x.rows, w.K
+    dev = w.data.device
+    if out is None:
+        out = torch.empty((batch, N, M), dtype=out_dtype, device=dev)
+    L = _b.lib()
+    with torch.cuda.device(dev):
+        nws = L.bgemm_packed_workspace_bytes(mode, batch, M, N, K, splitK, variant)
+        ws = _zeroed_workspace(nws, dev) if nws else None
+        _b.check(L.bgemm_packed_forward(
+            mode, w.data.data_ptr(), x.data.data_ptr(), x.data2.data_ptr() if x.ternary else None,
+            out.data_ptr(), OUT_F16 if out_dtype == torch.half else OUT_I32, batch, M, N, K,
+            w.words if w.batch > 1 else 0, x.words if x.batch > 1 else 0, N * M,
+            splitK, variant, ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0,
+            _stream()))
+    return out
+
+
+def bgemm_linear_forward_cuda(in_feats, weights, splitK=1, INSTR=1):
+    """Computes BGEMM: half ``in_feats [N,K]``, half ``weights [M,K]`` -> half ``[N,M]``.
+
+    INSTR 0 = and.popc, 1 = K - 2*xor.popc, 2 = attention ({0,1} weights side by sign bit clear).
+    Unlike the reference (fp6_linear.cu:288-290, 568-576) any N, M, K >= 1 is accepted, inputs need
+    not be contiguous, and the launch goes to the current stream."""
+    _need_cuda(in_feats, "in_feats")
+    _need_cuda(weights, "weights")
+    if in_feats.dim() != 2 or weights.dim() != 2:
+        raise ValueError("in_feats and weights must be 2-D")
+    if in_feats.dtype != torch.half or weights.dtype != torch.half:
+        raise TypeError("in_feats and weights must be torch.half")   # data_ptr<at::Half> in the reference
+    if in_feats.shape[1] != weights.shape[1]:
+        raise ValueError("K mismatch: in_feats %s vs weights %s" % (tuple(in_feats.shape), tuple(weights.shape)))
+    x, w = in_feats.contiguous(), weights.contiguous()
+    N, K = x.shape
+    M = w.shape[0]
+    out = torch.empty((N, M), dtype=torch.half, device=x.device)
+    L = _b.lib()
+    with torch.cuda.device(x.device):
+        total = L.bgemm_f16_workspace_bytes(M, N, K, splitK)
+        zb = L.bgemm_f16_workspace_zero_bytes(M, N, K, splitK)
+        # [split-K state | packed W | packed X]: only the first zb bytes must start at zero
+        ws = torch.empty(max(total, 1), dtype=torch.uint8, device=x.device)
+        if zb:
+            ws[:zb].zero_()
+        _b.check(L.bgemm_f16_forward(w.data_ptr(), x.data_ptr(), out.data_ptr(), M, N, K,
+                                     ws.data_ptr(), ws.numel(), int(splitK), int(INSTR), _stream()))
+    return out
+
+
+def _fp6_only(*_a, **_k):
+    raise NotImplementedError("FP6 entry points of the reference extension are outside this library")
+
+
+linear_forward_cuda = weight_prepacking_cpu = weight_dequant_cpu = _fp6_only

@@ -1,0 +1,123 @@
+/*
+ * bgemm_mi355x.h -- C ABI of the MI355X (gfx950) binary-GEMM library.
+ *
+ * Plain C, plain pointers and sizes: no torch, no C++ types.  Every entry point is
+ * asynchronous on the HIP stream it is given (NULL = the null stream), never
+ * allocates or frees device memory, keeps no global state apart from a
+ * thread-local error string, and returns 0 or a negative BGEMM_E* code.
+ * All device pointers are borrowed for the duration of the enqueued work.
+ *
+ * Citations name the reference interface each entry point stands in for
+ * (paths relative to the reference tree).
+ *
+ * Operand semantics (reference: lowbit_kernel/csrc/include/utils_core.cuh:242-303,
+ * ptx_mma.cuh:196-250,299-336).  With a = sign bit of the weight-side element,
+ * b = sign bit of the activation-side element (1 = negative, -0.0 included):
+ *   BGEMM_MODE_AND   C[n,m] = #{k : a=1 and b=1}
+ *   BGEMM_MODE_XOR   C[n,m] = K - 2*#{k : a != b}            ({-1,1} x {-1,1})
+ *   BGEMM_MODE_ATTN  C[n,m] = sum_k (1-a)(1-2b)              ({0,1} weight side x {-1,1})
+ *   BGEMM_MODE_BWTA  C[n,m] = sum_k t(1-2a), t in {-1,0,1} given as two planes
+ *                    (nonzero, sign&nonzero) on the activation side
+ *   BGEMM_MODE_ATTN_X  as ATTN with the roles swapped: {0,1} on the activation side
+ * The output is row-major [N][M] (kernel_matmul.cuh:534-545), int32 or fp16 where
+ * fp16 = the exact integer rounded to nearest even (kernel_matmul.cuh:540).
+ */
+#ifndef BGEMM_MI355X_H
+#define BGEMM_MI355X_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* INSTR values 0..2 are the reference's API (configs.h:70-72); 3 and 4 are supersets. */
+enum { BGEMM_MODE_AND = 0, BGEMM_MODE_XOR = 1, BGEMM_MODE_ATTN = 2, BGEMM_MODE_BWTA = 3,
+       BGEMM_MODE_ATTN_X = 4 };
+enum { BGEMM_OUT_I32 = 0, BGEMM_OUT_F16 = 1 };
+/* Kernel family: AUTO picks per shape; VALU = xor/and + popcount on the vector ALU;
+ * MFMA = bit planes expanded to int8 in registers feeding v_mfma_i32_32x32x32_i8. */
+enum { BGEMM_VARIANT_AUTO = 0, BGEMM_VARIANT_VALU = 1, BGEMM_VARIANT_MFMA = 2 };
+
+enum {
+    BGEMM_OK = 0,
+    BGEMM_EINVAL = -1,      /* bad shape, mode, dtype, variant or splitK            */
+    BGEMM_ENULL = -2,       /* a required pointer is NULL                            */
+    BGEMM_EWORKSPACE = -3,  /* workspace missing or smaller than *_workspace_bytes() */
+    BGEMM_ELAUNCH = -4,     /* HIP reported an error at launch                       */
+    BGEMM_EALIGN = -5       /* a pointer is not 16-byte aligned                      */
+};
+
+/* Message for the last error returned on the calling thread ("" if none). */
+const char* bgemm_last_error(void);
+/* ABI version; bumped when a signature or the tiled layout changes. */
+int bgemm_abi_version(void);
+
+/* ---- packed operand layout -------------------------------------------------------
+ * "Logical" format = the reference's (weight_prepacking.h:181-230): uint32 [rows][ceil(K/32)],
+ * bit (31-i) of word j = sign bit of element 32*j+i, unused tail bits 0.
+ * "Tiled" format = what the kernels stream: tiles of 32 rows x 256 K-bits, 1 KiB each,
+ * tile (rt, kt) at word offset (rt*KT + kt)*256, inside a tile 64 slots of 16 bytes,
+ * slot h*32 + r = logical words 8*kt + 4*h .. +3 of row 32*rt + r.  Rows and K are
+ * zero-padded to whole tiles (zero bits contribute nothing in any mode).
+ */
+/* Number of uint32 words of a tiled operand of `rows` x K bits. */
+int64_t bgemm_tiled_words(int64_t rows, int64_t K);
+
+/* fp16 [rows][K] (row stride ld elements) -> tiled sign bits.
+ * Replaces the in-kernel sign packing (ptx_mma.cuh:341-380) and the host routine
+ * bin_matrix_prepacking_to_uint32 (weight_prepacking.h:203-230); this is the weight
+ * prepack entry point that binary_weight_prepacking_cuda (fp6_linear.cu:519-542) stubs. */
+int bgemm_pack_sign_f16(const void* src, int64_t rows, int64_t K, int64_t ld,
+                        void* dst_tiled, void* stream);
+/* fp16 -> logical format exactly as weight_prepacking.h:181-230 defines it. */
+int bgemm_pack_sign_f16_logical(const void* src, int64_t rows, int64_t K, int64_t ld,
+                                uint32_t* dst_logical, void* stream);
+/* fp16 -> two tiled planes: nonzero, and sign&nonzero (ternary = torch.sign,
+ * tests/python/bgemm_linear.py:222-241). */
+int bgemm_pack_ternary_f16(const void* src, int64_t rows, int64_t K, int64_t ld,
+                           void* nz_tiled, void* sg_tiled, void* stream);
+/* logical <-> tiled re-layout of already packed bits (device buffers). */
+int bgemm_tile_from_logical(const uint32_t* logical, int64_t rows, int64_t K,
+                            void* dst_tiled, void* stream);
+int bgemm_logical_from_tiled(const void* tiled, int64_t rows, int64_t K,
+                             uint32_t* dst_logical, void* stream);
+
+/* ---- GEMM on packed operands -------------------------------------------------------
+ * Replaces bin_pack_linear_kernel + SplitK_Reduction (fp6_linear.cu:275-337,
+ * kernel_reduction.cuh:29-48) for operands that are already bit-packed.
+ *   W_tiled  : weight side, M rows.   X_tiled : activation side, N rows.
+ *   X2_tiled : BWTA only, the sign&nonzero plane (X_tiled is the nonzero plane).
+ *   batch    : number of independent GEMMs; strides in uint32 words / output elements
+ *              (a stride of 0 shares that operand across the batch).
+ *   splitK   : >= 1; K-tiles are divided into splitK contiguous ranges as in
+ *              kernel_matmul.cuh:397-404, reduced inside the kernel with integer adds,
+ *              so the result does not depend on it.
+ *   ws       : needed iff bgemm_packed_workspace_bytes() > 0.  Must be zero-filled
+ *              once before first use; every call leaves it zero-filled again.
+ */
+size_t bgemm_packed_workspace_bytes(int mode, int64_t batch, int64_t M, int64_t N, int64_t K,
+                                    int splitK, int variant);
+int bgemm_packed_forward(int mode, const void* W_tiled, const void* X_tiled, const void* X2_tiled,
+                         void* out, int out_dtype, int64_t batch, int64_t M, int64_t N, int64_t K,
+                         int64_t strideW, int64_t strideX, int64_t strideC,
+                         int splitK, int variant, void* ws, size_t ws_bytes, void* stream);
+
+/* ---- fp16-operand call, the drop-in for the reference launcher -----------------------
+ * Same argument meaning as bin_pack_linear_kernel (fp6_linear.cu:275-286):
+ * W = weights half [M][K], X = in_feats half [N][K], C = half [N][M], INSTR in {0,1,2}.
+ * Differences: any M, N, K >= 1 (the reference asserts M%32, N%32, K%128); the
+ * workspace is bytes of scratch (packed operands + split-K state) instead of fp32
+ * partial planes, and has the same zero-fill contract as above for its first
+ * bgemm_f16_workspace_zero_bytes() bytes.
+ */
+size_t bgemm_f16_workspace_bytes(int64_t M, int64_t N, int64_t K, int splitK);
+size_t bgemm_f16_workspace_zero_bytes(int64_t M, int64_t N, int64_t K, int splitK);
+int bgemm_f16_forward(const void* W, const void* X, void* C, int64_t M, int64_t N, int64_t K,
+                      void* ws, size_t ws_bytes, int splitK, int INSTR, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BGEMM_MI355X_H */

@@ -1,0 +1,125 @@
+"""The C-ABI library loads without a GPU, exports every symbol the header declares, and
+rejects bad arguments from the host side (no kernel is launched by any call here)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+import _lib
+
+HEADER = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include", "bgemm_mi355x.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(bgemm_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_exported():
+    names = declared_functions()
+    assert len(names) >= 12
+    L = ctypes.CDLL(_lib.SO_PATH)
+    for n in names:
+        assert hasattr(L, n), "missing export: %s" % n
+    # the binding table and the header list the same entry points
+    assert sorted(_lib.SIGNATURES) == names
+
+
+def test_layout_sizes():
+    L = _lib.lib()
+    assert L.bgemm_abi_version() == 1
+    assert L.bgemm_tiled_words(1, 1) == 256
+    assert L.bgemm_tiled_words(32, 256) == 256
+    assert L.bgemm_tiled_words(33, 257) == 4 * 256
+    assert L.bgemm_tiled_words(11008, 4096) == 11008 * 4096 // 32
+    assert L.bgemm_tiled_words(0, 128) == 0
+    assert L.bgemm_packed_workspace_bytes(1, 1, 64, 64, 1024, 1, 0) == 0
+    assert L.bgemm_packed_workspace_bytes(1, 1, 64, 64, 1024, 4, 0) >= 64 * 64 * 4 + 4
+    assert L.bgemm_f16_workspace_bytes(64, 32, 256, 1) >= (64 + 32) * 256 // 8
+
+
+@pytest.mark.parametrize("kwargs, code", [
+    (dict(mode=7), _lib.EINVAL),
+    (dict(out_dtype=5), _lib.EINVAL),
+    (dict(variant=9), _lib.EINVAL),
+    (dict(M=-1), _lib.EINVAL),
+    (dict(splitK=0), _lib.EINVAL),
+    (dict(K=1 << 24), _lib.EINVAL),
+    (dict(out=None), _lib.ENULL),
+    (dict(W=None), _lib.ENULL),
+    (dict(mode=3), _lib.ENULL),                       # BWTA without the second plane
+    (dict(W=0x1008), _lib.EALIGN),
+    (dict(splitK=2), _lib.EWORKSPACE),                # no workspace given
+    (dict(splitK=2, ws=0x10000, ws_bytes=16), _lib.EWORKSPACE),
+    (dict(strideW=2), _lib.EINVAL),
+])
+def test_packed_forward_rejects(kwargs, code):
+    L = _lib.lib()
+    a = dict(mode=1, W=0x1000, X=0x2000, X2=None, out=0x3000, out_dtype=0, batch=1, M=64, N=64, K=256,
+             strideW=0, strideX=0, strideC=0, splitK=1, variant=0, ws=None, ws_bytes=0, stream=None)
+    a.update(kwargs)
+    rc = L.bgemm_packed_forward(a["mode"], a["W"], a["X"], a["X2"], a["out"], a["out_dtype"], a["batch"], a["M"],
+                                a["N"], a["K"], a["strideW"], a["strideX"], a["strideC"], a["splitK"], a["variant"],
+                                a["ws"], a["ws_bytes"], a["stream"])
+    assert rc == code
+    assert L.bgemm_last_error()            # a message was recorded
+    with pytest.raises(ValueError):
+        _lib.check(rc)
+
+
+def test_empty_problems_are_ok_without_launch():
+    L = _lib.lib()
+    assert L.bgemm_packed_forward(1, None, None, None, None, 0, 0, 64, 64, 256, 0, 0, 0, 1, 0, None, 0, None) == 0
+    assert L.bgemm_packed_forward(1, None, None, None, None, 0, 1, 0, 64, 256, 0, 0, 0, 1, 0, None, 0, None) == 0
+    assert L.bgemm_pack_sign_f16(None, 0, 128, 128, None, None) == 0
+    assert L.bgemm_f16_forward(None, None, None, 0, 5, 128, None, 0, 1, 1, None) == 0
+
+
+def test_pack_and_f16_reject():
+    L = _lib.lib()
+    assert L.bgemm_pack_sign_f16(0x1000, 4, 128, 64, 0x2000, None) == _lib.EINVAL      # ld < K
+    assert L.bgemm_pack_sign_f16(None, 4, 128, 128, 0x2000, None) == _lib.ENULL
+    assert L.bgemm_pack_sign_f16(0x1000, 4, 128, 128, 0x2004, None) == _lib.EALIGN
+    assert L.bgemm_pack_ternary_f16(0x1000, 4, 128, 128, 0x2000, None, None) == _lib.ENULL
+    assert L.bgemm_f16_forward(0x1000, 0x2000, 0x3000, 32, 32, 128, None, 0, 1, 3, None) == _lib.EINVAL  # INSTR 3
+    assert L.bgemm_f16_forward(0x1000, 0x2000, 0x3000, 32, 32, 128, None, 0, 1, 1, None) == _lib.EWORKSPACE
+    assert L.bgemm_f16_forward(0x1000, 0x2000, None, 32, 32, 128, 0x4000, 1 << 20, 1, 1, None) == _lib.ENULL
+
+
+def test_missing_library_is_loud(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "SO_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(ImportError):
+        _lib.lib()
+
+
+def test_shim_rejects_cpu_tensors():
+    import torch
+    import lowbit_kernel
+    x = torch.zeros(32, 128, dtype=torch.half)
+    with pytest.raises(ValueError):
+        lowbit_kernel.bgemm_linear_forward_cuda(x, x)
+    with pytest.raises(NotImplementedError):
+        lowbit_kernel.linear_forward_cuda()
+
+
+def test_cpu_layers_match_reference_cpu_path(oracle):
+    """BNNLinear / NNLinear_elastic_signed are plain torch and run anywhere."""
+    import torch
+    import bgemm_linear
+    torch.manual_seed(0)
+    x = torch.randn(32, 128)
+    lin = bgemm_linear.BNNLinear(128, 64, False)
+    y = lin(x)
+    sw, sa, zpw, zpa = oracle.cpu_path_layer_scales(x, lin.weight)
+    want = oracle.cpu_path_bnn_linear(x, lin.weight, None, sw, sa, zpw, zpa)
+    assert torch.equal(y, want)
+    el = bgemm_linear.NNLinear_elastic_signed(128, 64, True)
+    y2 = el(x)
+    xs = ((x - x.mean().item()) / el.sa).half().sign()
+    ws = (el.weight - el.weight.mean().item()).half().sign()
+    assert torch.equal(y2, oracle.cpu_path_linear(xs, ws) * el.sa * el.sw + el.bias)
+    y2.sum().backward()
+    assert el.weight.grad is not None and el.sa.grad is not None

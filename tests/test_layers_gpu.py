@@ -1,0 +1,100 @@
+"""The layer mirror on the GPU: same numbers as the reference CPU path (torch matmul on +-1
+tensors) fed identical operands, compared bit for bit (tolerance 0)."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+import bgemm_linear as bl
+import lowbit_kernel as lk
+
+DEV = "cuda:0"
+
+
+def test_bgemm_linear_function_vs_sign_matmul():
+    torch.manual_seed(0)
+    x, w = torch.randn(64, 768, device=DEV), torch.randn(96, 768, device=DEV)
+    out = bl.bgemm_linear.apply(x, w)
+    want = (x.half().sign().float() @ w.half().sign().float().T)
+    assert out.dtype == torch.half and torch.equal(out.float(), want.half().float())
+    out_and = bl.bgemm_linear.apply(x, w, 'and')
+    assert torch.equal(out_and.float(), ((x < 0).float() @ (w < 0).float().T).half().float())
+
+
+def test_bgemm_matmul_and_attn_matmul():
+    torch.manual_seed(1)
+    q, k = torch.randn(32, 768, device=DEV), torch.randn(32, 768, device=DEV)
+    attn = bl.bgemm_matmul.apply(q, k.transpose(-1, -2))
+    assert torch.equal(attn.float(), torch.matmul(q.sign(), k.sign().T).half().float())
+    # a genuinely contiguous [K, M] right operand also works (the reference mis-reads it)
+    kt = k.T.contiguous()
+    assert torch.equal(bl.bgemm_matmul.apply(q, kt), attn)
+    a = torch.randn(128, 256, device=DEV)
+    v = torch.randn(256, 64, device=DEV)
+    out = bl.bgemm_attn_matmul.apply(a, v)
+    want = (a >= 0).float() @ v.sign()
+    assert tuple(out.shape) == (128, 64) and torch.equal(out.float(), want.half().float())
+
+
+def test_bgemm_linear_backward_shapes_and_values():
+    torch.manual_seed(2)
+    x = torch.randn(32, 128, device=DEV, requires_grad=True)
+    w = torch.randn(16, 128, device=DEV, requires_grad=True)
+    bl.bgemm_linear_bireal.apply(x, w).float().sum().backward()
+    g = torch.ones(32, 16, device=DEV)
+    assert torch.allclose(w.grad, (g.T @ x.detach().half().sign().float()), atol=0)
+    dx = 2 - 2 * x.detach().half().float().abs().clamp(max=1)
+    assert torch.allclose(x.grad, (g @ w.detach().half().sign().float()) * dx, atol=1e-3)
+
+
+@pytest.mark.parametrize("cls", [bl.BGEMMLinear, bl.BGEMMLinear_bireal])
+def test_bgemm_linear_module_vs_bnn(oracle, cls):
+    torch.manual_seed(3)
+    x = torch.randn(128, 784, device=DEV)
+    lin = cls(784, 4096, bias=True).to(DEV)
+    y = lin(x)
+    sw, sa, zpw, zpa = oracle.cpu_path_layer_scales(x, lin.weight)
+    # reference CPU path on the de-binarised operands; fp16 accumulator semantics of the kernel output
+    acc = oracle.cpu_path_linear(oracle.cpu_path_bin_active((x - zpa).half().float()).cpu(),
+                                 oracle.cpu_path_bin_active((lin.weight - zpw).half().float()).cpu()).to(DEV)
+    want = acc.half() * sw * sa + lin.bias.view(1, -1)
+    assert torch.equal(y, want)
+    # ragged batch (the reference asserts batch % 32 == 0)
+    assert torch.equal(lin(x[:5]), want[:5])
+
+
+def test_elastic_module_matches_cpu_twin():
+    torch.manual_seed(4)
+    x = torch.randn(64, 256, device=DEV)
+    a = bl.BGEMMLinear_elastic_signed(256, 128).to(DEV)
+    b = bl.NNLinear_elastic_signed(256, 128).to(DEV)
+    b.load_state_dict(a.state_dict())
+    ya, yb = a(x), b(x)
+    # the twin ternarises exact zeros to 0 while the kernel reads the sign bit; none occur here
+    assert torch.equal(ya.float(), yb.float())
+    ya.float().sum().backward()
+    assert a.weight.grad is not None and a.sa.grad is not None and a.sw.grad is not None
+
+
+def test_config2_mlp_forward_bitwise(oracle):
+    """BASELINE config 2: 784 -> 4096 -> 4096 -> 10, batch 128, fp16 outputs vs the CPU chain."""
+    g = torch.Generator().manual_seed(1002)
+    dims = [784, 4096, 4096, 10]
+    x = torch.randn(128, 784, generator=g).half()
+    Ws = [torch.randn(dims[i + 1], dims[i], generator=g).half() for i in range(3)]
+    h_gpu, h_cpu = x.to(DEV), x.clone()
+    for W in Ws:
+        sw = (W.float().norm(1, 1) / W.numel()).half()
+        sa = (2 * h_cpu.float().abs().mean()).half()
+        # GPU: binary kernel then fp16 scaling, left to right as the reference layer does
+        acc_gpu = lk.bgemm_linear_forward_cuda(h_gpu, W.to(DEV), 1, 1)
+        h_gpu = acc_gpu * sw.to(DEV) * sa.to(DEV)
+        # CPU reference path: torch matmul on +-1 tensors (sign-bit rule), fp16 rounding of the exact sum
+        sx = torch.where(torch.signbit(h_cpu), -1.0, 1.0)
+        swt = torch.where(torch.signbit(W), -1.0, 1.0)
+        acc_cpu = oracle.cpu_path_linear(sx, swt).half()
+        h_cpu = acc_cpu * sw * sa
+        assert torch.equal(acc_gpu.cpu(), acc_cpu)
+        assert torch.equal(h_gpu.cpu(), h_cpu)
+    assert tuple(h_gpu.shape) == (128, 10)

@@ -1,0 +1,303 @@
+"""Parity of the HIP path against the CPU oracle, through the C ABI (ctypes shim).
+
+Bar: bit-exact for int32 outputs; fp16 outputs equal the exact integer rounded to nearest
+even (tolerance 0 ulp).  Sizes the oracle finishes in seconds are compared element by element;
+BASELINE's full sizes are checked on sampled rows plus size-independent identities.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+import lowbit_kernel as lk
+from _lib import (MODE_AND, MODE_XOR, MODE_ATTN, MODE_BWTA, MODE_ATTN_X, VARIANT_AUTO, VARIANT_VALU, VARIANT_MFMA)
+
+DEV = "cuda:0"
+VARIANTS = [VARIANT_VALU, VARIANT_MFMA]
+
+
+def rand_f16(rng, rows, K, zeros=True):
+    x = rng.standard_normal((rows, K)).astype(np.float16)
+    if zeros and K > 4:
+        idx = rng.integers(0, K, size=max(1, K // 16))
+        x[:, idx] = np.float16(0.0)
+        x[::2, idx[: len(idx) // 2]] = np.float16(-0.0)
+    return x
+
+
+def to_dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+def f16_of(i32):
+    with np.errstate(over="ignore"):
+        return i32.astype(np.float32).astype(np.float16)
+
+
+def oracle_all_modes(oracle, w, x):
+    K = w.shape[1]
+    Wp, Xp = oracle.c_pack_sign(w), oracle.c_pack_sign(x)
+    nz, sg = oracle.c_pack_ternary(x)
+    return {
+        MODE_AND: oracle.c_bgemm_packed(0, Wp, Xp, K),
+        MODE_XOR: oracle.c_bgemm_packed(1, Wp, Xp, K),
+        MODE_ATTN: oracle.c_bgemm_packed(2, Wp, Xp, K),
+        MODE_ATTN_X: np.ascontiguousarray(oracle.c_bgemm_packed(2, Xp, Wp, K).T),
+        MODE_BWTA: oracle.c_bwta_packed(Wp, nz, sg, K),
+    }
+
+
+# ------------------------------------------------------------------ packing
+def test_pack_known_answers(golden_dir):
+    kat = json.load(open(os.path.join(golden_dir, "pack_kat.json")))
+    for case in kat["sign"]:
+        h = torch.tensor([case["halves"]], dtype=torch.int32).to(torch.int16).view(torch.half).to(DEV)
+        got = lk.binary_weight_prepacking(h).cpu().numpy().view(np.uint32)
+        assert [int(v) for v in got[0]] == case["words"]
+        tiled = lk.pack_sign(h)
+        assert [int(v) for v in lk.logical_from_tiled(tiled).cpu().numpy().view(np.uint32)[0]] == case["words"]
+    for case in kat["ternary"]:
+        h = torch.tensor([case["halves"]], dtype=torch.int32).to(torch.int16).view(torch.half).to(DEV)
+        p = lk.pack_ternary(h)
+        assert [int(v) for v in lk.logical_from_tiled(p, 0).cpu().numpy().view(np.uint32)[0]] == case["nz"]
+        assert [int(v) for v in lk.logical_from_tiled(p, 1).cpu().numpy().view(np.uint32)[0]] == case["sg"]
+
+
+@pytest.mark.parametrize("rows,K", [(1, 1), (3, 31), (5, 33), (32, 256), (33, 257), (7, 784), (100, 4096),
+                                    (64, 520), (11008, 128)])
+def test_pack_matches_oracle(oracle, rows, K):
+    rng = np.random.default_rng(rows * 7919 + K)
+    x = rand_f16(rng, rows, K)
+    xd = to_dev(x)
+    want = oracle.c_pack_sign(x)
+    assert (lk.binary_weight_prepacking(xd).cpu().numpy().view(np.uint32) == want).all()
+    tiled = lk.pack_sign(xd)
+    assert tiled.data.numel() == ((rows + 31) // 32) * ((K + 255) // 256) * 256
+    assert (lk.logical_from_tiled(tiled).cpu().numpy().view(np.uint32) == want).all()
+    # logical -> tiled re-layout gives the same tiled words, padding included (all zero)
+    again = lk.tile_from_logical(to_dev(want.view(np.int32)), K)
+    assert torch.equal(again.data, tiled.data)
+    nz, sg = oracle.c_pack_ternary(x)
+    t = lk.pack_ternary(xd)
+    assert (lk.logical_from_tiled(t, 0).cpu().numpy().view(np.uint32) == nz).all()
+    assert (lk.logical_from_tiled(t, 1).cpu().numpy().view(np.uint32) == sg).all()
+
+
+def test_pack_strided_and_unaligned(oracle):
+    """Row stride > K and 2-byte-aligned starts go through the C ABI directly (the shim copies)."""
+    import _lib
+    L = _lib.lib()
+    rng = np.random.default_rng(11)
+    big = rand_f16(rng, 40, 1000)
+    bd = to_dev(big)
+    st = torch.cuda.current_stream().cuda_stream
+    for (r0, r1, k0, k1) in [(0, 40, 0, 1000), (3, 37, 1, 778), (5, 6, 7, 8), (0, 33, 8, 520)]:
+        rows, K = r1 - r0, k1 - k0
+        want = oracle.c_pack_sign(big[r0:r1, k0:k1])
+        src = bd.data_ptr() + 2 * (r0 * 1000 + k0)
+        tiled = torch.empty(L.bgemm_tiled_words(rows, K), dtype=torch.int32, device=DEV)
+        _lib.check(L.bgemm_pack_sign_f16(src, rows, K, 1000, tiled.data_ptr(), st))
+        got = lk.logical_from_tiled(lk.PackedBits(tiled.view(1, -1), None, 1, rows, K))
+        assert (got.cpu().numpy().view(np.uint32) == want).all()
+        logical = torch.empty((rows, (K + 31) // 32), dtype=torch.int32, device=DEV)
+        _lib.check(L.bgemm_pack_sign_f16_logical(src, rows, K, 1000, logical.data_ptr(), st))
+        assert (logical.cpu().numpy().view(np.uint32) == want).all()
+
+
+# ------------------------------------------------------------------ packed GEMM, small and ragged
+SMALL = [(1, 1, 1), (8, 5, 32), (33, 7, 40), (32, 32, 128), (10, 3, 784), (64, 1, 256), (65, 17, 300),
+         (130, 70, 1000), (256, 256, 512), (40, 200, 2304)]
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+@pytest.mark.parametrize("M,N,K", SMALL)
+def test_packed_small_all_modes(oracle, variant, M, N, K):
+    rng = np.random.default_rng(M * 1000003 + N * 1009 + K)
+    w, x = rand_f16(rng, M, K, zeros=False), rand_f16(rng, N, K)
+    want = oracle_all_modes(oracle, w, x)
+    wp, xp, xt = lk.pack_sign(to_dev(w)), lk.pack_sign(to_dev(x)), lk.pack_ternary(to_dev(x))
+    for mode in (MODE_AND, MODE_XOR, MODE_ATTN, MODE_ATTN_X, MODE_BWTA):
+        xin = xt if mode == MODE_BWTA else xp
+        for splitK in (1, 2, 5):
+            got = lk.bgemm_packed_forward(wp, xin, mode, torch.int32, splitK, variant)[0].cpu().numpy()
+            assert (got == want[mode]).all(), (mode, splitK)
+        goth = lk.bgemm_packed_forward(wp, xin, mode, torch.half, 3, variant)[0].cpu().numpy()
+        assert (goth.view(np.uint16) == f16_of(want[mode]).view(np.uint16)).all(), mode
+
+
+def test_packed_golden_dense(golden_dir):
+    d = np.load(os.path.join(golden_dir, "dense_kat.npz"))
+    names = {MODE_AND: "and", MODE_XOR: "xor", MODE_ATTN: "attn", MODE_ATTN_X: "attnx", MODE_BWTA: "bwta"}
+    for i in range(int(d["n_cases"])):
+        w = to_dev(d["w%d" % i].view(np.float16))
+        x = to_dev(d["x%d" % i].view(np.float16))
+        wp, xp, xt = lk.pack_sign(w), lk.pack_sign(x), lk.pack_ternary(x)
+        for variant in VARIANTS:
+            for mode, nm in names.items():
+                got = lk.bgemm_packed_forward(wp, xt if mode == MODE_BWTA else xp, mode, torch.int32, 1, variant)
+                assert (got[0].cpu().numpy() == d["%s%d" % (nm, i)]).all(), (i, nm, variant)
+
+
+# ------------------------------------------------------------------ BASELINE configurations
+def dense_ref(mode, w, x):
+    """Closed forms in fp32 on the CPU (exact: K < 2^24); the reference drivers' own method."""
+    a = torch.from_numpy((w.view(np.uint16) >> 15).astype(np.float32))
+    xs = x.view(np.uint16)
+    b = torch.from_numpy((xs >> 15).astype(np.float32))
+    if mode == MODE_XOR:
+        r = (1 - 2 * b) @ (1 - 2 * a).T
+    elif mode == MODE_AND:
+        r = b @ a.T
+    elif mode == MODE_ATTN:
+        r = (1 - 2 * b) @ (1 - a).T
+    elif mode == MODE_ATTN_X:
+        r = (1 - b) @ (1 - 2 * a).T
+    else:
+        t = torch.from_numpy(np.where((xs & 0x7FFF) == 0, 0, np.where(xs >> 15, -1, 1)).astype(np.float32))
+        r = t @ (1 - 2 * a).T
+    return r.to(torch.int32).numpy()
+
+
+def test_config1_bgemm_1024(oracle):
+    g = torch.Generator().manual_seed(1001)
+    a_bits = torch.randint(0, 2, (1024, 1024), generator=g).numpy()
+    b_bits = torch.randint(0, 2, (1024, 64), generator=g).numpy()
+    w16, x16 = oracle.bits_to_f16(a_bits), oracle.bits_to_f16(b_bits.T)
+    want = oracle.c_bgemm_packed(1, oracle.c_pack_sign(w16), oracle.c_pack_sign(x16), 1024)
+    wp, xp = lk.pack_sign(to_dev(w16)), lk.pack_sign(to_dev(x16))
+    for variant in VARIANTS:
+        for splitK in (1, 2, 4):
+            got = lk.bgemm_packed_forward(wp, xp, MODE_XOR, torch.int32, splitK, variant)[0].cpu().numpy()
+            assert (got == want).all()
+    out = lk.bgemm_linear_forward_cuda(to_dev(x16), to_dev(w16), 1, 1).cpu().numpy()
+    assert (out.view(np.uint16) == f16_of(want).view(np.uint16)).all()
+
+
+@pytest.mark.parametrize("N", [1, 4, 16])
+def test_config4_decode_bwta(N):
+    rng = np.random.default_rng(4000 + N)
+    M, K = 11008, 4096
+    w = np.where(rng.integers(0, 2, (M, K)) == 1, np.float16(-1), np.float16(1)).astype(np.float16)
+    t = rng.choice(np.array([-1, 0, 0, 1], dtype=np.float16), size=(N, K)).astype(np.float16)
+    want = dense_ref(MODE_BWTA, w, t)
+    wp, xt = lk.pack_sign(to_dev(w)), lk.pack_ternary(to_dev(t))
+    for variant in (VARIANT_AUTO, VARIANT_VALU, VARIANT_MFMA):
+        for splitK in (1, 2, 4, 8):
+            got = lk.bgemm_packed_forward(wp, xt, MODE_BWTA, torch.int32, splitK, variant)[0].cpu().numpy()
+            assert (got == want).all(), (variant, splitK)
+    goth = lk.bgemm_packed_forward(wp, xt, MODE_BWTA, torch.half, 8)[0].cpu().numpy()
+    assert (goth.view(np.uint16) == f16_of(want).view(np.uint16)).all()
+
+
+def test_config3_attention_av_batched():
+    rng = np.random.default_rng(3000)
+    B, S, D = 24, 512, 64                      # 24 of the 192 heads element by element
+    attn_bits = rng.integers(0, 2, (B, S, S))  # {0,1}, 1 = attend
+    v = np.where(rng.integers(0, 2, (B, S, D)) == 1, np.float16(-1), np.float16(1)).astype(np.float16)
+    attn16 = (2 * attn_bits - 1).astype(np.float16)            # "1" must have its sign bit clear
+    want = np.einsum("bqk,bkd->bqd", attn_bits.astype(np.float32), v.astype(np.float32)).astype(np.int32)
+    vt = np.ascontiguousarray(v.transpose(0, 2, 1))            # [B, D, S_k]
+    ap, vp = lk.pack_sign(to_dev(attn16)), lk.pack_sign(to_dev(vt))
+    for variant in (VARIANT_AUTO, VARIANT_VALU, VARIANT_MFMA):
+        # weight side = value^T (M = D), activation side = attn (N = S_q): output [B, S_q, D] directly
+        got = lk.bgemm_packed_forward(vp, ap, MODE_ATTN_X, torch.int32, 1, variant).cpu().numpy()
+        assert (got == want).all()
+        # the reference's orientation (attn as the weight side, INSTR=2) gives the transpose
+        got_t = lk.bgemm_packed_forward(ap, vp, MODE_ATTN, torch.int32, 1, variant).cpu().numpy()
+        assert (got_t.transpose(0, 2, 1) == want).all()
+
+
+@pytest.mark.parametrize("M,N,K,splitK", [(8192, 256, 4096, 1), (8192, 256, 4096, 4), (8192, 2048, 4096, 2),
+                                          (4096, 128, 4096, 1), (4096, 128, 784, 1), (10, 128, 4096, 4)])
+def test_config5_sweep_mid(M, N, K, splitK):
+    rng = np.random.default_rng(M + N + K + splitK)
+    w = np.where(rng.integers(0, 2, (M, K)) == 1, np.float16(-1), np.float16(1)).astype(np.float16)
+    x = np.where(rng.integers(0, 2, (N, K)) == 1, np.float16(-1), np.float16(1)).astype(np.float16)
+    want = dense_ref(MODE_XOR, w, x)
+    wp, xp = lk.pack_sign(to_dev(w)), lk.pack_sign(to_dev(x))
+    for variant in VARIANTS:
+        got = lk.bgemm_packed_forward(wp, xp, MODE_XOR, torch.int32, splitK, variant)[0].cpu().numpy()
+        assert (got == want).all(), variant
+
+
+def test_config5_full_8192_sampled_and_identities():
+    M = N = K = 8192
+    g = torch.Generator(device=DEV).manual_seed(5000)
+    wbits = torch.randint(0, 2, (M, K), generator=g, device=DEV, dtype=torch.int8)
+    xbits = torch.randint(0, 2, (N, K), generator=g, device=DEV, dtype=torch.int8)
+    w16 = (1 - 2 * wbits).to(torch.half)
+    x16 = (1 - 2 * xbits).to(torch.half)
+    wp, xp = lk.pack_sign(w16), lk.pack_sign(x16)
+    out = lk.bgemm_packed_forward(wp, xp, MODE_XOR, torch.int32, 1, VARIANT_MFMA)[0]
+    # (1) sampled rows/columns against the fp32 closed form on the CPU
+    rs = np.random.default_rng(5).choice(M, 96, replace=False)
+    cs = np.random.default_rng(6).choice(N, 80, replace=False)
+    wsub = w16[torch.from_numpy(rs).to(DEV)].float().cpu()
+    xsub = x16[torch.from_numpy(cs).to(DEV)].float().cpu()
+    want = (xsub @ wsub.T).to(torch.int32)
+    got = out[torch.from_numpy(cs).to(DEV)][:, torch.from_numpy(rs).to(DEV)].cpu()
+    assert torch.equal(got, want)
+    # (2) identities over the whole output: parity, range, checksum of checksums
+    assert int(((out - K) % 2).abs().max()) == 0 and int(out.abs().max()) <= K
+    col_sum = (1 - 2 * wbits).to(torch.float64).sum(0)               # sum_m s(w[m,k])
+    row_sum = (1 - 2 * xbits).to(torch.float64).sum(0)               # sum_n s(x[n,k])
+    assert int(out.to(torch.int64).sum()) == int((col_sum * row_sum).sum().item())
+    # (3) split-K and the VALU design agree bit for bit with the MFMA design
+    assert torch.equal(lk.bgemm_packed_forward(wp, xp, MODE_XOR, torch.int32, 4, VARIANT_MFMA)[0], out)
+    assert torch.equal(lk.bgemm_packed_forward(wp, xp, MODE_XOR, torch.int32, 1, VARIANT_VALU)[0], out)
+    # (4) C(w, w) has K on the diagonal; negating the weights negates the output
+    assert int(lk.bgemm_packed_forward(wp, wp, MODE_XOR, torch.int32)[0].diagonal().min()) == K
+    assert torch.equal(lk.bgemm_packed_forward(lk.pack_sign(-w16), xp, MODE_XOR, torch.int32)[0], -out)
+
+
+# ------------------------------------------------------------------ drop-in fp16 entry point
+@pytest.mark.parametrize("M,N,K", [(32, 32, 128), (64, 96, 640), (800, 128, 128), (10, 128, 4096), (33, 5, 100)])
+@pytest.mark.parametrize("INSTR", [0, 1, 2])
+def test_dropin_matches_reference_call(oracle, M, N, K, INSTR):
+    rng = np.random.default_rng(M * 31 + N * 17 + K + INSTR)
+    w, x = rand_f16(rng, M, K), rand_f16(rng, N, K)
+    for splitK in (1, 3):
+        want_h, _ = oracle.c_bgemm_f16(x, w, splitK, INSTR)
+        got = lk.bgemm_linear_forward_cuda(to_dev(x), to_dev(w), splitK, INSTR)
+        assert got.dtype == torch.half and tuple(got.shape) == (N, M)
+        assert (got.cpu().numpy().view(np.uint16) == want_h.view(np.uint16)).all()
+
+
+def test_dropin_rounds_to_nearest_even(oracle):
+    K = 4224
+    w = -np.ones((32, K), dtype=np.float16)
+    x = np.ones((32, K), dtype=np.float16)
+    x[:, :4099] = -1
+    got = lk.bgemm_linear_forward_cuda(to_dev(x), to_dev(w), 1, 0).cpu().numpy()
+    assert (got == np.float16(4100)).all()
+    want_h, _ = oracle.c_bgemm_f16(x, w, 1, 0)
+    assert (got.view(np.uint16) == want_h.view(np.uint16)).all()
+
+
+def test_dropin_argument_errors():
+    x = torch.zeros(32, 128, dtype=torch.half, device=DEV)
+    with pytest.raises(TypeError):
+        lk.bgemm_linear_forward_cuda(x.float(), x)
+    with pytest.raises(ValueError):
+        lk.bgemm_linear_forward_cuda(x, x[:, :64])
+    with pytest.raises(ValueError):
+        lk.bgemm_linear_forward_cuda(x, x, 1, 3)
+    with pytest.raises(ValueError):
+        lk.bgemm_linear_forward_cuda(x, x, 0, 1)
+
+
+def test_split_k_workspace_left_clean():
+    rng = np.random.default_rng(77)
+    w, x = rand_f16(rng, 96, 2048, zeros=False), rand_f16(rng, 40, 2048, zeros=False)
+    wp, xp = lk.pack_sign(to_dev(w)), lk.pack_sign(to_dev(x))
+    first = lk.bgemm_packed_forward(wp, xp, MODE_XOR, torch.int32, 4, VARIANT_MFMA)
+    for variant in VARIANTS:
+        for _ in range(3):
+            assert torch.equal(lk.bgemm_packed_forward(wp, xp, MODE_XOR, torch.int32, 4, variant), first)
+    torch.cuda.synchronize()
+    for buf in lk._zero_ws.values():
+        assert int(buf.count_nonzero()) == 0
