@@ -45,6 +45,35 @@ def time_gpu(fn, warmup, steps):
     return e0.elapsed_time(e1) / steps
 
 
+def time_gpu_graph(fn, n_launch, warmup, replays):
+    """Average milliseconds per launch with the CPU launch cost removed: n_launch calls of fn(i)
+    are captured into one HIP graph, which is replayed `replays` times between two events."""
+    import torch
+    for i in range(min(n_launch, max(warmup, 1))):
+        fn(i)                                   # also grows any cached buffers before capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        for i in range(n_launch):
+            fn(i)                               # warm the side stream's buffers eagerly
+        side.synchronize()
+        with torch.cuda.graph(g, stream=side):
+            for i in range(n_launch):
+                fn(i)
+    torch.cuda.synchronize()
+    g.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(replays):
+        g.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / (replays * n_launch)
+
+
 def pm1_f16(shape, seed, device):
     import torch
     g = torch.Generator(device=device).manual_seed(seed)
@@ -123,13 +152,14 @@ def bench_c4(steps, warmup, N, splitK, variant=0, copies=64):
     wps = [lk.PackedBits(base.data.clone(), None, 1, M, K) for _ in range(copies)]
     out = torch.empty((1, N, M), dtype=torch.int32, device=dev)
     fn = lambda i: lk.bgemm_packed_forward(wps[i % copies], xt, lk.MODE_BWTA, torch.int32, splitK, variant, out=out)
-    ms = time_gpu(fn, warmup, steps)
+    ms_eager = time_gpu(fn, warmup, steps)
+    ms = time_gpu_graph(fn, copies, 4, max(2, steps // copies))
     want = (torch.sign(x16.float()).cpu() @ w16.float().cpu().T).to(torch.int32)
     ok = bool(torch.equal(out[0].cpu(), want))
     ops = 2.0 * M * N * K
     bytes_alg = M * K / 8 + 2 * N * K / 8 + 4.0 * M * N
     return {"name": "C4 BWTA W[11008,4096] N=%d splitK=%d" % (N, splitK), "ms": ms, "tops": ops / ms / 1e9,
-            "gbs": bytes_alg / ms / 1e6, "ops": ops, "bytes": bytes_alg, "bit_exact": ok}
+            "ms_eager_launch": ms_eager, "gbs": bytes_alg / ms / 1e6, "ops": ops, "bytes": bytes_alg, "bit_exact": ok}
 
 
 def bench_c3(steps, warmup, variant=0):
@@ -143,12 +173,14 @@ def bench_c3(steps, warmup, variant=0):
     ap, vp = lk.pack_sign(attn16), lk.pack_sign(v16.transpose(1, 2).contiguous())
     out = torch.empty((B, S, D), dtype=torch.int32, device=dev)
     fn = lambda i: lk.bgemm_packed_forward(vp, ap, lk.MODE_ATTN_X, torch.int32, 1, variant, out=out)
-    ms = time_gpu(fn, warmup, steps)
+    ms_eager = time_gpu(fn, warmup, steps)
+    ms = time_gpu_graph(fn, 20, 4, max(2, steps // 20))
     want = torch.bmm((attn16[:4] > 0).float(), v16[:4].float()).to(torch.int32)
     ok = bool(torch.equal(out[:4], want))
     ops = 2.0 * B * S * S * D
     bytes_alg = B * (S * S / 8 + S * D / 8 + 4.0 * S * D)
-    return {"name": "C3 attention AxV 192x[512,512]x[512,64]", "ms": ms, "tops": ops / ms / 1e9,
+    return {"name": "C3 attention AxV 192x[512,512]x[512,64]", "ms": ms, "ms_eager_launch": ms_eager,
+            "tops": ops / ms / 1e9,
             "gbs": bytes_alg / ms / 1e6, "ops": ops, "bytes": bytes_alg, "bit_exact": ok}
 
 
@@ -181,7 +213,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--all", action="store_true", help="also time the other BASELINE configurations")
-    ap.add_argument("--variant", type=int, default=0, help="0 auto, 1 VALU, 2 MFMA")
+    ap.add_argument("--variant", type=int, default=0, help="0 auto, 1 VALU, 2 MFMA int8, 3 MFMA fp4")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:

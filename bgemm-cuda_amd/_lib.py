@@ -12,7 +12,7 @@ SO_PATH = os.path.join(_HERE, "libbgemm_mi355x.so")
 OK, EINVAL, ENULL, EWORKSPACE, ELAUNCH, EALIGN = 0, -1, -2, -3, -4, -5
 MODE_AND, MODE_XOR, MODE_ATTN, MODE_BWTA, MODE_ATTN_X = 0, 1, 2, 3, 4
 OUT_I32, OUT_F16 = 0, 1
-VARIANT_AUTO, VARIANT_VALU, VARIANT_MFMA = 0, 1, 2
+VARIANT_AUTO, VARIANT_VALU, VARIANT_MFMA, VARIANT_MFMA_F4 = 0, 1, 2, 3
 
 _i64, _p, _int, _sz = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
 
@@ -27,10 +27,10 @@ SIGNATURES = {
     "bgemm_tile_from_logical": (_int, [_p, _i64, _i64, _p, _p]),
     "bgemm_logical_from_tiled": (_int, [_p, _i64, _i64, _p, _p]),
     "bgemm_packed_workspace_bytes": (_sz, [_int, _i64, _i64, _i64, _i64, _int, _int]),
+    "bgemm_packed_counter_bytes": (_sz, [_int, _i64, _i64, _i64, _i64, _int, _int]),
     "bgemm_packed_forward": (_int, [_int, _p, _p, _p, _p, _int, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
-                                    _int, _int, _p, _sz, _p]),
+                                    _int, _int, _p, _sz, _p, _sz, _p]),
     "bgemm_f16_workspace_bytes": (_sz, [_i64, _i64, _i64, _int]),
-    "bgemm_f16_workspace_zero_bytes": (_sz, [_i64, _i64, _i64, _int]),
     "bgemm_f16_forward": (_int, [_p, _p, _p, _i64, _i64, _i64, _p, _sz, _int, _int, _p]),
 }
 

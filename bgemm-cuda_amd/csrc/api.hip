@@ -24,18 +24,26 @@ int check_launch(const char* what)
 
 static size_t round256(size_t x) { return (x + 255) / 256 * 256; }
 
-// Split-K state: int32 running sums [batch][N][M], then one arrival counter per output tile
-// of the finest tiling any kernel uses (32 x 64 outputs).
-static size_t splitk_acc_bytes(int64_t batch, int64_t M, int64_t N) { return round256((size_t)batch * N * M * 4); }
-static size_t splitk_cnt_bytes(int64_t batch, int64_t M, int64_t N)
+// Shape policy.  The matrix-core path wins whenever there is enough work per weight tile to
+// amortise the bit expansion; the fp4 engine runs at twice the int8 rate.
+static int pick_variant(int mode, int64_t batch, int64_t M, int64_t N, int64_t K)
 {
-    return round256((size_t)batch * cdiv(N, 32) * cdiv(M, 64) * 4);
+    (void)mode; (void)batch; (void)M; (void)N; (void)K;
+    return BGEMM_VARIANT_MFMA;
 }
 
-static int pick_variant(const GemmArgs& a)
+static void ws_needs(int variant, int planes, int64_t batch, int64_t M, int64_t N, int splitK,
+                     size_t* part, size_t* counters)
 {
-    (void)a;
-    return BGEMM_VARIANT_MFMA;
+    if (variant == BGEMM_VARIANT_VALU) gemm_valu_ws(batch, M, N, splitK, planes, part, counters);
+    else gemm_mfma_ws(batch, M, N, splitK, planes, part, counters);
+}
+
+// one thread per counter
+__global__ void clear_counters_kernel(uint32_t* c, int64_t n)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) c[i] = 0u;
 }
 
 }  // namespace bgemm
@@ -43,20 +51,41 @@ static int pick_variant(const GemmArgs& a)
 using namespace bgemm;
 
 extern "C" const char* bgemm_last_error(void) { return g_err; }
-extern "C" int bgemm_abi_version(void) { return 1; }
+extern "C" int bgemm_abi_version(void) { return 2; }
+
+static bool ws_query(int mode, int64_t batch, int64_t M, int64_t N, int64_t K, int splitK, int variant,
+                     size_t* part, size_t* counters)
+{
+    ModeCoef mc;
+    *part = *counters = 0;
+    if (!mode_coef(mode, &mc) || splitK <= 1 || batch <= 0 || M <= 0 || N <= 0 || K <= 0) return false;
+    if (variant < BGEMM_VARIANT_AUTO || variant > BGEMM_VARIANT_MFMA_F4) return false;
+    const int v = variant == BGEMM_VARIANT_AUTO ? pick_variant(mode, batch, M, N, K) : variant;
+    ws_needs(v, mc.planes, batch, M, N, splitK, part, counters);
+    return true;
+}
 
 extern "C" size_t bgemm_packed_workspace_bytes(int mode, int64_t batch, int64_t M, int64_t N, int64_t K,
                                                int splitK, int variant)
 {
-    (void)mode; (void)K; (void)variant;
-    if (splitK <= 1 || batch <= 0 || M <= 0 || N <= 0) return 0;
-    return splitk_acc_bytes(batch, M, N) + splitk_cnt_bytes(batch, M, N);
+    size_t part, cnt;
+    ws_query(mode, batch, M, N, K, splitK, variant, &part, &cnt);
+    return round256(part);
+}
+
+extern "C" size_t bgemm_packed_counter_bytes(int mode, int64_t batch, int64_t M, int64_t N, int64_t K,
+                                             int splitK, int variant)
+{
+    size_t part, cnt;
+    ws_query(mode, batch, M, N, K, splitK, variant, &part, &cnt);
+    return round256(cnt * 4);
 }
 
 extern "C" int bgemm_packed_forward(int mode, const void* W_tiled, const void* X_tiled, const void* X2_tiled,
                                     void* out, int out_dtype, int64_t batch, int64_t M, int64_t N, int64_t K,
                                     int64_t strideW, int64_t strideX, int64_t strideC,
-                                    int splitK, int variant, void* ws, size_t ws_bytes, void* stream)
+                                    int splitK, int variant, void* ws, size_t ws_bytes,
+                                    void* counters, size_t counter_bytes, void* stream)
 {
     g_err[0] = 0;
     GemmArgs a;
@@ -64,12 +93,12 @@ extern "C" int bgemm_packed_forward(int mode, const void* W_tiled, const void* X
     if (!mode_coef(mode, &a.mc)) return fail(BGEMM_EINVAL, "bgemm_packed_forward: unknown mode %d", mode);
     if (out_dtype != BGEMM_OUT_I32 && out_dtype != BGEMM_OUT_F16)
         return fail(BGEMM_EINVAL, "bgemm_packed_forward: unknown output dtype %d", out_dtype);
-    if (variant < BGEMM_VARIANT_AUTO || variant > BGEMM_VARIANT_MFMA)
+    if (variant < BGEMM_VARIANT_AUTO || variant > BGEMM_VARIANT_MFMA_F4)
         return fail(BGEMM_EINVAL, "bgemm_packed_forward: unknown variant %d", variant);
     if (batch < 0 || M < 0 || N < 0 || K < 0 || splitK < 1 || splitK > 65535)
         return fail(BGEMM_EINVAL, "bgemm_packed_forward: bad shape batch=%lld M=%lld N=%lld K=%lld splitK=%d",
                     (long long)batch, (long long)M, (long long)N, (long long)K, splitK);
-    if (K >= (1LL << 24))   // keeps |C| below 2^24: exact in the fp32 step of the fp16 store
+    if (K >= (1LL << 24))   // keeps |C| below 2^24: exact in fp32 (fp16 store, fp4 engine accumulator)
         return fail(BGEMM_EINVAL, "bgemm_packed_forward: K=%lld exceeds 2^24-1", (long long)K);
     if (batch > 0x7fffffff || M > 0x7fffffff || N > 0x7fffffff)
         return fail(BGEMM_EINVAL, "bgemm_packed_forward: dimension too large");
@@ -98,31 +127,33 @@ extern "C" int bgemm_packed_forward(int mode, const void* W_tiled, const void* X
     a.MT = (int)row_tiles(M); a.NT = (int)row_tiles(N); a.KT = (int)k_tiles(K);
     a.strideW = strideW / 4; a.strideX = strideX / 4; a.strideC = strideC;
     a.batch = (int)batch; a.splitK = splitK;
+    const int v = variant == BGEMM_VARIANT_AUTO ? pick_variant(mode, batch, M, N, K) : variant;
     if (splitK > 1) {
-        const size_t need = bgemm_packed_workspace_bytes(mode, batch, M, N, K, splitK, variant);
-        if (!ws) return fail(BGEMM_EWORKSPACE, "bgemm_packed_forward: splitK=%d needs a workspace of %zu bytes", splitK, need);
-        if (ws_bytes < need) return fail(BGEMM_EWORKSPACE, "bgemm_packed_forward: workspace %zu < %zu bytes", ws_bytes, need);
-        if ((uintptr_t)ws & 15) return fail(BGEMM_EALIGN, "bgemm_packed_forward: workspace must be 16-byte aligned");
-        a.ws_acc = (int32_t*)ws;
-        a.ws_cnt = (uint32_t*)((char*)ws + splitk_acc_bytes(batch, M, N));
+        size_t part, cnt;
+        ws_needs(v, a.mc.planes, batch, M, N, splitK, &part, &cnt);
+        if (!ws || !counters)
+            return fail(BGEMM_EWORKSPACE, "bgemm_packed_forward: splitK=%d needs %zu workspace and %zu counter bytes",
+                        splitK, round256(part), round256(cnt * 4));
+        if (ws_bytes < part) return fail(BGEMM_EWORKSPACE, "bgemm_packed_forward: workspace %zu < %zu bytes", ws_bytes, part);
+        if (counter_bytes < cnt * 4)
+            return fail(BGEMM_EWORKSPACE, "bgemm_packed_forward: counters %zu < %zu bytes", counter_bytes, cnt * 4);
+        if (((uintptr_t)ws & 15) || ((uintptr_t)counters & 3))
+            return fail(BGEMM_EALIGN, "bgemm_packed_forward: workspace must be 16-byte aligned");
+        a.ws_part = (int32_t*)ws;
+        a.ws_cnt = (uint32_t*)counters;
     }
-    int v = variant == BGEMM_VARIANT_AUTO ? pick_variant(a) : variant;
     if (v == BGEMM_VARIANT_VALU) return launch_gemm_valu(a, (hipStream_t)stream);
-    return launch_gemm_mfma(a, (hipStream_t)stream);
+    return launch_gemm_mfma(a, (hipStream_t)stream, v == BGEMM_VARIANT_MFMA_F4);
 }
 
 // ---- fp16-operand call: pack both operands into the workspace, then the packed GEMM ----
-// Workspace layout: [split-K state (zero contract)] [W tiled] [X tiled]
-extern "C" size_t bgemm_f16_workspace_zero_bytes(int64_t M, int64_t N, int64_t K, int splitK)
-{
-    return bgemm_packed_workspace_bytes(BGEMM_MODE_XOR, 1, M, N, K, splitK, BGEMM_VARIANT_AUTO);
-}
-
+// Workspace layout: [counters] [partial tiles] [W tiled] [X tiled], each rounded to 256 bytes.
 extern "C" size_t bgemm_f16_workspace_bytes(int64_t M, int64_t N, int64_t K, int splitK)
 {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
-    return bgemm_f16_workspace_zero_bytes(M, N, K, splitK) + round256((size_t)bgemm_tiled_words(M, K) * 4) +
-           round256((size_t)bgemm_tiled_words(N, K) * 4);
+    return bgemm_packed_counter_bytes(BGEMM_MODE_XOR, 1, M, N, K, splitK, BGEMM_VARIANT_AUTO) +
+           bgemm_packed_workspace_bytes(BGEMM_MODE_XOR, 1, M, N, K, splitK, BGEMM_VARIANT_AUTO) +
+           round256((size_t)bgemm_tiled_words(M, K) * 4) + round256((size_t)bgemm_tiled_words(N, K) * 4);
 }
 
 extern "C" int bgemm_f16_forward(const void* W, const void* X, void* C, int64_t M, int64_t N, int64_t K,
@@ -138,20 +169,30 @@ extern "C" int bgemm_f16_forward(const void* W, const void* X, void* C, int64_t 
     if (!C) return fail(BGEMM_ENULL, "bgemm_f16_forward: C is NULL");
     if (K == 0)
         return bgemm_packed_forward(INSTR, nullptr, nullptr, nullptr, C, BGEMM_OUT_F16, 1, M, N, 0, 0, 0, 0, 1,
-                                    BGEMM_VARIANT_AUTO, nullptr, 0, stream);
+                                    BGEMM_VARIANT_AUTO, nullptr, 0, nullptr, 0, stream);
     if (!W || !X) return fail(BGEMM_ENULL, "bgemm_f16_forward: operand pointer is NULL");
     const size_t need = bgemm_f16_workspace_bytes(M, N, K, splitK);
     if (!ws || ws_bytes < need)
         return fail(BGEMM_EWORKSPACE, "bgemm_f16_forward: workspace of %zu bytes required, %zu given", need,
                     ws ? ws_bytes : (size_t)0);
     if ((uintptr_t)ws & 255) return fail(BGEMM_EALIGN, "bgemm_f16_forward: workspace must be 256-byte aligned");
-    const size_t zb = bgemm_f16_workspace_zero_bytes(M, N, K, splitK);
-    char* wt = (char*)ws + zb;
+    const size_t cb = bgemm_packed_counter_bytes(INSTR, 1, M, N, K, splitK, BGEMM_VARIANT_AUTO);
+    const size_t pb = bgemm_packed_workspace_bytes(INSTR, 1, M, N, K, splitK, BGEMM_VARIANT_AUTO);
+    char* cnt = (char*)ws;
+    char* part = cnt + cb;
+    char* wt = part + pb;
     char* xt = wt + round256((size_t)bgemm_tiled_words(M, K) * 4);
+    if (cb) {   // a fill kernel rather than a memset node, so the call can be captured in a HIP graph
+        const int64_t n = (int64_t)(cb / 4);
+        hipLaunchKernelGGL(clear_counters_kernel, dim3((unsigned)cdiv(n, 256)), dim3(256), 0, (hipStream_t)stream,
+                           (uint32_t*)cnt, n);
+        int rc = check_launch("bgemm_f16_forward: clear counters");
+        if (rc) return rc;
+    }
     int rc = bgemm_pack_sign_f16(W, M, K, K, wt, stream);
     if (rc) return rc;
     rc = bgemm_pack_sign_f16(X, N, K, K, xt, stream);
     if (rc) return rc;
     return bgemm_packed_forward(INSTR, wt, xt, nullptr, C, BGEMM_OUT_F16, 1, M, N, K, 0, 0, 0, splitK,
-                                BGEMM_VARIANT_AUTO, ws, zb, stream);
+                                BGEMM_VARIANT_AUTO, part, pb, cnt, cb, stream);
 }

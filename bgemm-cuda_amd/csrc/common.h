@@ -50,7 +50,7 @@ struct GemmArgs {
     int64_t strideW, strideX, strideC;   // uint4 units for W/X, elements for C
     int batch, splitK;
     ModeCoef mc;
-    int32_t* ws_acc;      // split-K running sums, [batch][N][M], zero between calls
+    int32_t* ws_part;     // split-K partial tiles, [batch][tile][split] in register order (scratch)
     uint32_t* ws_cnt;     // split-K arrival counters, one per output tile, zero between calls
 };
 
@@ -72,9 +72,10 @@ __device__ __forceinline__ void store_out(void* out, int out_f16, int64_t idx, i
 }
 
 // Kernel families (each in its own translation unit).
-int launch_gemm_mfma(const GemmArgs& a, hipStream_t st);
+int launch_gemm_mfma(const GemmArgs& a, hipStream_t st, bool fp4);
 int launch_gemm_valu(const GemmArgs& a, hipStream_t st);
-size_t gemm_mfma_ws_bytes(int64_t batch, int64_t M, int64_t N, int64_t K, int splitK, int planes);
-bool gemm_valu_supported(const GemmArgs& a);
+// Split-K needs of each family for a shape: bytes of partial-tile scratch, number of counters.
+void gemm_mfma_ws(int64_t batch, int64_t M, int64_t N, int splitK, int planes, size_t* part_bytes, size_t* counters);
+void gemm_valu_ws(int64_t batch, int64_t M, int64_t N, int splitK, int planes, size_t* part_bytes, size_t* counters);
 
 }  // namespace bgemm

@@ -1,29 +1,65 @@
-// Design (b): AND-dot on the int8 matrix cores.
+// Design (b): AND-dot on the matrix cores.
 //
 // CDNA4 has no 1-bit MFMA.  Every mode reduces to the AND-dot D[n,m] = popc(a_m & b_n)
-// plus rank-one terms in the row popcounts (see ModeCoef), and D is an ordinary int8
-// GEMM of {0,1} matrices.  The operands stay bit-packed all the way into registers:
-// one 16-byte load per lane fetches a 32-row x 256-bit tile in exactly the order
-// v_mfma_i32_32x32x32_i8 wants its fragments (lane = half*32 + row), and the eight
-// 32-deep MFMA steps of the tile are produced by (word >> j) & 0x01010101, which turns
-// bit (8c+j) of each word into byte c.  Both operands use the same rule, so the
-// K permutation it implies cancels.  Waves never exchange data: no LDS, no barriers
-// in the main loop.  Row popcounts for the rank-one terms are accumulated from the
-// same registers (4 v_bcnt per fragment per tile).
+// plus rank-one terms in the row popcounts (see ModeCoef), and D is an ordinary GEMM of
+// {0,1} matrices.  The operands stay bit-packed all the way into registers: one 16-byte
+// load per lane fetches a 32-row x 256-bit tile in exactly the order the 32x32 MFMA wants
+// its fragments (lane = half*32 + row), and the MFMA steps of the tile are produced by a
+// shift and a mask per register.  Both operands use the same rule, so the K permutation it
+// implies cancels.  Waves never exchange data: no LDS, no barriers in the main loop.  Row
+// popcounts for the rank-one terms come from the same registers (4 v_bcnt per fragment).
 #include "common.h"
 
 namespace bgemm {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
 
-__device__ __forceinline__ v4i expand_bits(const uint4 w, const int j)
-{
-    v4i r;
-    r.x = (w.x >> j) & 0x01010101u; r.y = (w.y >> j) & 0x01010101u;
-    r.z = (w.z >> j) & 0x01010101u; r.w = (w.w >> j) & 0x01010101u;
-    return r;
-}
+// int8 engine: a 256-bit K-tile is eight 32-deep steps of v_mfma_i32_32x32x32_i8;
+// byte c of word q at step s is bit 8c+s.
+struct EngI8 {
+    typedef v16i Acc;
+    typedef v4i Frag;
+    static constexpr int STEPS = 8;
+    __device__ static __forceinline__ Frag expand(const uint4 w, const int s)
+    {
+        Frag r;
+        r.x = (w.x >> s) & 0x01010101u; r.y = (w.y >> s) & 0x01010101u;
+        r.z = (w.z >> s) & 0x01010101u; r.w = (w.w >> s) & 0x01010101u;
+        return r;
+    }
+    __device__ static __forceinline__ Acc mma(const Frag a, const Frag b, const Acc c)
+    {
+        return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
+    }
+    __device__ static __forceinline__ int to_int(const Acc& c, const int v) { return c[v]; }
+};
+
+// fp4 engine: the same tile is four 64-deep steps of v_mfma_f32_32x32x64_f8f6f4 with E2M1
+// operands; nibble c of word q at step s is bit 4c+s, moved to nibble bit 1 (0b0010 = 1.0).
+// Products are 0 or 1 and the fp32 accumulator holds integers below 2^24, so it stays exact.
+struct EngF4 {
+    typedef v16f Acc;
+    typedef v8i Frag;
+    static constexpr int STEPS = 4;
+    __device__ static __forceinline__ unsigned nib(const unsigned w, const int s)
+    {
+        return (s == 0 ? (w << 1) : (w >> (s - 1))) & 0x22222222u;
+    }
+    __device__ static __forceinline__ Frag expand(const uint4 w, const int s)
+    {
+        Frag r = {0, 0, 0, 0, 0, 0, 0, 0};
+        r[0] = nib(w.x, s); r[1] = nib(w.y, s); r[2] = nib(w.z, s); r[3] = nib(w.w, s);
+        return r;
+    }
+    __device__ static __forceinline__ Acc mma(const Frag a, const Frag b, const Acc c)
+    {
+        return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 4, 4, 0, 0, 0, 0);
+    }
+    __device__ static __forceinline__ int to_int(const Acc& c, const int v) { return (int)c[v]; }
+};
 
 __device__ __forceinline__ int popc4(const uint4 w)
 {
@@ -31,11 +67,10 @@ __device__ __forceinline__ int popc4(const uint4 w)
 }
 
 // Block = WGN x WGM waves, each wave owns WN x WM tiles of 32x32 outputs, PL activation planes.
-template <int WGN, int WGM, int WN, int WM, int PL>
+template <typename Eng, int WGN, int WGM, int WN, int WM, int PL>
 __global__ __launch_bounds__(WGN* WGM * 64) void gemm_mfma_kernel(const GemmArgs a, const int tiles_n,
                                                                    const int tiles_m)
 {
-    constexpr int NW = WGN * WGM;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int wn = wave / WGM, wm = wave % WGM;
 
@@ -81,7 +116,7 @@ __global__ __launch_bounds__(WGN* WGM * 64) void gemm_mfma_kernel(const GemmArgs
         wp[j] = Wb + (rt * a.KT) * TILE_U4 + lane;
     }
 
-    v16i acc[PL][WN][WM];
+    typename Eng::Acc acc[PL][WN][WM];
 #pragma unroll
     for (int p = 0; p < PL; p++)
 #pragma unroll
@@ -129,23 +164,22 @@ __global__ __launch_bounds__(WGN* WGM * 64) void gemm_mfma_kernel(const GemmArgs
 #pragma unroll
             for (int i = 0; i < WN; i++) pb[p][i] += popc4(xf[p][i]);
 #pragma unroll
-        for (int s = 0; s < 8; s++) {
-            v4i bw[WM];
+        for (int s = 0; s < Eng::STEPS; s++) {
+            typename Eng::Frag bw[WM];
 #pragma unroll
-            for (int j = 0; j < WM; j++) bw[j] = expand_bits(wf[j], s);
+            for (int j = 0; j < WM; j++) bw[j] = Eng::expand(wf[j], s);
 #pragma unroll
             for (int p = 0; p < PL; p++)
 #pragma unroll
                 for (int i = 0; i < WN; i++) {
-                    const v4i ax = expand_bits(xf[p][i], s);
+                    const typename Eng::Frag ax = Eng::expand(xf[p][i], s);
 #pragma unroll
-                    for (int j = 0; j < WM; j++)
-                        acc[p][i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ax, bw[j], acc[p][i][j], 0, 0, 0);
+                    for (int j = 0; j < WM; j++) acc[p][i][j] = Eng::mma(ax, bw[j], acc[p][i][j]);
                 }
         }
     }
 
-    // ---- epilogue: rank-one terms, then store or split-K accumulate -----------------
+    // ---- epilogue: rank-one terms turn the AND-dot into this split's share of C ------------
     const int64_t kbit0 = (int64_t)kt0 * TILE_KBITS;
     int64_t kbit1 = (int64_t)kt1 * TILE_KBITS;
     if (kbit1 > a.K) kbit1 = a.K;
@@ -159,58 +193,110 @@ __global__ __launch_bounds__(WGN* WGM * 64) void gemm_mfma_kernel(const GemmArgs
 
     const ModeCoef mc = a.mc;
     const int col = lane & 31, half = lane >> 5;
-    const bool direct = a.splitK == 1;
-    int* accum = direct ? nullptr : a.ws_acc + (int64_t)b * a.N * a.M;
-    char* outb = reinterpret_cast<char*>(a.out);
-    const int64_t out_off = (int64_t)b * a.strideC;
-#pragma unroll
-    for (int i = 0; i < WN; i++) {
+    // this split's share of C for tile row i (recomputed rather than kept: registers are tight)
+    auto tile_row_vals = [&](const int i, int (&val)[WM][16]) {
 #pragma unroll
         for (int v = 0; v < 16; v++) {
             const int nrow = 8 * (v >> 2) + 4 * half + (v & 3);
             const int pbv = __shfl(pb[0][i], nrow);
             const int pbv2 = PL == 2 ? __shfl(pb[PL - 1][i], nrow) : 0;
-            const int64_t n = (int64_t)(nt0 + i) * 32 + nrow;
+#pragma unroll
+            for (int j = 0; j < WM; j++) {
+                int t = mc.c0 * bits + mc.ca * pa[j] + mc.cb * pbv + mc.cd * Eng::to_int(acc[0][i][j], v);
+                if (PL == 2) t += mc.cb2 * pbv2 + mc.cd2 * Eng::to_int(acc[PL - 1][i][j], v);
+                val[j][v] = t;
+            }
+        }
+    };
+
+    // ---- split-K: partial tiles go to the workspace in register order (lane-contiguous
+    // 16-byte stores); the last split to arrive on a tile adds the others to its own.
+    constexpr int TILE_I4 = WGN * WN * WGM * WM * 256;          // int4 per block tile
+    int4* tile_base = nullptr;
+    if (a.splitK > 1) {
+        tile_base = reinterpret_cast<int4*>(a.ws_part) + ((int64_t)b * per_gemm + tile_id) * a.splitK * TILE_I4 +
+                    (int64_t)wave * (WN * WM * 256) + lane;
+        int4* mine = tile_base + (int64_t)split * TILE_I4;
+#pragma unroll
+        for (int i = 0; i < WN; i++) {
+            int val[WM][16];
+            tile_row_vals(i, val);
+#pragma unroll
+            for (int j = 0; j < WM; j++)
+#pragma unroll
+                for (int g = 0; g < 4; g++)
+                    mine[((i * WM + j) * 4 + g) * 64] =
+                        make_int4(val[j][4 * g], val[j][4 * g + 1], val[j][4 * g + 2], val[j][4 * g + 3]);
+        }
+        __shared__ int s_last;
+        __threadfence();            // release: partial visible device-wide before the ticket
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            unsigned* cnt = a.ws_cnt + (int64_t)b * per_gemm + tile_id;
+            const unsigned t = atomicAdd(cnt, 1u);
+            s_last = (t == (unsigned)a.splitK - 1u);
+            if (s_last) atomicExch(cnt, 0u);                     // counters are zero again after the call
+        }
+        __syncthreads();
+        if (!s_last) return;
+        __threadfence();            // acquire: see the other splits' partials
+    }
+
+    const int64_t out_off = (int64_t)b * a.strideC;
+#pragma unroll
+    for (int i = 0; i < WN; i++) {
+        int val[WM][16];
+        tile_row_vals(i, val);
+        if (a.splitK > 1) {
+            for (int s = 0; s < a.splitK; s++) {
+                if (s == split) continue;
+                const int4* other = tile_base + (int64_t)s * TILE_I4;
+#pragma unroll
+                for (int j = 0; j < WM; j++)
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        const int4 o = other[((i * WM + j) * 4 + g) * 64];
+                        val[j][4 * g] += o.x; val[j][4 * g + 1] += o.y;
+                        val[j][4 * g + 2] += o.z; val[j][4 * g + 3] += o.w;
+                    }
+            }
+        }
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            const int64_t n = (int64_t)(nt0 + i) * 32 + 8 * (v >> 2) + 4 * half + (v & 3);
 #pragma unroll
             for (int j = 0; j < WM; j++) {
                 const int64_t m = (int64_t)(mt0 + j) * 32 + col;
-                int val = mc.c0 * bits + mc.ca * pa[j] + mc.cb * pbv + mc.cd * acc[0][i][j][v];
-                if (PL == 2) val += mc.cb2 * pbv2 + mc.cd2 * acc[PL - 1][i][j][v];
-                if (n < a.N && m < a.M) {
-                    if (direct) store_out(outb, a.out_f16, out_off + n * a.M + m, val);
-                    else atomicAdd(accum + n * a.M + m, val);
-                }
+                if (n < a.N && m < a.M) store_out(a.out, a.out_f16, out_off + n * a.M + m, val[j][v]);
             }
         }
     }
-    if (direct) return;
-
-    // ---- split-K: the last split to arrive on this output tile publishes it ---------
-    __shared__ int s_last;
-    __threadfence();
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        const unsigned t = atomicAdd(a.ws_cnt + (int64_t)b * per_gemm + tile_id, 1u);
-        s_last = (t == (unsigned)a.splitK - 1u);
-    }
-    __syncthreads();
-    if (!s_last) return;
-    __threadfence();
-    constexpr int BN = WGN * WN * 32, BM = WGM * WM * 32;
-    const int64_t n_base = (int64_t)tn * BN, m_base = (int64_t)tm * BM;
-    for (int e = threadIdx.x; e < BN * BM; e += NW * 64) {
-        const int64_t n = n_base + e / BM, m = m_base + e % BM;
-        if (n < a.N && m < a.M) {
-            const int v = atomicExch(accum + n * a.M + m, 0);   // read the sum and leave zero behind
-            store_out(outb, a.out_f16, out_off + n * a.M + m, v);
-        }
-    }
-    if (threadIdx.x == 0) atomicExch(a.ws_cnt + (int64_t)b * per_gemm + tile_id, 0u);
 }
 
-struct TileCfg { int bn, bm; };
+// ---- host side ---------------------------------------------------------------------------
+struct MfmaCfg { int id, bn, bm; };
 
-template <int WGN, int WGM, int WN, int WM>
+// Tile choice: the largest tile that still yields about two blocks per CU.
+static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int splitK, int planes)
+{
+    const int64_t want = 512;
+    auto blocks = [&](int bn, int bm) { return batch * splitK * cdiv(N, bn) * cdiv(M, bm); };
+    if (planes == 1 && blocks(256, 256) >= want) return {0, 256, 256};
+    if (blocks(128, 128) >= want) return {1, 128, 128};
+    if (blocks(64, 128) >= want || N > 32) return {2, 64, 128};
+    return {3, 32, 128};
+}
+
+void gemm_mfma_ws(int64_t batch, int64_t M, int64_t N, int splitK, int planes, size_t* part_bytes,
+                  size_t* counters)
+{
+    const MfmaCfg c = pick_cfg(batch, M, N, splitK, planes);
+    const int64_t tiles = batch * cdiv(N, c.bn) * cdiv(M, c.bm);
+    *part_bytes = splitK > 1 ? (size_t)tiles * splitK * c.bn * c.bm * 4 : 0;
+    *counters = splitK > 1 ? (size_t)tiles : 0;
+}
+
+template <typename Eng, int WGN, int WGM, int WN, int WM>
 static int launch_cfg(const GemmArgs& a, hipStream_t st)
 {
     constexpr int BN = WGN * WN * 32, BM = WGM * WM * 32;
@@ -220,45 +306,30 @@ static int launch_cfg(const GemmArgs& a, hipStream_t st)
     if (a.mc.planes == 2) {
         // two accumulator sets: only the tiles whose registers fit are built for two planes
         if constexpr (WN * WM <= 4)
-            hipLaunchKernelGGL((gemm_mfma_kernel<WGN, WGM, WN, WM, 2>), dim3((unsigned)grid), dim3(WGN * WGM * 64), 0,
-                               st, a, tiles_n, tiles_m);
+            hipLaunchKernelGGL((gemm_mfma_kernel<Eng, WGN, WGM, WN, WM, 2>), dim3((unsigned)grid),
+                               dim3(WGN * WGM * 64), 0, st, a, tiles_n, tiles_m);
         else
             return fail(BGEMM_EINVAL, "gemm_mfma: tile not built for two planes");
     } else
-        hipLaunchKernelGGL((gemm_mfma_kernel<WGN, WGM, WN, WM, 1>), dim3((unsigned)grid), dim3(WGN * WGM * 64), 0, st,
-                           a, tiles_n, tiles_m);
+        hipLaunchKernelGGL((gemm_mfma_kernel<Eng, WGN, WGM, WN, WM, 1>), dim3((unsigned)grid), dim3(WGN * WGM * 64),
+                           0, st, a, tiles_n, tiles_m);
     return check_launch("gemm_mfma");
 }
 
-// Tile choice: the largest tile that still yields about two blocks per CU.
-static int pick_cfg(const GemmArgs& a)
+template <typename Eng>
+static int launch_eng(const GemmArgs& a, hipStream_t st)
 {
-    const int64_t want = 512;
-    auto blocks = [&](int bn, int bm) { return (int64_t)a.batch * a.splitK * cdiv(a.N, bn) * cdiv(a.M, bm); };
-    if (a.mc.planes == 1 && blocks(256, 256) >= want) return 0;
-    if (blocks(128, 128) >= want) return 1;
-    if (blocks(64, 128) >= want || a.N > 32) return 2;
-    return 3;
-}
-
-size_t gemm_mfma_ws_bytes(int64_t batch, int64_t M, int64_t N, int64_t K, int splitK, int planes)
-{
-    (void)K; (void)planes;
-    if (splitK <= 1) return 0;
-    // running sums + one counter per smallest tile (32 x 128 outputs), rounded to 256 bytes
-    const size_t accb = (size_t)batch * N * M * 4;
-    const size_t cnt = (size_t)batch * cdiv(N, 32) * cdiv(M, 128) * 4;
-    return ((accb + 255) / 256) * 256 + ((cnt + 255) / 256) * 256;
-}
-
-int launch_gemm_mfma(const GemmArgs& a, hipStream_t st)
-{
-    switch (pick_cfg(a)) {
-    case 0: return launch_cfg<2, 2, 4, 4>(a, st);    // 256 x 256
-    case 1: return launch_cfg<2, 2, 2, 2>(a, st);    // 128 x 128
-    case 2: return launch_cfg<1, 4, 2, 1>(a, st);    // 64 x 128
-    default: return launch_cfg<1, 4, 1, 1>(a, st);   // 32 x 128
+    switch (pick_cfg(a.batch, a.M, a.N, a.splitK, a.mc.planes).id) {
+    case 0: return launch_cfg<Eng, 2, 2, 4, 4>(a, st);    // 256 x 256
+    case 1: return launch_cfg<Eng, 2, 2, 2, 2>(a, st);    // 128 x 128
+    case 2: return launch_cfg<Eng, 1, 4, 2, 1>(a, st);    // 64 x 128
+    default: return launch_cfg<Eng, 1, 4, 1, 1>(a, st);   // 32 x 128
     }
+}
+
+int launch_gemm_mfma(const GemmArgs& a, hipStream_t st, bool fp4)
+{
+    return fp4 ? launch_eng<EngF4>(a, st) : launch_eng<EngI8>(a, st);
 }
 
 }  // namespace bgemm

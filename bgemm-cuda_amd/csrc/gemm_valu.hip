@@ -106,46 +106,61 @@ __global__ __launch_bounds__(256) void gemm_valu_kernel(const GemmArgs a, const 
     if (kbit1 > a.K) kbit1 = a.K;
     const int bits = kbit1 > kbit0 ? (int)(kbit1 - kbit0) : 0;
     const ModeCoef mc = a.mc;
-    const bool direct = a.splitK == 1;
-    int* accum = direct ? nullptr : a.ws_acc + (int64_t)b * a.N * a.M;
-    const int64_t out_off = (int64_t)b * a.strideC;
+    int val[4][4];
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const int nl = ty + 16 * i;
-        const int64_t n = (int64_t)tn * 64 + nl;
+    for (int i = 0; i < 4; i++)
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            const int ml = tx + 16 * j;
-            const int64_t m = (int64_t)tm * 64 + ml;
-            int val = mc.c0 * bits + mc.ca * sPopW[ml] + mc.cb * sPopX[0][nl] + mc.cd * acc[0][i][j];
-            if (PL == 2) val += mc.cb2 * sPopX[PL - 1][nl] + mc.cd2 * acc[PL - 1][i][j];
-            if (n < a.N && m < a.M) {
-                if (direct) store_out(a.out, a.out_f16, out_off + n * a.M + m, val);
-                else atomicAdd(accum + n * a.M + m, val);
+            int t = mc.c0 * bits + mc.ca * sPopW[tx + 16 * j] + mc.cb * sPopX[0][ty + 16 * i] + mc.cd * acc[0][i][j];
+            if (PL == 2) t += mc.cb2 * sPopX[PL - 1][ty + 16 * i] + mc.cd2 * acc[PL - 1][i][j];
+            val[i][j] = t;
+        }
+    if (a.splitK > 1) {
+        // partial tiles in register order; the last split to arrive adds the others to its own
+        int4* tile_base = reinterpret_cast<int4*>(a.ws_part) + ((int64_t)b * per_gemm + tile_id) * a.splitK * 1024 + tid;
+        int4* mine = tile_base + (int64_t)split * 1024;
+#pragma unroll
+        for (int i = 0; i < 4; i++) mine[i * 256] = make_int4(val[i][0], val[i][1], val[i][2], val[i][3]);
+        __threadfence();
+        __syncthreads();
+        if (tid == 0) {
+            unsigned* cnt = a.ws_cnt + (int64_t)b * per_gemm + tile_id;
+            const unsigned t = atomicAdd(cnt, 1u);
+            s_last = (t == (unsigned)a.splitK - 1u);
+            if (s_last) atomicExch(cnt, 0u);
+        }
+        __syncthreads();
+        if (!s_last) return;
+        __threadfence();
+        for (int s = 0; s < a.splitK; s++) {
+            if (s == split) continue;
+            const int4* other = tile_base + (int64_t)s * 1024;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int4 o = other[i * 256];
+                val[i][0] += o.x; val[i][1] += o.y; val[i][2] += o.z; val[i][3] += o.w;
             }
         }
     }
-    if (direct) return;
-    __threadfence();
-    __syncthreads();
-    if (tid == 0) {
-        const unsigned t = atomicAdd(a.ws_cnt + (int64_t)b * per_gemm + tile_id, 1u);
-        s_last = (t == (unsigned)a.splitK - 1u);
-    }
-    __syncthreads();
-    if (!s_last) return;
-    __threadfence();
-    for (int e = tid; e < 64 * 64; e += 256) {
-        const int64_t n = (int64_t)tn * 64 + e / 64, m = (int64_t)tm * 64 + e % 64;
-        if (n < a.N && m < a.M) {
-            const int v = atomicExch(accum + n * a.M + m, 0);
-            store_out(a.out, a.out_f16, out_off + n * a.M + m, v);
+    const int64_t out_off = (int64_t)b * a.strideC;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int64_t n = (int64_t)tn * 64 + ty + 16 * i;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int64_t m = (int64_t)tm * 64 + tx + 16 * j;
+            if (n < a.N && m < a.M) store_out(a.out, a.out_f16, out_off + n * a.M + m, val[i][j]);
         }
     }
-    if (tid == 0) atomicExch(a.ws_cnt + (int64_t)b * per_gemm + tile_id, 0u);
 }
 
-bool gemm_valu_supported(const GemmArgs&) { return true; }
+void gemm_valu_ws(int64_t batch, int64_t M, int64_t N, int splitK, int planes, size_t* part_bytes, size_t* counters)
+{
+    (void)planes;
+    const int64_t tiles = batch * cdiv(N, 64) * cdiv(M, 64);
+    *part_bytes = splitK > 1 ? (size_t)tiles * splitK * 64 * 64 * 4 : 0;
+    *counters = splitK > 1 ? (size_t)tiles : 0;
+}
 
 int launch_gemm_valu(const GemmArgs& a, hipStream_t st)
 {

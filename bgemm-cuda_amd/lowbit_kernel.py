@@ -13,7 +13,7 @@ import torch
 
 import _lib as _b
 from _lib import (MODE_AND, MODE_XOR, MODE_ATTN, MODE_BWTA, MODE_ATTN_X, OUT_I32, OUT_F16,
-                  VARIANT_AUTO, VARIANT_VALU, VARIANT_MFMA)
+                  VARIANT_AUTO, VARIANT_VALU, VARIANT_MFMA, VARIANT_MFMA_F4)
 
 AND_POP, XOR_POP, ATTN_MM = 0, 1, 2   # lowbit_kernel/csrc/include/configs.h:70-72
 
@@ -32,18 +32,24 @@ def _need_cuda(t, name):
         raise ValueError("%s must live on the GPU" % name)
 
 
-# Split-K state must be zero before first use and is left zero by every call, so one
-# zero-filled buffer per (device, stream) is grown on demand and reused.
-_zero_ws = {}
+# Split-K arrival counters must be zero before first use and every call leaves them zero, so
+# one zero-filled buffer per (device, stream) is grown on demand and reused; partial tiles
+# are plain scratch.
+_counters = {}
+_scratch = {}
 
 
-def _zeroed_workspace(nbytes, device):
+def _split_k_buffers(part_bytes, counter_bytes, device):
     key = (device.index, _stream())
-    buf = _zero_ws.get(key)
-    if buf is None or buf.numel() < nbytes:
-        buf = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
-        _zero_ws[key] = buf
-    return buf
+    cnt = _counters.get(key)
+    if cnt is None or cnt.numel() < counter_bytes:
+        cnt = torch.zeros(max(counter_bytes, 1 << 16), dtype=torch.uint8, device=device)
+        _counters[key] = cnt
+    ws = _scratch.get(key)
+    if ws is None or ws.numel() < part_bytes:
+        ws = torch.empty(max(part_bytes, 1 << 20), dtype=torch.uint8, device=device)
+        _scratch[key] = ws
+    return ws, cnt
 
 
 class PackedBits:
@@ -161,14 +167,16 @@ def bgemm_packed_forward(w, x, mode=MODE_XOR, out_dtype=torch.int32, splitK=1, v
         out = torch.empty((batch, N, M), dtype=out_dtype, device=dev)
     L = _b.lib()
     with torch.cuda.device(dev):
-        nws = L.bgemm_packed_workspace_bytes(mode, batch, M, N, K, splitK, variant)
-        ws = _zeroed_workspace(nws, dev) if nws else None
+        ws = cnt = None
+        if splitK > 1:
+            ws, cnt = _split_k_buffers(L.bgemm_packed_workspace_bytes(mode, batch, M, N, K, splitK, variant),
+                                       L.bgemm_packed_counter_bytes(mode, batch, M, N, K, splitK, variant), dev)
         _b.check(L.bgemm_packed_forward(
             mode, w.data.data_ptr(), x.data.data_ptr(), x.data2.data_ptr() if x.ternary else None,
             out.data_ptr(), OUT_F16 if out_dtype == torch.half else OUT_I32, batch, M, N, K,
-            w.words if w.batch > 1 else 0, x.words if x.batch > 1 else 0, N * M,
-            splitK, variant, ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0,
-            _stream()))
+            w.words if w.batch > 1 else 0, x.words if x.batch > 1 else 0, N * M, splitK, variant,
+            ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0,
+            cnt.data_ptr() if cnt is not None else None, cnt.numel() if cnt is not None else 0, _stream()))
     return out
 
 
@@ -192,12 +200,7 @@ def bgemm_linear_forward_cuda(in_feats, weights, splitK=1, INSTR=1):
     out = torch.empty((N, M), dtype=torch.half, device=x.device)
     L = _b.lib()
     with torch.cuda.device(x.device):
-        total = L.bgemm_f16_workspace_bytes(M, N, K, splitK)
-        zb = L.bgemm_f16_workspace_zero_bytes(M, N, K, splitK)
-        # [split-K state | packed W | packed X]: only the first zb bytes must start at zero
-        ws = torch.empty(max(total, 1), dtype=torch.uint8, device=x.device)
-        if zb:
-            ws[:zb].zero_()
+        ws = torch.empty(max(L.bgemm_f16_workspace_bytes(M, N, K, splitK), 1), dtype=torch.uint8, device=x.device)
         _b.check(L.bgemm_f16_forward(w.data_ptr(), x.data_ptr(), out.data_ptr(), M, N, K,
                                      ws.data_ptr(), ws.numel(), int(splitK), int(INSTR), _stream()))
     return out

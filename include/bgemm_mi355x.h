@@ -36,9 +36,11 @@ extern "C" {
 enum { BGEMM_MODE_AND = 0, BGEMM_MODE_XOR = 1, BGEMM_MODE_ATTN = 2, BGEMM_MODE_BWTA = 3,
        BGEMM_MODE_ATTN_X = 4 };
 enum { BGEMM_OUT_I32 = 0, BGEMM_OUT_F16 = 1 };
-/* Kernel family: AUTO picks per shape; VALU = xor/and + popcount on the vector ALU;
- * MFMA = bit planes expanded to int8 in registers feeding v_mfma_i32_32x32x32_i8. */
-enum { BGEMM_VARIANT_AUTO = 0, BGEMM_VARIANT_VALU = 1, BGEMM_VARIANT_MFMA = 2 };
+/* Kernel family: AUTO picks per shape; VALU = and + popcount on the vector ALU;
+ * MFMA = bit planes expanded to int8 in registers feeding v_mfma_i32_32x32x32_i8;
+ * MFMA_F4 = bit planes expanded to E2M1 nibbles feeding v_mfma_f32_32x32x64_f8f6f4
+ * (products are 0/1 and the fp32 accumulator stays below 2^24, so it is exact too). */
+enum { BGEMM_VARIANT_AUTO = 0, BGEMM_VARIANT_VALU = 1, BGEMM_VARIANT_MFMA = 2, BGEMM_VARIANT_MFMA_F4 = 3 };
 
 enum {
     BGEMM_OK = 0,
@@ -92,28 +94,32 @@ int bgemm_logical_from_tiled(const void* tiled, int64_t rows, int64_t K,
  *   batch    : number of independent GEMMs; strides in uint32 words / output elements
  *              (a stride of 0 shares that operand across the batch).
  *   splitK   : >= 1; K-tiles are divided into splitK contiguous ranges as in
- *              kernel_matmul.cuh:397-404, reduced inside the kernel with integer adds,
- *              so the result does not depend on it.
- *   ws       : needed iff bgemm_packed_workspace_bytes() > 0.  Must be zero-filled
- *              once before first use; every call leaves it zero-filled again.
+ *              kernel_matmul.cuh:397-404 and reduced inside the same launch with integer
+ *              adds, so the result does not depend on it.
+ *   ws       : scratch for split-K partial tiles, bgemm_packed_workspace_bytes() bytes,
+ *              no initialisation needed (NULL when that is 0).
+ *   counters : split-K arrival counters, bgemm_packed_counter_bytes() bytes.  Must be
+ *              zero-filled once before first use; every call leaves them zero again.
+ *              Calls that share counters must not overlap in time.
  */
 size_t bgemm_packed_workspace_bytes(int mode, int64_t batch, int64_t M, int64_t N, int64_t K,
                                     int splitK, int variant);
+size_t bgemm_packed_counter_bytes(int mode, int64_t batch, int64_t M, int64_t N, int64_t K,
+                                  int splitK, int variant);
 int bgemm_packed_forward(int mode, const void* W_tiled, const void* X_tiled, const void* X2_tiled,
                          void* out, int out_dtype, int64_t batch, int64_t M, int64_t N, int64_t K,
                          int64_t strideW, int64_t strideX, int64_t strideC,
-                         int splitK, int variant, void* ws, size_t ws_bytes, void* stream);
+                         int splitK, int variant, void* ws, size_t ws_bytes,
+                         void* counters, size_t counter_bytes, void* stream);
 
 /* ---- fp16-operand call, the drop-in for the reference launcher -----------------------
  * Same argument meaning as bin_pack_linear_kernel (fp6_linear.cu:275-286):
  * W = weights half [M][K], X = in_feats half [N][K], C = half [N][M], INSTR in {0,1,2}.
  * Differences: any M, N, K >= 1 (the reference asserts M%32, N%32, K%128); the
- * workspace is bytes of scratch (packed operands + split-K state) instead of fp32
- * partial planes, and has the same zero-fill contract as above for its first
- * bgemm_f16_workspace_zero_bytes() bytes.
+ * workspace is bytes of scratch (packed operands + split-K state, no initialisation
+ * needed: the call clears its own counters) instead of fp32 partial planes.
  */
 size_t bgemm_f16_workspace_bytes(int64_t M, int64_t N, int64_t K, int splitK);
-size_t bgemm_f16_workspace_zero_bytes(int64_t M, int64_t N, int64_t K, int splitK);
 int bgemm_f16_forward(const void* W, const void* X, void* C, int64_t M, int64_t N, int64_t K,
                       void* ws, size_t ws_bytes, int splitK, int INSTR, void* stream);
 

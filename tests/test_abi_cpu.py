@@ -29,21 +29,25 @@ def test_header_symbols_exported():
 
 def test_layout_sizes():
     L = _lib.lib()
-    assert L.bgemm_abi_version() == 1
+    assert L.bgemm_abi_version() == 2
     assert L.bgemm_tiled_words(1, 1) == 256
     assert L.bgemm_tiled_words(32, 256) == 256
     assert L.bgemm_tiled_words(33, 257) == 4 * 256
     assert L.bgemm_tiled_words(11008, 4096) == 11008 * 4096 // 32
     assert L.bgemm_tiled_words(0, 128) == 0
     assert L.bgemm_packed_workspace_bytes(1, 1, 64, 64, 1024, 1, 0) == 0
-    assert L.bgemm_packed_workspace_bytes(1, 1, 64, 64, 1024, 4, 0) >= 64 * 64 * 4 + 4
+    assert L.bgemm_packed_workspace_bytes(1, 1, 64, 64, 1024, 4, 0) >= 4 * 64 * 64 * 4
+    assert L.bgemm_packed_counter_bytes(1, 1, 64, 64, 1024, 4, 0) >= 4
+    assert L.bgemm_packed_counter_bytes(1, 1, 64, 64, 1024, 1, 0) == 0
+    for variant in (1, 2, 3):           # every family states its needs for the same shape
+        assert L.bgemm_packed_workspace_bytes(1, 2, 100, 70, 1024, 3, variant) >= 2 * 3 * 100 * 70 * 4
     assert L.bgemm_f16_workspace_bytes(64, 32, 256, 1) >= (64 + 32) * 256 // 8
 
 
 @pytest.mark.parametrize("kwargs, code", [
     (dict(mode=7), _lib.EINVAL),
     (dict(out_dtype=5), _lib.EINVAL),
-    (dict(variant=9), _lib.EINVAL),
+    (dict(variant=4), _lib.EINVAL),
     (dict(M=-1), _lib.EINVAL),
     (dict(splitK=0), _lib.EINVAL),
     (dict(K=1 << 24), _lib.EINVAL),
@@ -52,17 +56,21 @@ def test_layout_sizes():
     (dict(mode=3), _lib.ENULL),                       # BWTA without the second plane
     (dict(W=0x1008), _lib.EALIGN),
     (dict(splitK=2), _lib.EWORKSPACE),                # no workspace given
-    (dict(splitK=2, ws=0x10000, ws_bytes=16), _lib.EWORKSPACE),
+    (dict(splitK=2, ws=0x10000, ws_bytes=1 << 20), _lib.EWORKSPACE),            # no counters given
+    (dict(splitK=2, ws=0x10000, ws_bytes=16, cnt=0x20000, cnt_bytes=4096), _lib.EWORKSPACE),
+    (dict(splitK=2, ws=0x10000, ws_bytes=1 << 20, cnt=0x20000, cnt_bytes=0), _lib.EWORKSPACE),
+    (dict(splitK=2, ws=0x10004, ws_bytes=1 << 20, cnt=0x20000, cnt_bytes=4096), _lib.EALIGN),
     (dict(strideW=2), _lib.EINVAL),
 ])
 def test_packed_forward_rejects(kwargs, code):
     L = _lib.lib()
     a = dict(mode=1, W=0x1000, X=0x2000, X2=None, out=0x3000, out_dtype=0, batch=1, M=64, N=64, K=256,
-             strideW=0, strideX=0, strideC=0, splitK=1, variant=0, ws=None, ws_bytes=0, stream=None)
+             strideW=0, strideX=0, strideC=0, splitK=1, variant=0, ws=None, ws_bytes=0, cnt=None, cnt_bytes=0,
+             stream=None)
     a.update(kwargs)
     rc = L.bgemm_packed_forward(a["mode"], a["W"], a["X"], a["X2"], a["out"], a["out_dtype"], a["batch"], a["M"],
                                 a["N"], a["K"], a["strideW"], a["strideX"], a["strideC"], a["splitK"], a["variant"],
-                                a["ws"], a["ws_bytes"], a["stream"])
+                                a["ws"], a["ws_bytes"], a["cnt"], a["cnt_bytes"], a["stream"])
     assert rc == code
     assert L.bgemm_last_error()            # a message was recorded
     with pytest.raises(ValueError):
@@ -71,8 +79,8 @@ def test_packed_forward_rejects(kwargs, code):
 
 def test_empty_problems_are_ok_without_launch():
     L = _lib.lib()
-    assert L.bgemm_packed_forward(1, None, None, None, None, 0, 0, 64, 64, 256, 0, 0, 0, 1, 0, None, 0, None) == 0
-    assert L.bgemm_packed_forward(1, None, None, None, None, 0, 1, 0, 64, 256, 0, 0, 0, 1, 0, None, 0, None) == 0
+    assert L.bgemm_packed_forward(1, None, None, None, None, 0, 0, 64, 64, 256, 0, 0, 0, 1, 0, None, 0, None, 0, None) == 0
+    assert L.bgemm_packed_forward(1, None, None, None, None, 0, 1, 0, 64, 256, 0, 0, 0, 1, 0, None, 0, None, 0, None) == 0
     assert L.bgemm_pack_sign_f16(None, 0, 128, 128, None, None) == 0
     assert L.bgemm_f16_forward(None, None, None, 0, 5, 128, None, 0, 1, 1, None) == 0
 

@@ -14,10 +14,11 @@ import torch
 pytestmark = pytest.mark.gpu
 
 import lowbit_kernel as lk
-from _lib import (MODE_AND, MODE_XOR, MODE_ATTN, MODE_BWTA, MODE_ATTN_X, VARIANT_AUTO, VARIANT_VALU, VARIANT_MFMA)
+from _lib import (MODE_AND, MODE_XOR, MODE_ATTN, MODE_BWTA, MODE_ATTN_X, VARIANT_AUTO, VARIANT_VALU, VARIANT_MFMA,
+                  VARIANT_MFMA_F4)
 
 DEV = "cuda:0"
-VARIANTS = [VARIANT_VALU, VARIANT_MFMA]
+VARIANTS = [VARIANT_VALU, VARIANT_MFMA, VARIANT_MFMA_F4]
 
 
 def rand_f16(rng, rows, K, zeros=True):
@@ -185,7 +186,7 @@ def test_config4_decode_bwta(N):
     t = rng.choice(np.array([-1, 0, 0, 1], dtype=np.float16), size=(N, K)).astype(np.float16)
     want = dense_ref(MODE_BWTA, w, t)
     wp, xt = lk.pack_sign(to_dev(w)), lk.pack_ternary(to_dev(t))
-    for variant in (VARIANT_AUTO, VARIANT_VALU, VARIANT_MFMA):
+    for variant in [VARIANT_AUTO] + VARIANTS:
         for splitK in (1, 2, 4, 8):
             got = lk.bgemm_packed_forward(wp, xt, MODE_BWTA, torch.int32, splitK, variant)[0].cpu().numpy()
             assert (got == want).all(), (variant, splitK)
@@ -202,7 +203,7 @@ def test_config3_attention_av_batched():
     want = np.einsum("bqk,bkd->bqd", attn_bits.astype(np.float32), v.astype(np.float32)).astype(np.int32)
     vt = np.ascontiguousarray(v.transpose(0, 2, 1))            # [B, D, S_k]
     ap, vp = lk.pack_sign(to_dev(attn16)), lk.pack_sign(to_dev(vt))
-    for variant in (VARIANT_AUTO, VARIANT_VALU, VARIANT_MFMA):
+    for variant in [VARIANT_AUTO] + VARIANTS:
         # weight side = value^T (M = D), activation side = attn (N = S_q): output [B, S_q, D] directly
         got = lk.bgemm_packed_forward(vp, ap, MODE_ATTN_X, torch.int32, 1, variant).cpu().numpy()
         assert (got == want).all()
@@ -249,9 +250,27 @@ def test_config5_full_8192_sampled_and_identities():
     # (3) split-K and the VALU design agree bit for bit with the MFMA design
     assert torch.equal(lk.bgemm_packed_forward(wp, xp, MODE_XOR, torch.int32, 4, VARIANT_MFMA)[0], out)
     assert torch.equal(lk.bgemm_packed_forward(wp, xp, MODE_XOR, torch.int32, 1, VARIANT_VALU)[0], out)
+    assert torch.equal(lk.bgemm_packed_forward(wp, xp, MODE_XOR, torch.int32, 1, VARIANT_MFMA_F4)[0], out)
+    assert torch.equal(lk.bgemm_packed_forward(wp, xp, MODE_XOR, torch.int32, 2, VARIANT_MFMA_F4)[0], out)
     # (4) C(w, w) has K on the diagonal; negating the weights negates the output
     assert int(lk.bgemm_packed_forward(wp, wp, MODE_XOR, torch.int32)[0].diagonal().min()) == K
     assert torch.equal(lk.bgemm_packed_forward(lk.pack_sign(-w16), xp, MODE_XOR, torch.int32)[0], -out)
+
+
+@pytest.mark.parametrize("variant", [VARIANT_MFMA, VARIANT_MFMA_F4, VARIANT_VALU])
+def test_large_k_accumulators_stay_exact(variant):
+    """Worst case for the accumulators: every bit set, so the AND-dot equals K.  K = 2^22 keeps the fp4
+    engine's fp32 accumulator far above the point where a narrower internal adder would lose bits."""
+    K = 1 << 22
+    ones = torch.full((32, K // 32), -1, dtype=torch.int32, device=DEV)         # all sign bits set
+    half_ones = ones.clone()
+    half_ones[:, ::2] = 0                                                        # every other word clear
+    wp, xp = lk.tile_from_logical(ones, K), lk.tile_from_logical(half_ones, K)
+    assert int(lk.bgemm_packed_forward(wp, wp, MODE_AND, torch.int32, 1, variant).min()) == K
+    assert int(lk.bgemm_packed_forward(wp, wp, MODE_XOR, torch.int32, 1, variant).min()) == K
+    got = lk.bgemm_packed_forward(wp, xp, MODE_AND, torch.int32, 3, variant)
+    assert int(got.min()) == K // 2 and int(got.max()) == K // 2
+    assert int(lk.bgemm_packed_forward(wp, xp, MODE_XOR, torch.int32, 1, variant).abs().max()) == 0
 
 
 # ------------------------------------------------------------------ drop-in fp16 entry point
@@ -299,5 +318,6 @@ def test_split_k_workspace_left_clean():
         for _ in range(3):
             assert torch.equal(lk.bgemm_packed_forward(wp, xp, MODE_XOR, torch.int32, 4, variant), first)
     torch.cuda.synchronize()
-    for buf in lk._zero_ws.values():
+    assert lk._counters
+    for buf in lk._counters.values():
         assert int(buf.count_nonzero()) == 0
