@@ -127,6 +127,7 @@ extern "C" int bgemm_packed_forward(int mode, const void* W_tiled, const void* X
     a.MT = (int)row_tiles(M); a.NT = (int)row_tiles(N); a.KT = (int)k_tiles(K);
     a.strideW = strideW / 4; a.strideX = strideX / 4; a.strideC = strideC;
     a.batch = (int)batch; a.splitK = splitK;
+    a.vec_store = (M % 4 == 0) && (strideC % 4 == 0) && (((uintptr_t)out & 15) == 0);
     const int v = variant == BGEMM_VARIANT_AUTO ? pick_variant(mode, batch, M, N, K) : variant;
     if (splitK > 1) {
         size_t part, cnt;

@@ -45,6 +45,7 @@ static inline bool mode_coef(int mode, ModeCoef* mc)
 struct GemmArgs {
     const uint4* W; const uint4* X; const uint4* X2;
     void* out; int out_f16;
+    int vec_store;        // rows of `out` are 16-byte aligned: the epilogue may store four elements per lane
     int64_t M, N, K;
     int MT, NT, KT;
     int64_t strideW, strideX, strideC;   // uint4 units for W/X, elements for C

@@ -133,6 +133,7 @@ __global__ __launch_bounds__(WGN* WGM * 64) void gemm_mfma_kernel(const GemmArgs
 #pragma unroll
         for (int i = 0; i < WN; i++) pb[p][i] = 0;
 
+    // ---- main loop: raw tiles are prefetched one K-tile ahead ----------------------------------
     uint4 xf[PL][WN], wf[WM], xn[PL][WN], wn_[WM];
     if (kt0 < kt1) {
 #pragma unroll
@@ -191,19 +192,24 @@ __global__ __launch_bounds__(WGN* WGM * 64) void gemm_mfma_kernel(const GemmArgs
 #pragma unroll
         for (int i = 0; i < WN; i++) pb[p][i] += __shfl_xor(pb[p][i], 32);
 
+    // All factors stay below 2^24 (K < 2^24, small coefficients), so the full-rate 24-bit
+    // multiply is exact; v_mul_lo_u32 would cost four times as much per element.
     const ModeCoef mc = a.mc;
     const int col = lane & 31, half = lane >> 5;
+    int capa[WM];
+#pragma unroll
+    for (int j = 0; j < WM; j++) capa[j] = __mul24(mc.c0, bits) + __mul24(mc.ca, pa[j]);
     // this split's share of C for tile row i (recomputed rather than kept: registers are tight)
     auto tile_row_vals = [&](const int i, int (&val)[WM][16]) {
 #pragma unroll
         for (int v = 0; v < 16; v++) {
             const int nrow = 8 * (v >> 2) + 4 * half + (v & 3);
-            const int pbv = __shfl(pb[0][i], nrow);
-            const int pbv2 = PL == 2 ? __shfl(pb[PL - 1][i], nrow) : 0;
+            int rowterm = __mul24(mc.cb, __shfl(pb[0][i], nrow));
+            if (PL == 2) rowterm += __mul24(mc.cb2, __shfl(pb[PL - 1][i], nrow));
 #pragma unroll
             for (int j = 0; j < WM; j++) {
-                int t = mc.c0 * bits + mc.ca * pa[j] + mc.cb * pbv + mc.cd * Eng::to_int(acc[0][i][j], v);
-                if (PL == 2) t += mc.cb2 * pbv2 + mc.cd2 * Eng::to_int(acc[PL - 1][i][j], v);
+                int t = capa[j] + rowterm + __mul24(mc.cd, Eng::to_int(acc[0][i][j], v));
+                if (PL == 2) t += __mul24(mc.cd2, Eng::to_int(acc[PL - 1][i][j], v));
                 val[j][v] = t;
             }
         }
@@ -242,7 +248,21 @@ __global__ __launch_bounds__(WGN* WGM * 64) void gemm_mfma_kernel(const GemmArgs
         __threadfence();            // acquire: see the other splits' partials
     }
 
-    const int64_t out_off = (int64_t)b * a.strideC;
+    // ---- store ------------------------------------------------------------------------------
+    constexpr int ROW_I = WM * 32 + 8;       // staged row stride in ints (+8 keeps the two lane halves on
+                                             // different LDS banks)
+    __shared__ __align__(16) int stage[WGN * WGM * 32 * ROW_I];
+    const int esz_shift = a.out_f16 ? 1 : 2;
+    char* const out_base = reinterpret_cast<char*>(a.out) + (((int64_t)b * a.strideC) << esz_shift);
+    const int64_t row_bytes = a.M << esz_shift;
+    int coff[WM];
+    bool cok[WM];
+#pragma unroll
+    for (int j = 0; j < WM; j++) {
+        const int64_t m = (int64_t)(mt0 + j) * 32 + col;
+        cok[j] = m < a.M;
+        coff[j] = (int)(cok[j] ? m : 0) << esz_shift;
+    }
 #pragma unroll
     for (int i = 0; i < WN; i++) {
         int val[WM][16];
@@ -261,13 +281,47 @@ __global__ __launch_bounds__(WGN* WGM * 64) void gemm_mfma_kernel(const GemmArgs
                     }
             }
         }
+        if (a.vec_store) {
+            // transpose through LDS so that every lane owns four consecutive outputs of one row:
+            // 16-byte stores, one instruction covers 64 * 4 consecutive elements of the tile row
+            int* st = stage + wave * (32 * ROW_I);
+#pragma unroll
+            for (int v = 0; v < 16; v++)
+#pragma unroll
+                for (int j = 0; j < WM; j++) st[(8 * (v >> 2) + 4 * half + (v & 3)) * ROW_I + j * 32 + col] = val[j][v];
+            __syncthreads();
+            constexpr int C4 = WM * 8;               // int4 per staged row
+#pragma unroll
+            for (int p = 0; p < 32 * C4 / 64; p++) {
+                const int idx = p * 64 + lane, row = idx / C4, c4 = idx % C4;
+                const int4 q = *reinterpret_cast<const int4*>(st + row * ROW_I + c4 * 4);
+                const int64_t n = (int64_t)(nt0 + i) * 32 + row, m = (int64_t)mt0 * 32 + c4 * 4;
+                if (n < a.N && m < a.M) {
+                    char* const dst = out_base + n * row_bytes + (m << esz_shift);
+                    if (a.out_f16) {
+                        union { __half h[4]; uint2 u; } pk;
+                        pk.h[0] = __float2half_rn((float)q.x); pk.h[1] = __float2half_rn((float)q.y);
+                        pk.h[2] = __float2half_rn((float)q.z); pk.h[3] = __float2half_rn((float)q.w);
+                        *reinterpret_cast<uint2*>(dst) = pk.u;
+                    } else
+                        *reinterpret_cast<int4*>(dst) = q;
+                }
+            }
+            __syncthreads();
+            continue;
+        }
+        const int64_t n0 = (int64_t)(nt0 + i) * 32 + 4 * half;
+        char* const tile_row0 = out_base + n0 * row_bytes;
 #pragma unroll
         for (int v = 0; v < 16; v++) {
-            const int64_t n = (int64_t)(nt0 + i) * 32 + 8 * (v >> 2) + 4 * half + (v & 3);
+            const int dn = 8 * (v >> 2) + (v & 3);
+            if (n0 + dn >= a.N) continue;
+            char* const rowp = tile_row0 + dn * row_bytes;
 #pragma unroll
             for (int j = 0; j < WM; j++) {
-                const int64_t m = (int64_t)(mt0 + j) * 32 + col;
-                if (n < a.N && m < a.M) store_out(a.out, a.out_f16, out_off + n * a.M + m, val[j][v]);
+                if (!cok[j]) continue;
+                if (a.out_f16) *reinterpret_cast<__half*>(rowp + coff[j]) = __float2half_rn((float)val[j][v]);
+                else *reinterpret_cast<int*>(rowp + coff[j]) = val[j][v];
             }
         }
     }
@@ -321,6 +375,8 @@ static int launch_eng(const GemmArgs& a, hipStream_t st)
 {
     switch (pick_cfg(a.batch, a.M, a.N, a.splitK, a.mc.planes).id) {
     case 0: return launch_cfg<Eng, 2, 2, 4, 4>(a, st);    // 256 x 256
+    case 4: return launch_cfg<Eng, 2, 2, 4, 2>(a, st);    // 256 x 128, two blocks per CU
+    case 5: return launch_cfg<Eng, 2, 2, 2, 4>(a, st);    // 128 x 256, two blocks per CU
     case 1: return launch_cfg<Eng, 2, 2, 2, 2>(a, st);    // 128 x 128
     case 2: return launch_cfg<Eng, 1, 4, 2, 1>(a, st);    // 64 x 128
     default: return launch_cfg<Eng, 1, 4, 1, 1>(a, st);   // 32 x 128
