@@ -29,12 +29,16 @@ static size_t round256(size_t x) { return (x + 255) / 256 * 256; }
 static int pick_variant(int mode, int64_t batch, int64_t M, int64_t N, int64_t K)
 {
     (void)mode; (void)batch; (void)M; (void)N; (void)K;
-    return BGEMM_VARIANT_MFMA;
+    return BGEMM_VARIANT_MFMA_F4;
 }
+
+static bool skinny_shape(int planes, int64_t N) { return planes == 2 ? N <= 16 : N <= 32; }
 
 static void ws_needs(int variant, int planes, int64_t batch, int64_t M, int64_t N, int splitK,
                      size_t* part, size_t* counters)
 {
+    *part = *counters = 0;
+    if (variant != BGEMM_VARIANT_VALU && skinny_shape(planes, N)) return;      // split inside the block
     if (variant == BGEMM_VARIANT_VALU) gemm_valu_ws(batch, M, N, splitK, planes, part, counters);
     else gemm_mfma_ws(batch, M, N, splitK, planes, part, counters);
 }
@@ -129,7 +133,8 @@ extern "C" int bgemm_packed_forward(int mode, const void* W_tiled, const void* X
     a.batch = (int)batch; a.splitK = splitK;
     a.vec_store = (M % 4 == 0) && (strideC % 4 == 0) && (((uintptr_t)out & 15) == 0);
     const int v = variant == BGEMM_VARIANT_AUTO ? pick_variant(mode, batch, M, N, K) : variant;
-    if (splitK > 1) {
+    const bool skinny = v != BGEMM_VARIANT_VALU && gemm_skinny_eligible(a);
+    if (splitK > 1 && !skinny) {
         size_t part, cnt;
         ws_needs(v, a.mc.planes, batch, M, N, splitK, &part, &cnt);
         if (!ws || !counters)
@@ -144,6 +149,7 @@ extern "C" int bgemm_packed_forward(int mode, const void* W_tiled, const void* X
         a.ws_cnt = (uint32_t*)counters;
     }
     if (v == BGEMM_VARIANT_VALU) return launch_gemm_valu(a, (hipStream_t)stream);
+    if (skinny) return launch_gemm_skinny(a, (hipStream_t)stream, v == BGEMM_VARIANT_MFMA_F4);
     return launch_gemm_mfma(a, (hipStream_t)stream, v == BGEMM_VARIANT_MFMA_F4);
 }
 

@@ -64,6 +64,69 @@ __host__ __device__ static inline void split_range(int KT, int splitK, int s, in
     *k0 = st; *k1 = st + n;
 }
 
+// Hardware deals workgroups round-robin over the 8 XCDs (workgroup i runs on XCD i % 8, each XCD
+// with its own L2).  This maps the hardware id to a logical id such that every XCD owns one
+// contiguous run of logical ids: neighbouring tiles then share an L2.
+__device__ __forceinline__ unsigned xcd_contiguous_id(const unsigned hw_id, const unsigned grid)
+{
+    const unsigned per = grid / 8, rem = grid % 8, x = hw_id % 8, y = hw_id / 8;
+    return x * per + (x < rem ? x : rem) + y;
+}
+
+// Split-K hand-over between the blocks that share an output tile.  The grid is laid out so that
+// these blocks carry the same hardware id modulo 8, i.e. run on one XCD and meet in one L2: the
+// partial tile only has to have reached that L2 (stores complete) before the arrival ticket is
+// taken, and the last block reads it with device-scope loads that bypass its L1.  A block that
+// finds itself on another XCD than its id implies says so in the ticket and falls back to
+// device-scope fences (whole-L2 write-back / invalidate, far slower), as does the reader then.
+// Returns true in every thread of the block that arrived last.  Counters return to zero.
+__device__ __forceinline__ bool splitk_arrive(unsigned* counter, const unsigned splits, int* s_flag)
+{
+    asm volatile("s_waitcnt vmcnt(0)" : : : "memory");     // this thread's partial stores have been acknowledged
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const unsigned xcc = __builtin_amdgcn_s_getreg((3 << 11) | 20) & 0xf;    // XCC_ID[3:0]
+        const bool home = xcc == (blockIdx.x & 7u);
+        if (!home) __threadfence();
+        const unsigned t = atomicAdd(counter, home ? 1u : 0x10001u);
+        const int last = (t & 0xffffu) == splits - 1u;
+        if (last) {
+            atomicExch(counter, 0u);
+            if (!home || (t >> 16)) __threadfence();
+        }
+        *s_flag = last;
+    }
+    __syncthreads();
+    return *s_flag != 0;
+}
+
+// Device-scope load of one partial-tile vector (bypasses the reader's L1).
+__device__ __forceinline__ int4 load_partial(const int4* p)
+{
+    const int* q = reinterpret_cast<const int*>(p);
+    int4 v;
+    v.x = __hip_atomic_load(q + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    v.y = __hip_atomic_load(q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    v.z = __hip_atomic_load(q + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    v.w = __hip_atomic_load(q + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return v;
+}
+
+// Split-K grids are padded to a multiple of 8 * splitK blocks and numbered split-fastest, so
+// the splits of a tile fall into one XCD's contiguous run of logical ids.
+static inline int64_t splitk_grid(int64_t real_blocks, int splitK)
+{
+    return splitK > 1 ? cdiv(real_blocks, 8 * (int64_t)splitK) * 8 * splitK : real_blocks;
+}
+// More K ranges than needed to give every CU a few blocks only add hand-over traffic: the
+// result does not depend on the split, so the caller's value is treated as an upper bound.
+static inline int effective_split(int64_t tiles, int splitK, int KT)
+{
+    int s = splitK;
+    while (s > 1 && (tiles * s > 512 || s > KT)) s--;
+    return s;
+}
+
 // Final store of one output element: int32 as is, or fp16 = the integer rounded to nearest
 // even (exact through fp32 because |v| < 2^24).
 __device__ __forceinline__ void store_out(void* out, int out_f16, int64_t idx, int v)
@@ -75,6 +138,9 @@ __device__ __forceinline__ void store_out(void* out, int out_f16, int64_t idx, i
 // Kernel families (each in its own translation unit).
 int launch_gemm_mfma(const GemmArgs& a, hipStream_t st, bool fp4);
 int launch_gemm_valu(const GemmArgs& a, hipStream_t st);
+// Skinny shapes (activation side fits one 32-row operand): in-block split-K, no workspace.
+bool gemm_skinny_eligible(const GemmArgs& a);
+int launch_gemm_skinny(const GemmArgs& a, hipStream_t st, bool fp4);
 // Split-K needs of each family for a shape: bytes of partial-tile scratch, number of counters.
 void gemm_mfma_ws(int64_t batch, int64_t M, int64_t N, int splitK, int planes, size_t* part_bytes, size_t* counters);
 void gemm_valu_ws(int64_t batch, int64_t M, int64_t N, int splitK, int planes, size_t* part_bytes, size_t* counters);

@@ -9,62 +9,9 @@
 // implies cancels.  Waves never exchange data: no LDS, no barriers in the main loop.  Row
 // popcounts for the rank-one terms come from the same registers (4 v_bcnt per fragment).
 #include "common.h"
+#include "mfma_engines.h"
 
 namespace bgemm {
-
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef int v8i __attribute__((ext_vector_type(8)));
-typedef int v16i __attribute__((ext_vector_type(16)));
-typedef float v16f __attribute__((ext_vector_type(16)));
-
-// int8 engine: a 256-bit K-tile is eight 32-deep steps of v_mfma_i32_32x32x32_i8;
-// byte c of word q at step s is bit 8c+s.
-struct EngI8 {
-    typedef v16i Acc;
-    typedef v4i Frag;
-    static constexpr int STEPS = 8;
-    __device__ static __forceinline__ Frag expand(const uint4 w, const int s)
-    {
-        Frag r;
-        r.x = (w.x >> s) & 0x01010101u; r.y = (w.y >> s) & 0x01010101u;
-        r.z = (w.z >> s) & 0x01010101u; r.w = (w.w >> s) & 0x01010101u;
-        return r;
-    }
-    __device__ static __forceinline__ Acc mma(const Frag a, const Frag b, const Acc c)
-    {
-        return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
-    }
-    __device__ static __forceinline__ int to_int(const Acc& c, const int v) { return c[v]; }
-};
-
-// fp4 engine: the same tile is four 64-deep steps of v_mfma_f32_32x32x64_f8f6f4 with E2M1
-// operands; nibble c of word q at step s is bit 4c+s, moved to nibble bit 1 (0b0010 = 1.0).
-// Products are 0 or 1 and the fp32 accumulator holds integers below 2^24, so it stays exact.
-struct EngF4 {
-    typedef v16f Acc;
-    typedef v8i Frag;
-    static constexpr int STEPS = 4;
-    __device__ static __forceinline__ unsigned nib(const unsigned w, const int s)
-    {
-        return (s == 0 ? (w << 1) : (w >> (s - 1))) & 0x22222222u;
-    }
-    __device__ static __forceinline__ Frag expand(const uint4 w, const int s)
-    {
-        Frag r = {0, 0, 0, 0, 0, 0, 0, 0};
-        r[0] = nib(w.x, s); r[1] = nib(w.y, s); r[2] = nib(w.z, s); r[3] = nib(w.w, s);
-        return r;
-    }
-    __device__ static __forceinline__ Acc mma(const Frag a, const Frag b, const Acc c)
-    {
-        return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 4, 4, 0, 0, 0, 0);
-    }
-    __device__ static __forceinline__ int to_int(const Acc& c, const int v) { return (int)c[v]; }
-};
-
-__device__ __forceinline__ int popc4(const uint4 w)
-{
-    return __popc(w.x) + __popc(w.y) + __popc(w.z) + __popc(w.w);
-}
 
 // Block = WGN x WGM waves, each wave owns WN x WM tiles of 32x32 outputs, PL activation planes.
 template <typename Eng, int WGN, int WGM, int WN, int WM, int PL>
@@ -74,18 +21,13 @@ __global__ __launch_bounds__(WGN* WGM * 64) void gemm_mfma_kernel(const GemmArgs
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int wn = wave / WGM, wm = wave % WGM;
 
-    // XCD-aware decode: hardware deals workgroups round-robin over the 8 XCDs, so give
-    // each XCD a contiguous run of logical ids (neighbouring tiles then share one L2).
-    const unsigned G = gridDim.x;
-    unsigned bid = blockIdx.x;
-    {
-        const unsigned per = G / 8, rem = G % 8, x = bid % 8, y = bid / 8;
-        bid = x * per + (x < rem ? x : rem) + y;
-    }
+    // logical block id: XCD-contiguous, split fastest (see xcd_contiguous_id / splitk_grid)
+    const unsigned bid = xcd_contiguous_id(blockIdx.x, gridDim.x);
     const int per_gemm = tiles_n * tiles_m;
-    const int tile_id = bid % per_gemm;
-    const int bs = bid / per_gemm;
-    const int split = bs % a.splitK, b = bs / a.splitK;
+    const int split = bid % a.splitK;
+    const unsigned rest = bid / a.splitK;
+    const int tile_id = rest % per_gemm, b = rest / per_gemm;
+    if (b >= a.batch) return;                    // padding blocks of a split-K grid
     // group tiles in bands of 8 along n so a band reuses its weight panels
     const int band = 8;
     const int band_id = tile_id / (band * tiles_m), in_band = tile_id % (band * tiles_m);
@@ -235,17 +177,7 @@ __global__ __launch_bounds__(WGN* WGM * 64) void gemm_mfma_kernel(const GemmArgs
                         make_int4(val[j][4 * g], val[j][4 * g + 1], val[j][4 * g + 2], val[j][4 * g + 3]);
         }
         __shared__ int s_last;
-        __threadfence();            // release: partial visible device-wide before the ticket
-        __syncthreads();
-        if (threadIdx.x == 0) {
-            unsigned* cnt = a.ws_cnt + (int64_t)b * per_gemm + tile_id;
-            const unsigned t = atomicAdd(cnt, 1u);
-            s_last = (t == (unsigned)a.splitK - 1u);
-            if (s_last) atomicExch(cnt, 0u);                     // counters are zero again after the call
-        }
-        __syncthreads();
-        if (!s_last) return;
-        __threadfence();            // acquire: see the other splits' partials
+        if (!splitk_arrive(a.ws_cnt + (int64_t)b * per_gemm + tile_id, (unsigned)a.splitK, &s_last)) return;
     }
 
     // ---- store ------------------------------------------------------------------------------
@@ -275,7 +207,7 @@ __global__ __launch_bounds__(WGN* WGM * 64) void gemm_mfma_kernel(const GemmArgs
                 for (int j = 0; j < WM; j++)
 #pragma unroll
                     for (int g = 0; g < 4; g++) {
-                        const int4 o = other[((i * WM + j) * 4 + g) * 64];
+                        const int4 o = load_partial(other + ((i * WM + j) * 4 + g) * 64);
                         val[j][4 * g] += o.x; val[j][4 * g + 1] += o.y;
                         val[j][4 * g + 2] += o.z; val[j][4 * g + 3] += o.w;
                     }
@@ -355,7 +287,7 @@ static int launch_cfg(const GemmArgs& a, hipStream_t st)
 {
     constexpr int BN = WGN * WN * 32, BM = WGM * WM * 32;
     const int tiles_n = (int)cdiv(a.N, BN), tiles_m = (int)cdiv(a.M, BM);
-    const int64_t grid = (int64_t)a.batch * a.splitK * tiles_n * tiles_m;
+    const int64_t grid = splitk_grid((int64_t)a.batch * a.splitK * tiles_n * tiles_m, a.splitK);
     if (grid <= 0 || grid > 0x7fffffffLL) return fail(BGEMM_EINVAL, "gemm_mfma: grid of %lld blocks", (long long)grid);
     if (a.mc.planes == 2) {
         // two accumulator sets: only the tiles whose registers fit are built for two planes
@@ -371,9 +303,12 @@ static int launch_cfg(const GemmArgs& a, hipStream_t st)
 }
 
 template <typename Eng>
-static int launch_eng(const GemmArgs& a, hipStream_t st)
+static int launch_eng(const GemmArgs& a_in, hipStream_t st)
 {
-    switch (pick_cfg(a.batch, a.M, a.N, a.splitK, a.mc.planes).id) {
+    GemmArgs a = a_in;
+    const MfmaCfg cfg = pick_cfg(a.batch, a.M, a.N, a.splitK, a.mc.planes);   // as the workspace was sized
+    a.splitK = effective_split((int64_t)a.batch * cdiv(a.N, cfg.bn) * cdiv(a.M, cfg.bm), a.splitK, a.KT);
+    switch (cfg.id) {
     case 0: return launch_cfg<Eng, 2, 2, 4, 4>(a, st);    // 256 x 256
     case 4: return launch_cfg<Eng, 2, 2, 4, 2>(a, st);    // 256 x 128, two blocks per CU
     case 5: return launch_cfg<Eng, 2, 2, 2, 4>(a, st);    // 128 x 256, two blocks per CU

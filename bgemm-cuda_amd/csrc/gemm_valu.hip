@@ -31,9 +31,11 @@ __global__ __launch_bounds__(256) void gemm_valu_kernel(const GemmArgs a, const 
 
     const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
     const int per_gemm = tiles_n * tiles_m;
-    const unsigned bid = blockIdx.x;
-    const int tile_id = bid % per_gemm, bs = bid / per_gemm;
-    const int split = bs % a.splitK, b = bs / a.splitK;
+    const unsigned bid = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    const int split = bid % a.splitK;
+    const unsigned rest = bid / a.splitK;
+    const int tile_id = rest % per_gemm, b = rest / per_gemm;
+    if (b >= a.batch) return;                    // padding blocks of a split-K grid
     const int tn = tile_id / tiles_m, tm = tile_id % tiles_m;
     int kt0, kt1;
     split_range(a.KT, a.splitK, split, &kt0, &kt1);
@@ -121,23 +123,13 @@ __global__ __launch_bounds__(256) void gemm_valu_kernel(const GemmArgs a, const 
         int4* mine = tile_base + (int64_t)split * 1024;
 #pragma unroll
         for (int i = 0; i < 4; i++) mine[i * 256] = make_int4(val[i][0], val[i][1], val[i][2], val[i][3]);
-        __threadfence();
-        __syncthreads();
-        if (tid == 0) {
-            unsigned* cnt = a.ws_cnt + (int64_t)b * per_gemm + tile_id;
-            const unsigned t = atomicAdd(cnt, 1u);
-            s_last = (t == (unsigned)a.splitK - 1u);
-            if (s_last) atomicExch(cnt, 0u);
-        }
-        __syncthreads();
-        if (!s_last) return;
-        __threadfence();
+        if (!splitk_arrive(a.ws_cnt + (int64_t)b * per_gemm + tile_id, (unsigned)a.splitK, &s_last)) return;
         for (int s = 0; s < a.splitK; s++) {
             if (s == split) continue;
             const int4* other = tile_base + (int64_t)s * 1024;
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                const int4 o = other[i * 256];
+                const int4 o = load_partial(other + i * 256);
                 val[i][0] += o.x; val[i][1] += o.y; val[i][2] += o.z; val[i][3] += o.w;
             }
         }
@@ -162,10 +154,12 @@ void gemm_valu_ws(int64_t batch, int64_t M, int64_t N, int splitK, int planes, s
     *counters = splitK > 1 ? (size_t)tiles : 0;
 }
 
-int launch_gemm_valu(const GemmArgs& a, hipStream_t st)
+int launch_gemm_valu(const GemmArgs& a_in, hipStream_t st)
 {
+    GemmArgs a = a_in;
     const int tiles_n = (int)cdiv(a.N, 64), tiles_m = (int)cdiv(a.M, 64);
-    const int64_t grid = (int64_t)a.batch * a.splitK * tiles_n * tiles_m;
+    a.splitK = effective_split((int64_t)a.batch * tiles_n * tiles_m, a.splitK, a.KT);
+    const int64_t grid = splitk_grid((int64_t)a.batch * a.splitK * tiles_n * tiles_m, a.splitK);
     if (grid <= 0 || grid > 0x7fffffffLL) return fail(BGEMM_EINVAL, "gemm_valu: grid of %lld blocks", (long long)grid);
     if (a.mc.planes == 2)
         hipLaunchKernelGGL((gemm_valu_kernel<2>), dim3((unsigned)grid), dim3(256), 0, st, a, tiles_n, tiles_m);
