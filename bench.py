@@ -23,6 +23,7 @@ for _p in (ROOT, os.path.join(ROOT, "bgemm-cuda_amd")):
         sys.path.insert(0, _p)
 
 INT8_MFMA_PEAK_TOPS = 5000.0      # MI355X dense int8 MFMA, published
+FP4_MFMA_PEAK_TOPS = 10100.0      # MI355X dense fp4 MFMA, published
 HBM_PEAK_GBS = 8000.0             # MI355X HBM3E, published
 
 
@@ -207,14 +208,44 @@ def bench_c2(steps, warmup):
             "tops": ops / ms / 1e9, "ops": ops}
 
 
+def run_extra(which):
+    """The non-headline BASELINE configurations: 'c4' decode BWTA, 'c3' attention, 'c2' MLP, 'sweep'."""
+    extra = []
+    if which in ("c4", "all"):
+        for N in (1, 4, 16):
+            for sk in (1, 8):
+                extra.append(bench_c4(2000, 200, N, sk))
+                log(json.dumps(extra[-1]))
+    if which in ("c3", "all"):
+        extra.append(bench_c3(200, 20))
+        log(json.dumps(extra[-1]))
+    if which in ("c2", "all"):
+        extra.append(bench_c2(200, 20))
+        log(json.dumps(extra[-1]))
+    if which in ("sweep", "all"):
+        for (K, N) in [(4096, 256), (4096, 2048), (16384, 256), (16384, 2048)]:
+            for sk in (1, 2, 4):
+                r, _ = bench_c5(20, 3, 8192, N, K, sk)
+                extra.append(r)
+                log(json.dumps(r))
+    for r in extra:
+        r["frac_int8_mfma"] = r["tops"] / INT8_MFMA_PEAK_TOPS
+        if "gbs" in r:
+            r["frac_hbm"] = r["gbs"] / HBM_PEAK_GBS
+    return extra
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--all", action="store_true", help="also time the other BASELINE configurations")
+    ap.add_argument("--only", choices=["c2", "c3", "c4", "sweep"], help="time just that configuration (for profiling)")
     ap.add_argument("--variant", type=int, default=0, help="0 auto, 1 VALU, 2 MFMA int8, 3 MFMA fp4")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also run a 256 MiB device-to-device copy (known traffic, for scaling rocprof counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build targets one GPU (its boxes have one); run with --gpus 1")
@@ -225,41 +256,37 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
 
+    if args.calib_copy:
+        src = torch.empty(64 << 20, dtype=torch.int32, device="cuda:0")
+        dst = torch.empty_like(src)
+        ms = time_gpu(lambda i: dst.copy_(src), 2, 5)
+        log("calibration copy: 256 MiB read + 256 MiB written per launch, %.4f ms" % ms)
+    if args.only:
+        print(json.dumps({"configs": run_extra(args.only)}), flush=True)
+        return
+
     c5, (w16, x16) = bench_c5(args.steps, args.warmup, variant=args.variant)
     log("C5:", json.dumps(c5))
     cpu = None if args.no_cpu else cpu_baseline_c5(w16, x16)
     del w16, x16
-    extra = []
-    if args.all:
-        for N in (1, 4, 16):
-            for sk in (1, 8):
-                extra.append(bench_c4(2000, 200, N, sk))
-                log(json.dumps(extra[-1]))
-        extra.append(bench_c3(200, 20))
-        log(json.dumps(extra[-1]))
-        extra.append(bench_c2(200, 20))
-        log(json.dumps(extra[-1]))
-        for (K, N) in [(4096, 256), (4096, 2048), (16384, 256), (16384, 2048)]:
-            for sk in (1, 2, 4):
-                r, _ = bench_c5(20, 3, 8192, N, K, sk)
-                extra.append(r)
-                log(json.dumps(r))
-        for r in extra:
-            r["frac_int8_mfma"] = r["tops"] / INT8_MFMA_PEAK_TOPS
-            if "gbs" in r:
-                r["frac_hbm"] = r["gbs"] / HBM_PEAK_GBS
+    extra = run_extra("all") if args.all else []
+    fp4 = args.variant in (0, 3)
+    peak = FP4_MFMA_PEAK_TOPS if fp4 else INT8_MFMA_PEAK_TOPS
 
     line = {
         "metric": "effective binary TOPS (2*M*N*K/t), bit-exact int32",
         "value": c5["tops"], "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": c5["ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "int8 MFMA on 1-bit operands, int32 accumulate", "data": "synthetic",
+        "dtype": ("fp4 (E2M1) MFMA on 1-bit operands, fp32 accumulate of exact integers" if fp4 else
+                  "int8 MFMA on 1-bit operands, int32 accumulate"),
+        "data": "synthetic",
         "config": {"workload": "BASELINE config 5: BGEMM M=N=K=8192, {-1,+1}x{-1,+1}, weights and activations "
                                "prepacked (tiled bit layout), int32 output, splitK=1",
                    "bit_exact_sampled": c5["bit_exact"], "hbm_gbs_algorithmic": c5["gbs"],
-                   "activation_pack_ms": c5["act_pack_ms"]},
-        "roofline": {"bound": "mfma", "achieved": c5["tops"], "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOP/s",
-                     "frac": c5["tops"] / INT8_MFMA_PEAK_TOPS, "traffic": None},
+                   "activation_pack_ms": c5["act_pack_ms"],
+                   "frac_of_int8_mfma_peak": c5["tops"] / INT8_MFMA_PEAK_TOPS},
+        "roofline": {"bound": "mfma", "achieved": c5["tops"], "peak": peak, "unit": "TOP/s",
+                     "frac": c5["tops"] / peak, "traffic": None},
         "cpu_baseline": cpu,
     }
     if extra:
