@@ -13,8 +13,11 @@
 
 namespace bgemm {
 
+// One all-zero operand tile (never written): K-tiles past a range are read from here.
+__device__ const uint4 g_zero_tile[TILE_U4] = {};
+
 // Block = WGN x WGM waves, each wave owns WN x WM tiles of 32x32 outputs, PL activation planes.
-template <typename Eng, int WGN, int WGM, int WN, int WM, int PL>
+template <typename Eng, int WGN, int WGM, int WN, int WM, int PL, bool PIPE>
 __global__ __launch_bounds__(WGN* WGM * 64) void gemm_mfma_kernel(const GemmArgs a, const int tiles_n,
                                                                    const int tiles_m)
 {
@@ -75,6 +78,69 @@ __global__ __launch_bounds__(WGN* WGM * 64) void gemm_mfma_kernel(const GemmArgs
 #pragma unroll
         for (int i = 0; i < WN; i++) pb[p][i] = 0;
 
+    if constexpr (PIPE) {
+        // ---- main loop, software-pipelined by hand -------------------------------------------------
+        // One MFMA is followed by the two-register slice of the NEXT step's bit expansion (four VALU
+        // ops that fit in the MFMA's shadow); a scheduling barrier after each such group keeps the
+        // compiler from clustering them.  Two raw tile buffers ping-pong: while K-tile kt is consumed
+        // from A, B holds kt+1, and A is refilled with kt+2 during kt's last step.
+        static_assert(PL == 1, "pipelined loop is built for one activation plane");
+        constexpr int NF = WN + WM, ND = NF * 4, NM = WN * WM, STEPS = Eng::STEPS;
+        static_assert(ND % NM == 0 && NF <= NM && STEPS % 2 == 0, "tile shape does not pipeline");
+        constexpr int DPG = ND / NM;                       // expanded registers produced per MFMA
+        const uint4* fp[NF];
+#pragma unroll
+        for (int i = 0; i < WN; i++) fp[i] = xp[0][i];
+#pragma unroll
+        for (int j = 0; j < WM; j++) fp[WN + j] = wp[j];
+        unsigned rawA[NF][4], rawB[NF][4], buf[2][NF][4];
+        int pop[NF];
+#pragma unroll
+        for (int f = 0; f < NF; f++) pop[f] = 0;
+        const int kt_last = kt1 - 1;
+        // K-tiles past the range read as zero bits (which add nothing to the dot or the popcounts),
+        // so the loop can always run whole pairs of K-tiles
+        auto load_frag = [&](unsigned (&r)[4], const int f, const int kt) {
+            const uint4* src = kt <= kt_last ? fp[f] + (int64_t)kt * TILE_U4 : g_zero_tile + lane;
+            const uint4 v = *src;
+            r[0] = v.x; r[1] = v.y; r[2] = v.z; r[3] = v.w;
+        };
+        auto k_tile = [&](unsigned (&A)[NF][4], unsigned (&B)[NF][4], const int kt) {
+#pragma unroll
+            for (int s = 0; s < STEPS; s++) {
+                unsigned (&cur)[NF][4] = buf[s & 1];
+                unsigned (&nxt)[NF][4] = buf[(s + 1) & 1];
+#pragma unroll
+                for (int q = 0; q < NM; q++) {
+                    const int i = q / WM, j = q % WM;
+                    acc[0][i][j] = Eng::mma(Eng::make(cur[i]), Eng::make(cur[WN + j]), acc[0][i][j]);
+#pragma unroll
+                    for (int d = q * DPG; d < (q + 1) * DPG; d++)
+                        nxt[d / 4][d % 4] = s + 1 < STEPS ? Eng::expand1(A[d / 4][d % 4], s + 1)
+                                                          : Eng::expand1(B[d / 4][d % 4], 0);
+                    if (s == 0 && q < NF) pop[q] += __popc(A[q][0]) + __popc(A[q][1]) + __popc(A[q][2]) + __popc(A[q][3]);
+                    if (s == STEPS - 1 && q < NF) load_frag(A[q], q, kt + 2);   // A is dead after step STEPS-2
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        };
+        if (kt0 < kt1) {
+#pragma unroll
+            for (int f = 0; f < NF; f++) { load_frag(rawA[f], f, kt0); load_frag(rawB[f], f, kt0 + 1); }
+#pragma unroll
+            for (int f = 0; f < NF; f++)
+#pragma unroll
+                for (int c = 0; c < 4; c++) buf[0][f][c] = Eng::expand1(rawA[f][c], 0);
+            for (int kt = kt0; kt < kt1; kt += 2) {
+                k_tile(rawA, rawB, kt);
+                k_tile(rawB, rawA, kt + 1);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < WN; i++) pb[0][i] = pop[i];
+#pragma unroll
+        for (int j = 0; j < WM; j++) pa[j] = pop[WN + j];
+    } else {
     // ---- main loop: raw tiles are prefetched one K-tile ahead ----------------------------------
     uint4 xf[PL][WN], wf[WM], xn[PL][WN], wn_[WM];
     if (kt0 < kt1) {
@@ -120,6 +186,8 @@ __global__ __launch_bounds__(WGN* WGM * 64) void gemm_mfma_kernel(const GemmArgs
                     for (int j = 0; j < WM; j++) acc[p][i][j] = Eng::mma(ax, bw[j], acc[p][i][j]);
                 }
         }
+    }
+
     }
 
     // ---- epilogue: rank-one terms turn the AND-dot into this split's share of C ------------
@@ -292,13 +360,13 @@ static int launch_cfg(const GemmArgs& a, hipStream_t st)
     if (a.mc.planes == 2) {
         // two accumulator sets: only the tiles whose registers fit are built for two planes
         if constexpr (WN * WM <= 4)
-            hipLaunchKernelGGL((gemm_mfma_kernel<Eng, WGN, WGM, WN, WM, 2>), dim3((unsigned)grid),
+            hipLaunchKernelGGL((gemm_mfma_kernel<Eng, WGN, WGM, WN, WM, 2, false>), dim3((unsigned)grid),
                                dim3(WGN * WGM * 64), 0, st, a, tiles_n, tiles_m);
         else
             return fail(BGEMM_EINVAL, "gemm_mfma: tile not built for two planes");
     } else
-        hipLaunchKernelGGL((gemm_mfma_kernel<Eng, WGN, WGM, WN, WM, 1>), dim3((unsigned)grid), dim3(WGN * WGM * 64),
-                           0, st, a, tiles_n, tiles_m);
+        hipLaunchKernelGGL((gemm_mfma_kernel<Eng, WGN, WGM, WN, WM, 1, (WN * WM >= 16)>), dim3((unsigned)grid),
+                           dim3(WGN * WGM * 64), 0, st, a, tiles_n, tiles_m);
     return check_launch("gemm_mfma");
 }
 

@@ -22,6 +22,12 @@ struct EngI8 {
         r.z = (w.z >> s) & 0x01010101u; r.w = (w.w >> s) & 0x01010101u;
         return r;
     }
+    __device__ static __forceinline__ unsigned expand1(const unsigned w, const int s) { return (w >> s) & 0x01010101u; }
+    __device__ static __forceinline__ Frag make(const unsigned (&f)[4])
+    {
+        Frag r = {(int)f[0], (int)f[1], (int)f[2], (int)f[3]};
+        return r;
+    }
     __device__ static __forceinline__ Acc mma(const Frag a, const Frag b, const Acc c)
     {
         return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
@@ -44,6 +50,12 @@ struct EngF4 {
     {
         Frag r = {0, 0, 0, 0, 0, 0, 0, 0};
         r[0] = nib(w.x, s); r[1] = nib(w.y, s); r[2] = nib(w.z, s); r[3] = nib(w.w, s);
+        return r;
+    }
+    __device__ static __forceinline__ unsigned expand1(const unsigned w, const int s) { return nib(w, s); }
+    __device__ static __forceinline__ Frag make(const unsigned (&f)[4])
+    {
+        Frag r = {(int)f[0], (int)f[1], (int)f[2], (int)f[3], 0, 0, 0, 0};
         return r;
     }
     __device__ static __forceinline__ Acc mma(const Frag a, const Frag b, const Acc c)
