@@ -335,6 +335,7 @@ static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int splitK, int pla
 {
     const int64_t want = 512;
     auto blocks = [&](int bn, int bm) { return batch * splitK * cdiv(N, bn) * cdiv(M, bm); };
+    if (M <= 64) return blocks(128, 64) >= want ? MfmaCfg{7, 128, 64} : MfmaCfg{6, 64, 64};   // narrow outputs
     if (planes == 1 && blocks(256, 256) >= want) return {0, 256, 256};
     if (blocks(128, 128) >= want) return {1, 128, 128};
     if (blocks(64, 128) >= want || N > 32) return {2, 64, 128};
@@ -380,6 +381,8 @@ static int launch_eng(const GemmArgs& a_in, hipStream_t st)
     case 0: return launch_cfg<Eng, 2, 2, 4, 4>(a, st);    // 256 x 256
     case 4: return launch_cfg<Eng, 2, 2, 4, 2>(a, st);    // 256 x 128, two blocks per CU
     case 5: return launch_cfg<Eng, 2, 2, 2, 4>(a, st);    // 128 x 256, two blocks per CU
+    case 6: return launch_cfg<Eng, 2, 2, 1, 1>(a, st);    // 64 x 64
+    case 7: return launch_cfg<Eng, 2, 2, 2, 1>(a, st);    // 128 x 64
     case 1: return launch_cfg<Eng, 2, 2, 2, 2>(a, st);    // 128 x 128
     case 2: return launch_cfg<Eng, 1, 4, 2, 1>(a, st);    // 64 x 128
     default: return launch_cfg<Eng, 1, 4, 1, 1>(a, st);   // 32 x 128
