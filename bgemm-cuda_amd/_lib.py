@@ -11,7 +11,9 @@ SO_PATH = os.path.join(_HERE, "libbgemm_mi355x.so")
 
 OK, EINVAL, ENULL, EWORKSPACE, ELAUNCH, EALIGN = 0, -1, -2, -3, -4, -5
 MODE_AND, MODE_XOR, MODE_ATTN, MODE_BWTA, MODE_ATTN_X = 0, 1, 2, 3, 4
-OUT_I32, OUT_F16 = 0, 1
+OUT_I32, OUT_F16, OUT_F32_SCALED, OUT_F16_SCALED = 0, 1, 2, 3
+SRC_F16, SRC_F32 = 0, 1
+ABI_VERSION = 3
 VARIANT_AUTO, VARIANT_VALU, VARIANT_MFMA, VARIANT_MFMA_F4 = 0, 1, 2, 3
 
 _i64, _p, _int, _sz = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
@@ -23,6 +25,7 @@ SIGNATURES = {
     "bgemm_tiled_words": (_i64, [_i64, _i64]),
     "bgemm_pack_sign_f16": (_int, [_p, _i64, _i64, _i64, _p, _p]),
     "bgemm_pack_sign_f16_logical": (_int, [_p, _i64, _i64, _i64, _p, _p]),
+    "bgemm_pack_sign_centered": (_int, [_p, _int, _i64, _i64, _i64, _p, _p, _p]),
     "bgemm_pack_ternary_f16": (_int, [_p, _i64, _i64, _i64, _p, _p, _p]),
     "bgemm_tile_from_logical": (_int, [_p, _i64, _i64, _p, _p]),
     "bgemm_logical_from_tiled": (_int, [_p, _i64, _i64, _p, _p]),
@@ -30,6 +33,8 @@ SIGNATURES = {
     "bgemm_packed_counter_bytes": (_sz, [_int, _i64, _i64, _i64, _i64, _int, _int]),
     "bgemm_packed_forward": (_int, [_int, _p, _p, _p, _p, _int, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
                                     _int, _int, _p, _sz, _p, _sz, _p]),
+    "bgemm_packed_forward_scaled": (_int, [_int, _p, _p, _p, _p, _int, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
+                                           _int, _int, _p, _sz, _p, _sz, _p, _p, _p, _p]),
     "bgemm_f16_workspace_bytes": (_sz, [_i64, _i64, _i64, _int]),
     "bgemm_f16_forward": (_int, [_p, _p, _p, _i64, _i64, _i64, _p, _sz, _int, _int, _p]),
 }
@@ -48,6 +53,9 @@ def lib():
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(L, name)
             fn.restype, fn.argtypes = res, args
+        if L.bgemm_abi_version() != ABI_VERSION:
+            raise ImportError("%s is ABI version %d, this binding needs %d: rebuild it" %
+                              (SO_PATH, L.bgemm_abi_version(), ABI_VERSION))
         _lib = L
     return _lib
 

@@ -4,8 +4,10 @@ Host-side mirror of the reference's layer file (tests/python/bgemm_linear.py): t
 class and function names, argument meaning and forward arithmetic, calling
 ``lowbit_kernel.bgemm_linear_forward_cuda`` exactly where the reference does.  Supersets:
 any batch size (the reference asserts ``x.shape[0] % 32 == 0``, bgemm_linear.py:475),
-inputs with leading batch dimensions, non-contiguous operands, and an inference cache of
-the bit-packed weight.
+inputs with leading batch dimensions, non-contiguous operands, and, when no gradient is being
+recorded, a fused forward for BGEMMLinear / BGEMMLinear_bireal: the centred weight is bit-packed
+once and cached, ``x - zpa`` is centred and packed in one pass, and ``* sw * sa (+ bias)`` is
+applied in the GEMM's store, rounded step by step as the separate torch kernels would.
 """
 import math
 
@@ -210,10 +212,34 @@ class _ScaledBinaryLinear(nn.Linear):
 class BGEMMLinear(_ScaledBinaryLinear):
     """out = bgemm(x - zpa, w - zpw) * sw * sa (+ bias)  (bgemm_linear.py:460-486)."""
     _fn = bgemm_linear
+    fuse_inference = True
+
+    def _fusable(self, x):
+        dt = self.weight.dtype
+        return (self.fuse_inference and not torch.is_grad_enabled() and x.is_cuda and dt in (torch.float32, torch.half)
+                and x.dtype == dt and self.sw.dtype == dt and self.sa.dtype == dt
+                and (self.bias is None or self.bias.dtype == dt))
+
+    def _packed_weight(self):
+        key = (self.weight._version, self.weight.data_ptr(), self.weight.dtype)
+        if getattr(self, "_wp_key", None) != key:
+            self._wp = lowbit_kernel.pack_sign(self.weight.detach(), zero_point=self.zpw)
+            self._wp_key = key
+        return self._wp
+
+    def _fused_forward(self, x):
+        lead = x.shape[:-1]
+        xp = lowbit_kernel.pack_sign(x.reshape(-1, x.shape[-1]), zero_point=self.zpa)
+        bias = None if self.bias is None else self.bias.detach()
+        out = lowbit_kernel.bgemm_packed_forward(self._packed_weight(), xp, lowbit_kernel.MODE_XOR,
+                                                 scale=(self.sw.detach(), self.sa.detach().reshape(1), bias))
+        return out.reshape(*lead, self.weight.shape[0])
 
     def forward(self, x):
         if not self.initialized:
             self._initialize(x, self.weight)
+        if self._fusable(x):
+            return self._fused_forward(x)
         out = self._fn.apply(x - self.zpa, self.weight - self.zpw) * self.sw * self.sa
         return self._add_bias(out)
 

@@ -55,7 +55,7 @@ __global__ void clear_counters_kernel(uint32_t* c, int64_t n)
 using namespace bgemm;
 
 extern "C" const char* bgemm_last_error(void) { return g_err; }
-extern "C" int bgemm_abi_version(void) { return 2; }
+extern "C" int bgemm_abi_version(void) { return 3; }
 
 static bool ws_query(int mode, int64_t batch, int64_t M, int64_t N, int64_t K, int splitK, int variant,
                      size_t* part, size_t* counters)
@@ -85,18 +85,30 @@ extern "C" size_t bgemm_packed_counter_bytes(int mode, int64_t batch, int64_t M,
     return round256(cnt * 4);
 }
 
-extern "C" int bgemm_packed_forward(int mode, const void* W_tiled, const void* X_tiled, const void* X2_tiled,
-                                    void* out, int out_dtype, int64_t batch, int64_t M, int64_t N, int64_t K,
-                                    int64_t strideW, int64_t strideX, int64_t strideC,
-                                    int splitK, int variant, void* ws, size_t ws_bytes,
-                                    void* counters, size_t counter_bytes, void* stream)
+// Fills a whole [batch][N][M] output with one value per column: what every mode gives for K = 0
+// (an empty sum), after the output kind's scaling.  A kernel rather than a memset node, so the
+// call can be captured in a HIP graph.
+__global__ void fill_empty_sum_kernel(const GemmArgs a)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= a.N * a.M) return;
+    store_out(a, (int64_t)blockIdx.y * a.strideC + (i / a.M) * a.M, i % a.M, 0);
+}
+
+static int packed_forward(int mode, const void* W_tiled, const void* X_tiled, const void* X2_tiled,
+                          void* out, int out_dtype, int64_t batch, int64_t M, int64_t N, int64_t K,
+                          int64_t strideW, int64_t strideX, int64_t strideC,
+                          int splitK, int variant, void* ws, size_t ws_bytes,
+                          void* counters, size_t counter_bytes,
+                          const void* sw, const void* sa, const void* bias, void* stream)
 {
     g_err[0] = 0;
     GemmArgs a;
     memset(&a, 0, sizeof a);
     if (!mode_coef(mode, &a.mc)) return fail(BGEMM_EINVAL, "bgemm_packed_forward: unknown mode %d", mode);
-    if (out_dtype != BGEMM_OUT_I32 && out_dtype != BGEMM_OUT_F16)
+    if (out_dtype < BGEMM_OUT_I32 || out_dtype > BGEMM_OUT_F16_SCALED)
         return fail(BGEMM_EINVAL, "bgemm_packed_forward: unknown output dtype %d", out_dtype);
+    const bool scaled = out_dtype == BGEMM_OUT_F32_SCALED || out_dtype == BGEMM_OUT_F16_SCALED;
     if (variant < BGEMM_VARIANT_AUTO || variant > BGEMM_VARIANT_MFMA_F4)
         return fail(BGEMM_EINVAL, "bgemm_packed_forward: unknown variant %d", variant);
     if (batch < 0 || M < 0 || N < 0 || K < 0 || splitK < 1 || splitK > 65535)
@@ -110,26 +122,27 @@ extern "C" int bgemm_packed_forward(int mode, const void* W_tiled, const void* X
         return fail(BGEMM_EINVAL, "bgemm_packed_forward: operand strides must be non-negative multiples of 4 words");
     if (batch == 0 || M == 0 || N == 0) return BGEMM_OK;
     if (!out) return fail(BGEMM_ENULL, "bgemm_packed_forward: out is NULL");
+    if (scaled && (!sw || !sa)) return fail(BGEMM_ENULL, "bgemm_packed_forward_scaled: sw or sa is NULL");
+    if (batch > 1 && strideC < M * N)
+        return fail(BGEMM_EINVAL, "bgemm_packed_forward: strideC=%lld smaller than N*M", (long long)strideC);
+    a.out = out; a.out_kind = out_dtype;
+    a.ep_sw = sw; a.ep_sa = sa; a.ep_bias = bias;
+    a.M = M; a.N = N; a.K = K;
+    a.strideC = strideC;
     if (K == 0) {   // empty sum: every mode gives 0
-        const size_t esz = out_dtype == BGEMM_OUT_F16 ? 2 : 4;
-        for (int64_t b = 0; b < batch; b++) {
-            hipError_t e = hipMemsetAsync((char*)out + (size_t)b * strideC * esz, 0, (size_t)N * M * esz, (hipStream_t)stream);
-            if (e != hipSuccess) return fail(BGEMM_ELAUNCH, "bgemm_packed_forward: memset: %s", hipGetErrorString(e));
-        }
-        return BGEMM_OK;
+        if (batch > 65535 || cdiv(N * M, 256) > 0x7fffffffLL) return fail(BGEMM_EINVAL, "bgemm_packed_forward: output too large");
+        hipLaunchKernelGGL(fill_empty_sum_kernel, dim3((unsigned)cdiv(N * M, 256), (unsigned)batch), dim3(256), 0,
+                           (hipStream_t)stream, a);
+        return check_launch("bgemm_packed_forward: fill");
     }
     if (!W_tiled || !X_tiled || (a.mc.planes == 2 && !X2_tiled))
         return fail(BGEMM_ENULL, "bgemm_packed_forward: operand pointer is NULL");
     if (((uintptr_t)W_tiled & 15) || ((uintptr_t)X_tiled & 15) || ((uintptr_t)X2_tiled & 15))
         return fail(BGEMM_EALIGN, "bgemm_packed_forward: operands must be 16-byte aligned");
-    if (batch > 1 && strideC < M * N)
-        return fail(BGEMM_EINVAL, "bgemm_packed_forward: strideC=%lld smaller than N*M", (long long)strideC);
 
     a.W = (const uint4*)W_tiled; a.X = (const uint4*)X_tiled; a.X2 = (const uint4*)X2_tiled;
-    a.out = out; a.out_f16 = out_dtype == BGEMM_OUT_F16;
-    a.M = M; a.N = N; a.K = K;
     a.MT = (int)row_tiles(M); a.NT = (int)row_tiles(N); a.KT = (int)k_tiles(K);
-    a.strideW = strideW / 4; a.strideX = strideX / 4; a.strideC = strideC;
+    a.strideW = strideW / 4; a.strideX = strideX / 4;
     a.batch = (int)batch; a.splitK = splitK;
     a.vec_store = (M % 4 == 0) && (strideC % 4 == 0) && (((uintptr_t)out & 15) == 0);
     const int v = variant == BGEMM_VARIANT_AUTO ? pick_variant(mode, batch, M, N, K) : variant;
@@ -151,6 +164,32 @@ extern "C" int bgemm_packed_forward(int mode, const void* W_tiled, const void* X
     if (v == BGEMM_VARIANT_VALU) return launch_gemm_valu(a, (hipStream_t)stream);
     if (skinny) return launch_gemm_skinny(a, (hipStream_t)stream, v == BGEMM_VARIANT_MFMA_F4);
     return launch_gemm_mfma(a, (hipStream_t)stream, v == BGEMM_VARIANT_MFMA_F4);
+}
+
+extern "C" int bgemm_packed_forward(int mode, const void* W_tiled, const void* X_tiled, const void* X2_tiled,
+                                    void* out, int out_dtype, int64_t batch, int64_t M, int64_t N, int64_t K,
+                                    int64_t strideW, int64_t strideX, int64_t strideC,
+                                    int splitK, int variant, void* ws, size_t ws_bytes,
+                                    void* counters, size_t counter_bytes, void* stream)
+{
+    if (out_dtype != BGEMM_OUT_I32 && out_dtype != BGEMM_OUT_F16)
+        return fail(BGEMM_EINVAL, "bgemm_packed_forward: unknown output dtype %d", out_dtype);
+    return packed_forward(mode, W_tiled, X_tiled, X2_tiled, out, out_dtype, batch, M, N, K, strideW, strideX, strideC,
+                          splitK, variant, ws, ws_bytes, counters, counter_bytes, nullptr, nullptr, nullptr, stream);
+}
+
+extern "C" int bgemm_packed_forward_scaled(int mode, const void* W_tiled, const void* X_tiled, const void* X2_tiled,
+                                           void* out, int out_dtype, int64_t batch, int64_t M, int64_t N, int64_t K,
+                                           int64_t strideW, int64_t strideX, int64_t strideC,
+                                           int splitK, int variant, void* ws, size_t ws_bytes,
+                                           void* counters, size_t counter_bytes,
+                                           const void* sw, const void* sa, const void* bias, void* stream)
+{
+    if (out_dtype != BGEMM_OUT_F32_SCALED && out_dtype != BGEMM_OUT_F16_SCALED)
+        return fail(BGEMM_EINVAL, "bgemm_packed_forward_scaled: output dtype must be BGEMM_OUT_F32_SCALED or "
+                                  "BGEMM_OUT_F16_SCALED, got %d", out_dtype);
+    return packed_forward(mode, W_tiled, X_tiled, X2_tiled, out, out_dtype, batch, M, N, K, strideW, strideX, strideC,
+                          splitK, variant, ws, ws_bytes, counters, counter_bytes, sw, sa, bias, stream);
 }
 
 // ---- fp16-operand call: pack both operands into the workspace, then the packed GEMM ----
@@ -196,9 +235,7 @@ extern "C" int bgemm_f16_forward(const void* W, const void* X, void* C, int64_t 
         int rc = check_launch("bgemm_f16_forward: clear counters");
         if (rc) return rc;
     }
-    int rc = bgemm_pack_sign_f16(W, M, K, K, wt, stream);
-    if (rc) return rc;
-    rc = bgemm_pack_sign_f16(X, N, K, K, xt, stream);
+    int rc = pack_sign_pair(W, M, wt, X, N, xt, K, (hipStream_t)stream, "bgemm_f16_forward: pack");
     if (rc) return rc;
     return bgemm_packed_forward(INSTR, wt, xt, nullptr, C, BGEMM_OUT_F16, 1, M, N, K, 0, 0, 0, splitK,
                                 BGEMM_VARIANT_AUTO, part, pb, cnt, cb, stream);

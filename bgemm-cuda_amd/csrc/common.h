@@ -44,7 +44,8 @@ static inline bool mode_coef(int mode, ModeCoef* mc)
 
 struct GemmArgs {
     const uint4* W; const uint4* X; const uint4* X2;
-    void* out; int out_f16;
+    void* out; int out_kind;       // BGEMM_OUT_*
+    const void* ep_sw; const void* ep_sa; const void* ep_bias;   // scaled output kinds: per-column scale, scalar, bias
     int vec_store;        // rows of `out` are 16-byte aligned: the epilogue may store four elements per lane
     int64_t M, N, K;
     int MT, NT, KT;
@@ -127,13 +128,50 @@ static inline int effective_split(int64_t tiles, int splitK, int KT)
     return s;
 }
 
-// Final store of one output element: int32 as is, or fp16 = the integer rounded to nearest
-// even (exact through fp32 because |v| < 2^24).
-__device__ __forceinline__ void store_out(void* out, int out_f16, int64_t idx, int v)
+// Output kinds: the int32 accumulator itself; fp16 = the integer rounded to nearest even (exact
+// through fp32 because |v| < 2^24); or the binary Linear's scaling fused in, op for op as torch
+// evaluates `half(acc) * sw * sa (+ bias)` (tests/python/bgemm_linear.py:482-484): with fp32
+// parameters every step is an fp32 op, with fp16 parameters every step rounds to fp16.  No step
+// may be contracted into an FMA.
+__device__ __forceinline__ float scaled_f32(const GemmArgs& a, const int64_t m, const int v)
 {
-    if (out_f16) reinterpret_cast<__half*>(out)[idx] = __float2half_rn((float)v);
-    else reinterpret_cast<int*>(out)[idx] = v;
+    float r = __fmul_rn(__half2float(__float2half_rn((float)v)), reinterpret_cast<const float*>(a.ep_sw)[m]);
+    r = __fmul_rn(r, *reinterpret_cast<const float*>(a.ep_sa));
+    if (a.ep_bias) r = __fadd_rn(r, reinterpret_cast<const float*>(a.ep_bias)[m]);
+    return r;
 }
+__device__ __forceinline__ __half scaled_f16(const GemmArgs& a, const int64_t m, const int v)
+{
+    __half r = __float2half_rn((float)v);
+    r = __float2half_rn(__fmul_rn(__half2float(r), __half2float(reinterpret_cast<const __half*>(a.ep_sw)[m])));
+    r = __float2half_rn(__fmul_rn(__half2float(r), __half2float(*reinterpret_cast<const __half*>(a.ep_sa))));
+    if (a.ep_bias) r = __float2half_rn(__fadd_rn(__half2float(r), __half2float(reinterpret_cast<const __half*>(a.ep_bias)[m])));
+    return r;
+}
+__device__ __forceinline__ int out_elem_shift(const int kind) { return (kind == BGEMM_OUT_F16 || kind == BGEMM_OUT_F16_SCALED) ? 1 : 2; }
+
+// Final store of one output element (column m of a row whose first element has index row0).
+template <int KIND>
+__device__ __forceinline__ void store_out_as(const GemmArgs& a, const int64_t row0, const int64_t m, const int v)
+{
+    if constexpr (KIND == BGEMM_OUT_I32) reinterpret_cast<int*>(a.out)[row0 + m] = v;
+    else if constexpr (KIND == BGEMM_OUT_F16) reinterpret_cast<__half*>(a.out)[row0 + m] = __float2half_rn((float)v);
+    else if constexpr (KIND == BGEMM_OUT_F32_SCALED) reinterpret_cast<float*>(a.out)[row0 + m] = scaled_f32(a, m, v);
+    else reinterpret_cast<__half*>(a.out)[row0 + m] = scaled_f16(a, m, v);
+}
+__device__ __forceinline__ void store_out(const GemmArgs& a, const int64_t row0, const int64_t m, const int v)
+{
+    switch (a.out_kind) {
+    case BGEMM_OUT_I32: store_out_as<BGEMM_OUT_I32>(a, row0, m, v); break;
+    case BGEMM_OUT_F16: store_out_as<BGEMM_OUT_F16>(a, row0, m, v); break;
+    case BGEMM_OUT_F32_SCALED: store_out_as<BGEMM_OUT_F32_SCALED>(a, row0, m, v); break;
+    default: store_out_as<BGEMM_OUT_F16_SCALED>(a, row0, m, v); break;
+    }
+}
+
+// Sign-packs two fp16 [rows][K] operands (row stride K) into tiled buffers with one launch.
+int pack_sign_pair(const void* srcA, int64_t rowsA, void* dstA, const void* srcB, int64_t rowsB, void* dstB,
+                   int64_t K, hipStream_t st, const char* who);
 
 // Kernel families (each in its own translation unit).
 int launch_gemm_mfma(const GemmArgs& a, hipStream_t st, bool fp4);

@@ -249,20 +249,18 @@ __global__ __launch_bounds__(WGN* WGM * 64) void gemm_mfma_kernel(const GemmArgs
     }
 
     // ---- store ------------------------------------------------------------------------------
+    // Every 32-row strip of the wave's tile is transposed through LDS, so that lanes own consecutive
+    // outputs of one row.  Only the plain int32 case with 16-byte-aligned rows is unrolled; the
+    // conversions of the other output kinds sit in rolled loops after the staging, which keeps them
+    // out of the fully unrolled part of the kernel.
     constexpr int ROW_I = WM * 32 + 8;       // staged row stride in ints (+8 keeps the two lane halves on
                                              // different LDS banks)
     __shared__ __align__(16) int stage[WGN * WGM * 32 * ROW_I];
-    const int esz_shift = a.out_f16 ? 1 : 2;
-    char* const out_base = reinterpret_cast<char*>(a.out) + (((int64_t)b * a.strideC) << esz_shift);
+    const int esz_shift = out_elem_shift(a.out_kind);
+    const int64_t out_off = (int64_t)b * a.strideC;
+    char* const out_base = reinterpret_cast<char*>(a.out) + (out_off << esz_shift);
     const int64_t row_bytes = a.M << esz_shift;
-    int coff[WM];
-    bool cok[WM];
-#pragma unroll
-    for (int j = 0; j < WM; j++) {
-        const int64_t m = (int64_t)(mt0 + j) * 32 + col;
-        cok[j] = m < a.M;
-        coff[j] = (int)(cok[j] ? m : 0) << esz_shift;
-    }
+    int* const st = stage + wave * (32 * ROW_I);
 #pragma unroll
     for (int i = 0; i < WN; i++) {
         int val[WM][16];
@@ -281,49 +279,60 @@ __global__ __launch_bounds__(WGN* WGM * 64) void gemm_mfma_kernel(const GemmArgs
                     }
             }
         }
-        if (a.vec_store) {
-            // transpose through LDS so that every lane owns four consecutive outputs of one row:
-            // 16-byte stores, one instruction covers 64 * 4 consecutive elements of the tile row
-            int* st = stage + wave * (32 * ROW_I);
 #pragma unroll
-            for (int v = 0; v < 16; v++)
+        for (int v = 0; v < 16; v++)
 #pragma unroll
-                for (int j = 0; j < WM; j++) st[(8 * (v >> 2) + 4 * half + (v & 3)) * ROW_I + j * 32 + col] = val[j][v];
-            __syncthreads();
-            constexpr int C4 = WM * 8;               // int4 per staged row
+            for (int j = 0; j < WM; j++) st[(8 * (v >> 2) + 4 * half + (v & 3)) * ROW_I + j * 32 + col] = val[j][v];
+        __syncthreads();
+        const int64_t nrow0 = (int64_t)(nt0 + i) * 32, mcol0 = (int64_t)mt0 * 32;
+        constexpr int C4 = WM * 8;               // int4 per staged row
+        constexpr int NP = 32 * C4 / 64;
+        if (a.vec_store && a.out_kind == BGEMM_OUT_I32) {
+            // 16-byte stores: one instruction covers 64 * 4 consecutive elements of the strip
 #pragma unroll
-            for (int p = 0; p < 32 * C4 / 64; p++) {
+            for (int p = 0; p < NP; p++) {
                 const int idx = p * 64 + lane, row = idx / C4, c4 = idx % C4;
                 const int4 q = *reinterpret_cast<const int4*>(st + row * ROW_I + c4 * 4);
-                const int64_t n = (int64_t)(nt0 + i) * 32 + row, m = (int64_t)mt0 * 32 + c4 * 4;
+                const int64_t n = nrow0 + row, m = mcol0 + c4 * 4;
+                if (n < a.N && m < a.M) *reinterpret_cast<int4*>(out_base + n * row_bytes + (m << 2)) = q;
+            }
+        } else if (a.vec_store) {
+#pragma unroll 4
+            for (int p = 0; p < NP; p++) {
+                const int idx = p * 64 + lane, row = idx / C4, c4 = idx % C4;
+                const int4 q = *reinterpret_cast<const int4*>(st + row * ROW_I + c4 * 4);
+                const int64_t n = nrow0 + row, m = mcol0 + c4 * 4;
                 if (n < a.N && m < a.M) {
                     char* const dst = out_base + n * row_bytes + (m << esz_shift);
-                    if (a.out_f16) {
-                        union { __half h[4]; uint2 u; } pk;
+                    union { __half h[4]; uint2 u; } pk;
+                    switch (a.out_kind) {
+                    case BGEMM_OUT_F16:
                         pk.h[0] = __float2half_rn((float)q.x); pk.h[1] = __float2half_rn((float)q.y);
                         pk.h[2] = __float2half_rn((float)q.z); pk.h[3] = __float2half_rn((float)q.w);
                         *reinterpret_cast<uint2*>(dst) = pk.u;
-                    } else
-                        *reinterpret_cast<int4*>(dst) = q;
+                        break;
+                    case BGEMM_OUT_F32_SCALED:
+                        *reinterpret_cast<float4*>(dst) = make_float4(scaled_f32(a, m, q.x), scaled_f32(a, m + 1, q.y),
+                                                                      scaled_f32(a, m + 2, q.z), scaled_f32(a, m + 3, q.w));
+                        break;
+                    default:
+                        pk.h[0] = scaled_f16(a, m, q.x); pk.h[1] = scaled_f16(a, m + 1, q.y);
+                        pk.h[2] = scaled_f16(a, m + 2, q.z); pk.h[3] = scaled_f16(a, m + 3, q.w);
+                        *reinterpret_cast<uint2*>(dst) = pk.u;
+                        break;
+                    }
                 }
             }
-            __syncthreads();
-            continue;
-        }
-        const int64_t n0 = (int64_t)(nt0 + i) * 32 + 4 * half;
-        char* const tile_row0 = out_base + n0 * row_bytes;
-#pragma unroll
-        for (int v = 0; v < 16; v++) {
-            const int dn = 8 * (v >> 2) + (v & 3);
-            if (n0 + dn >= a.N) continue;
-            char* const rowp = tile_row0 + dn * row_bytes;
-#pragma unroll
-            for (int j = 0; j < WM; j++) {
-                if (!cok[j]) continue;
-                if (a.out_f16) *reinterpret_cast<__half*>(rowp + coff[j]) = __float2half_rn((float)val[j][v]);
-                else *reinterpret_cast<int*>(rowp + coff[j]) = val[j][v];
+        } else {
+            // ragged or unaligned rows: one element per lane and step
+#pragma unroll 4
+            for (int p = 0; p < 16 * WM; p++) {
+                const int idx = p * 64 + lane, row = idx / (32 * WM), c = idx % (32 * WM);
+                const int64_t n = nrow0 + row, m = mcol0 + c;
+                if (n < a.N && m < a.M) store_out(a, out_off + n * a.M, m, st[row * ROW_I + c]);
             }
         }
+        __syncthreads();
     }
 }
 

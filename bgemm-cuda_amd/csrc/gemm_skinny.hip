@@ -108,7 +108,7 @@ __global__ __launch_bounds__(KW * 64) void gemm_skinny_kernel(const GemmArgs a, 
         const int64_t m = ((int64_t)grp * RT + t) * 32 + r;
         int val = __mul24(mc.c0, kbits) + __mul24(mc.ca, sPa[t][r]) + __mul24(mc.cb, sPb[n]) + __mul24(mc.cd, d);
         if (two) val += __mul24(mc.cb2, sPb[n + 16]) + __mul24(mc.cd2, d2);
-        if (n < a.N && m < a.M) store_out(a.out, a.out_f16, (int64_t)b * a.strideC + (int64_t)n * a.M + m, val);
+        if (n < a.N && m < a.M) store_out(a, (int64_t)b * a.strideC + (int64_t)n * a.M, m, val);
     }
 }
 

@@ -141,7 +141,7 @@ __global__ __launch_bounds__(256) void gemm_valu_kernel(const GemmArgs a, const 
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const int64_t m = (int64_t)tm * 64 + tx + 16 * j;
-            if (n < a.N && m < a.M) store_out(a.out, a.out_f16, out_off + n * a.M + m, val[i][j]);
+            if (n < a.N && m < a.M) store_out(a, out_off + n * a.M, m, val[i][j]);
         }
     }
 }

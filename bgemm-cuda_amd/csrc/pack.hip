@@ -2,6 +2,7 @@
 // one 16-byte load per lane, eight sign (and nonzero) bits extracted per lane, four
 // lanes merged into a 32-bit word, 16-byte-contiguous stores into the tiled layout.
 #include "common.h"
+#include <string.h>
 
 namespace bgemm {
 
@@ -12,32 +13,61 @@ __host__ __device__ static inline int64_t tiled_word_offset(int64_t row, int64_t
     return ((rt * KT + kt) * TILE_U4 + h * 32 + r) * 4 + q;
 }
 
-// One wave packs 512 consecutive K elements of one row (16 words).
-// mode bit0: also write the (sign & nonzero) plane and make plane 0 the nonzero plane.
-// mode bit1: write the logical layout instead of the tiled one.
-__global__ __launch_bounds__(256) void pack_f16_kernel(
-    const uint16_t* __restrict__ src, int64_t rows, int64_t K, int64_t ld,
-    uint32_t* __restrict__ dst0, uint32_t* __restrict__ dst1, int mode,
-    int64_t rows_out, int64_t nseg, int64_t KT, int64_t Kw)
+// One operand to pack.  mode bit0: also write the (sign & nonzero) plane and make plane 0 the
+// nonzero plane.  mode bit1: write the logical layout instead of the tiled one.  mode bit2: the
+// source is fp32 (rounded to fp16 first, as the layers' `.to(torch.half)` does).
+// zp: device scalar of the source type subtracted before that rounding, or null.
+struct PackJob {
+    const void* src; int64_t rows, K, ld;
+    uint32_t* dst0; uint32_t* dst1; int mode;
+    const void* zp;
+    int64_t rows_out, nseg, KT, Kw, waves;
+};
+
+__device__ __forceinline__ uint16_t half_bits(const float f)
 {
-    const int lane = threadIdx.x & 63;
-    const int64_t gw = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    const int64_t row = gw / nseg, seg = gw - row * nseg;
-    if (row >= rows_out) return;          // whole wave leaves together
+    return __half_as_ushort(__float2half_rn(f));
+}
+
+// One wave packs 512 consecutive K elements of one row (16 words).
+__device__ __forceinline__ void pack_wave(const PackJob& j, const int64_t gw, const int lane)
+{
+    const int64_t row = gw / j.nseg, seg = gw - row * j.nseg;
+    if (row >= j.rows_out) return;        // whole wave leaves together
     const int64_t k0 = seg * 512 + 8 * lane;
 
-    uint16_t h[8];
+    uint16_t h[8];                        // fp16 bit patterns; elements past K stay +0.0
 #pragma unroll
     for (int e = 0; e < 8; e++) h[e] = 0;
-    if (row < rows && k0 < K) {
-        const uint16_t* p = src + row * ld + k0;
-        if (k0 + 8 <= K && (((uintptr_t)p) & 15) == 0) {
-            const uint4 v = *reinterpret_cast<const uint4*>(p);
-            h[0] = v.x & 0xffff; h[1] = v.x >> 16; h[2] = v.y & 0xffff; h[3] = v.y >> 16;
-            h[4] = v.z & 0xffff; h[5] = v.z >> 16; h[6] = v.w & 0xffff; h[7] = v.w >> 16;
-        } else {
+    if (row < j.rows && k0 < j.K) {
+        if (j.mode & 4) {
+            const float* p = reinterpret_cast<const float*>(j.src) + row * j.ld + k0;
+            const float z = j.zp ? *reinterpret_cast<const float*>(j.zp) : 0.f;
+            if (k0 + 8 <= j.K && (((uintptr_t)p) & 15) == 0) {
+                const float4 u = *reinterpret_cast<const float4*>(p), v = *reinterpret_cast<const float4*>(p + 4);
+                const float f[8] = {u.x, u.y, u.z, u.w, v.x, v.y, v.z, v.w};
 #pragma unroll
-            for (int e = 0; e < 8; e++) if (k0 + e < K) h[e] = p[e];
+                for (int e = 0; e < 8; e++) h[e] = half_bits(j.zp ? __fsub_rn(f[e], z) : f[e]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; e++) if (k0 + e < j.K) h[e] = half_bits(j.zp ? __fsub_rn(p[e], z) : p[e]);
+            }
+        } else {
+            const uint16_t* p = reinterpret_cast<const uint16_t*>(j.src) + row * j.ld + k0;
+            if (k0 + 8 <= j.K && (((uintptr_t)p) & 15) == 0) {
+                const uint4 v = *reinterpret_cast<const uint4*>(p);
+                h[0] = v.x & 0xffff; h[1] = v.x >> 16; h[2] = v.y & 0xffff; h[3] = v.y >> 16;
+                h[4] = v.z & 0xffff; h[5] = v.z >> 16; h[6] = v.w & 0xffff; h[7] = v.w >> 16;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; e++) if (k0 + e < j.K) h[e] = p[e];
+            }
+            if (j.zp) {
+                const float z = __half2float(*reinterpret_cast<const __half*>(j.zp));
+#pragma unroll
+                for (int e = 0; e < 8; e++)
+                    if (k0 + e < j.K) h[e] = half_bits(__fsub_rn(__half2float(__ushort_as_half(h[e])), z));
+            }
         }
     }
     uint32_t sg = 0, nz = 0;
@@ -46,7 +76,7 @@ __global__ __launch_bounds__(256) void pack_f16_kernel(
         sg |= (uint32_t)(h[e] >> 15) << (7 - e);
         nz |= (uint32_t)((h[e] & 0x7fff) != 0) << (7 - e);
     }
-    const bool ternary = mode & 1;
+    const bool ternary = j.mode & 1;
     uint32_t p0 = ternary ? nz : sg, p1 = sg & nz;
     const int sh = 8 * (3 - (lane & 3));
     p0 <<= sh; p1 <<= sh;
@@ -54,13 +84,22 @@ __global__ __launch_bounds__(256) void pack_f16_kernel(
     if (ternary) { p1 |= __shfl_xor(p1, 1); p1 |= __shfl_xor(p1, 2); }
     if (lane & 3) return;
     const int64_t jw = seg * 16 + (lane >> 2);
-    if (mode & 2) {
-        if (row < rows && jw < Kw) { dst0[row * Kw + jw] = p0; if (ternary) dst1[row * Kw + jw] = p1; }
-    } else if (jw < KT * 8) {
-        const int64_t o = tiled_word_offset(row, jw, KT);
-        dst0[o] = p0;
-        if (ternary) dst1[o] = p1;
+    if (j.mode & 2) {
+        if (row < j.rows && jw < j.Kw) { j.dst0[row * j.Kw + jw] = p0; if (ternary) j.dst1[row * j.Kw + jw] = p1; }
+    } else if (jw < j.KT * 8) {
+        const int64_t o = tiled_word_offset(row, jw, j.KT);
+        j.dst0[o] = p0;
+        if (ternary) j.dst1[o] = p1;
     }
+}
+
+// Up to two operands per launch (the fp16 entry point packs weights and activations together).
+__global__ __launch_bounds__(256) void pack_f16_kernel(const PackJob j0, const PackJob j1)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t gw = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (gw < j0.waves) pack_wave(j0, gw, lane);
+    else if (gw - j0.waves < j1.waves) pack_wave(j1, gw - j0.waves, lane);
 }
 
 // dir 0: logical -> tiled (zero padding), dir 1: tiled -> logical.  One thread per tiled word.
@@ -79,23 +118,50 @@ __global__ __launch_bounds__(256) void relayout_kernel(
     else if (real) dst[row * Kw + jw] = src[i];
 }
 
-static int pack_common(const void* src, int64_t rows, int64_t K, int64_t ld, void* d0, void* d1,
-                       int mode, hipStream_t st, const char* who)
+static int make_job(PackJob* j, const void* src, int64_t rows, int64_t K, int64_t ld, void* d0, void* d1, int mode,
+                    const void* zp, const char* who)
 {
     if (rows < 0 || K < 0 || ld < K) return fail(BGEMM_EINVAL, "%s: bad shape rows=%lld K=%lld ld=%lld", who,
                                                  (long long)rows, (long long)K, (long long)ld);
+    memset(j, 0, sizeof *j);
     if (rows == 0 || K == 0) return BGEMM_OK;
     if (!src || !d0 || ((mode & 1) && !d1)) return fail(BGEMM_ENULL, "%s: null pointer", who);
     if (((uintptr_t)d0 & 15) || ((uintptr_t)d1 & 15)) return fail(BGEMM_EALIGN, "%s: destination not 16-byte aligned", who);
-    const int64_t KT = k_tiles(K), Kw = cdiv(K, 32);
-    const int64_t rows_out = (mode & 2) ? rows : row_tiles(rows) * TILE_ROWS;
-    const int64_t nseg = cdiv(KT * TILE_KBITS, 512);
-    const int64_t waves = rows_out * nseg, blocks = cdiv(waves, 4);
+    j->src = src; j->zp = zp; j->rows = rows; j->K = K; j->ld = ld;
+    j->dst0 = (uint32_t*)d0; j->dst1 = (uint32_t*)d1; j->mode = mode;
+    j->KT = k_tiles(K); j->Kw = cdiv(K, 32);
+    j->rows_out = (mode & 2) ? rows : row_tiles(rows) * TILE_ROWS;
+    j->nseg = cdiv(j->KT * TILE_KBITS, 512);
+    j->waves = j->rows_out * j->nseg;
+    return BGEMM_OK;
+}
+
+static int launch_jobs(const PackJob& j0, const PackJob& j1, hipStream_t st, const char* who)
+{
+    const int64_t blocks = cdiv(j0.waves + j1.waves, 4);
+    if (blocks == 0) return BGEMM_OK;
     if (blocks > 0x7fffffffLL) return fail(BGEMM_EINVAL, "%s: operand too large", who);
-    hipLaunchKernelGGL(pack_f16_kernel, dim3((unsigned)blocks), dim3(256), 0, st,
-                       (const uint16_t*)src, rows, K, ld, (uint32_t*)d0, (uint32_t*)d1, mode,
-                       rows_out, nseg, KT, Kw);
+    hipLaunchKernelGGL(pack_f16_kernel, dim3((unsigned)blocks), dim3(256), 0, st, j0, j1);
     return check_launch(who);
+}
+
+static int pack_common(const void* src, int64_t rows, int64_t K, int64_t ld, void* d0, void* d1,
+                       int mode, const void* zp, hipStream_t st, const char* who)
+{
+    PackJob j0, j1;
+    memset(&j1, 0, sizeof j1);
+    const int rc = make_job(&j0, src, rows, K, ld, d0, d1, mode, zp, who);
+    return rc ? rc : launch_jobs(j0, j1, st, who);
+}
+
+// Sign-packs two fp16 operands into their tiled buffers with one launch.
+int pack_sign_pair(const void* srcA, int64_t rowsA, void* dstA, const void* srcB, int64_t rowsB, void* dstB,
+                   int64_t K, hipStream_t st, const char* who)
+{
+    PackJob j0, j1;
+    int rc = make_job(&j0, srcA, rowsA, K, K, dstA, nullptr, 0, nullptr, who);
+    if (!rc) rc = make_job(&j1, srcB, rowsB, K, K, dstB, nullptr, 0, nullptr, who);
+    return rc ? rc : launch_jobs(j0, j1, st, who);
 }
 
 }  // namespace bgemm
@@ -111,19 +177,28 @@ extern "C" int64_t bgemm_tiled_words(int64_t rows, int64_t K)
 extern "C" int bgemm_pack_sign_f16(const void* src, int64_t rows, int64_t K, int64_t ld,
                                    void* dst_tiled, void* stream)
 {
-    return pack_common(src, rows, K, ld, dst_tiled, nullptr, 0, (hipStream_t)stream, "bgemm_pack_sign_f16");
+    return pack_common(src, rows, K, ld, dst_tiled, nullptr, 0, nullptr, (hipStream_t)stream, "bgemm_pack_sign_f16");
 }
 
 extern "C" int bgemm_pack_sign_f16_logical(const void* src, int64_t rows, int64_t K, int64_t ld,
                                            uint32_t* dst_logical, void* stream)
 {
-    return pack_common(src, rows, K, ld, dst_logical, nullptr, 2, (hipStream_t)stream, "bgemm_pack_sign_f16_logical");
+    return pack_common(src, rows, K, ld, dst_logical, nullptr, 2, nullptr, (hipStream_t)stream, "bgemm_pack_sign_f16_logical");
 }
 
 extern "C" int bgemm_pack_ternary_f16(const void* src, int64_t rows, int64_t K, int64_t ld,
                                       void* nz_tiled, void* sg_tiled, void* stream)
 {
-    return pack_common(src, rows, K, ld, nz_tiled, sg_tiled, 1, (hipStream_t)stream, "bgemm_pack_ternary_f16");
+    return pack_common(src, rows, K, ld, nz_tiled, sg_tiled, 1, nullptr, (hipStream_t)stream, "bgemm_pack_ternary_f16");
+}
+
+extern "C" int bgemm_pack_sign_centered(const void* src, int src_dtype, int64_t rows, int64_t K, int64_t ld,
+                                        const void* zero_point, void* dst_tiled, void* stream)
+{
+    if (src_dtype != BGEMM_SRC_F16 && src_dtype != BGEMM_SRC_F32)
+        return fail(BGEMM_EINVAL, "bgemm_pack_sign_centered: unknown source type %d", src_dtype);
+    return pack_common(src, rows, K, ld, dst_tiled, nullptr, src_dtype == BGEMM_SRC_F32 ? 4 : 0, zero_point,
+                       (hipStream_t)stream, "bgemm_pack_sign_centered");
 }
 
 static int relayout(const void* src, void* dst, int64_t rows, int64_t K, int dir, void* stream, const char* who)

@@ -12,8 +12,8 @@ include/bgemm_mi355x.h; torch supplies device memory and streams only.
 import torch
 
 import _lib as _b
-from _lib import (MODE_AND, MODE_XOR, MODE_ATTN, MODE_BWTA, MODE_ATTN_X, OUT_I32, OUT_F16,
-                  VARIANT_AUTO, VARIANT_VALU, VARIANT_MFMA, VARIANT_MFMA_F4)
+from _lib import (MODE_AND, MODE_XOR, MODE_ATTN, MODE_BWTA, MODE_ATTN_X, OUT_I32, OUT_F16, OUT_F32_SCALED,
+                  OUT_F16_SCALED, SRC_F16, SRC_F32, VARIANT_AUTO, VARIANT_VALU, VARIANT_MFMA, VARIANT_MFMA_F4)
 
 AND_POP, XOR_POP, ATTN_MM = 0, 1, 2   # lowbit_kernel/csrc/include/configs.h:70-72
 
@@ -74,11 +74,22 @@ class PackedBits:
         return self.data.numel() * 4 * (2 if self.ternary else 1)
 
 
-def _pack(x, ternary):
+def _pack(x, ternary, zero_point=None):
     _need_cuda(x, "input")
     if x.dim() not in (2, 3):
         raise ValueError("expected a 2-D or 3-D tensor, got %d-D" % x.dim())
-    x = x.to(torch.half).contiguous()
+    if zero_point is not None:
+        if ternary:
+            raise ValueError("a zero point is only taken by the sign pack")
+        if x.dtype not in (torch.half, torch.float32):
+            raise TypeError("centred packing reads fp16 or fp32 sources, got %s" % x.dtype)
+        if not isinstance(zero_point, torch.Tensor) or zero_point.numel() != 1:
+            raise TypeError("zero_point must be a one-element tensor")
+        _need_cuda(zero_point, "zero_point")
+        zero_point = zero_point.detach().to(x.dtype)
+        x = x.contiguous()
+    else:
+        x = x.to(torch.half).contiguous()
     batch = 1 if x.dim() == 2 else x.shape[0]
     rows, K = x.shape[-2], x.shape[-1]
     L = _b.lib()
@@ -96,14 +107,21 @@ def _pack(x, ternary):
         for src, r, p0, p1 in groups:
             if ternary:
                 _b.check(L.bgemm_pack_ternary_f16(src, r, K, K, p0, p1, st))
+            elif zero_point is not None:
+                _b.check(L.bgemm_pack_sign_centered(src, SRC_F32 if x.dtype == torch.float32 else SRC_F16, r, K, K,
+                                                    zero_point.data_ptr(), p0, st))
             else:
                 _b.check(L.bgemm_pack_sign_f16(src, r, K, K, p0, st))
     return PackedBits(d0, d1, batch, rows, K)
 
 
-def pack_sign(x):
-    """fp16 (or castable) ``[R,K]`` / ``[B,R,K]`` -> tiled sign bits (bit = 1 for negative, -0.0 included)."""
-    return _pack(x, False)
+def pack_sign(x, zero_point=None):
+    """fp16 (or castable) ``[R,K]`` / ``[B,R,K]`` -> tiled sign bits (bit = 1 for negative, -0.0 included).
+
+    With ``zero_point`` (a one-element device tensor) the bits are those of
+    ``(x - zero_point).to(torch.half)`` for an fp16 or fp32 ``x``, computed in the same pass: the
+    operand the binary Linear layers feed the kernel (bgemm_linear.py:479-482)."""
+    return _pack(x, False, zero_point)
 
 
 def pack_ternary(x):
@@ -147,9 +165,14 @@ def logical_from_tiled(packed, plane=0):
     return out
 
 
-def bgemm_packed_forward(w, x, mode=MODE_XOR, out_dtype=torch.int32, splitK=1, variant=VARIANT_AUTO, out=None):
+def bgemm_packed_forward(w, x, mode=MODE_XOR, out_dtype=torch.int32, splitK=1, variant=VARIANT_AUTO, out=None,
+                         scale=None):
     """GEMM on packed operands: ``out[b,n,m]`` for weight-side ``w`` (M rows) and activation-side
-    ``x`` (N rows).  A batch of 1 on either side is shared across the other side's batch."""
+    ``x`` (N rows).  A batch of 1 on either side is shared across the other side's batch.
+
+    ``scale=(sw, sa, bias)`` fuses the binary Linear's ``half(acc) * sw * sa (+ bias)``
+    (bgemm_linear.py:482-484) into the store: ``sw`` [M], ``sa`` one element, ``bias`` [M] or None,
+    all fp32 (fp32 output) or all fp16 (fp16 output), rounded step by step as torch does."""
     if w.K != x.K:
         raise ValueError("K mismatch: %d vs %d" % (w.K, x.K))
     if (mode == MODE_BWTA) != x.ternary:
@@ -159,10 +182,24 @@ def bgemm_packed_forward(w, x, mode=MODE_XOR, out_dtype=torch.int32, splitK=1, v
     batch = max(w.batch, x.batch)
     if w.batch not in (1, batch) or x.batch not in (1, batch):
         raise ValueError("batch mismatch: %d vs %d" % (w.batch, x.batch))
-    if out_dtype not in (torch.int32, torch.half):
-        raise ValueError("out_dtype must be torch.int32 or torch.half")
     M, N, K = w.rows, x.rows, w.K
     dev = w.data.device
+    if scale is not None:
+        sw, sa, bias = scale
+        out_dtype = sw.dtype
+        if out_dtype not in (torch.float32, torch.half):
+            raise TypeError("scales must be fp32 or fp16")
+        for name, t, n in (("sw", sw, M), ("sa", sa, 1), ("bias", bias, M)):
+            if t is None and name == "bias":
+                continue
+            _need_cuda(t, name)
+            if t.dtype != out_dtype or t.numel() != n or not t.is_contiguous():
+                raise ValueError("%s must be a contiguous %s tensor of %d elements" % (name, out_dtype, n))
+        kind = OUT_F32_SCALED if out_dtype == torch.float32 else OUT_F16_SCALED
+    elif out_dtype not in (torch.int32, torch.half):
+        raise ValueError("out_dtype must be torch.int32 or torch.half")
+    else:
+        kind = OUT_F16 if out_dtype == torch.half else OUT_I32
     if out is None:
         out = torch.empty((batch, N, M), dtype=out_dtype, device=dev)
     L = _b.lib()
@@ -171,12 +208,16 @@ def bgemm_packed_forward(w, x, mode=MODE_XOR, out_dtype=torch.int32, splitK=1, v
         if splitK > 1:
             ws, cnt = _split_k_buffers(L.bgemm_packed_workspace_bytes(mode, batch, M, N, K, splitK, variant),
                                        L.bgemm_packed_counter_bytes(mode, batch, M, N, K, splitK, variant), dev)
-        _b.check(L.bgemm_packed_forward(
-            mode, w.data.data_ptr(), x.data.data_ptr(), x.data2.data_ptr() if x.ternary else None,
-            out.data_ptr(), OUT_F16 if out_dtype == torch.half else OUT_I32, batch, M, N, K,
-            w.words if w.batch > 1 else 0, x.words if x.batch > 1 else 0, N * M, splitK, variant,
-            ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0,
-            cnt.data_ptr() if cnt is not None else None, cnt.numel() if cnt is not None else 0, _stream()))
+        args = (mode, w.data.data_ptr(), x.data.data_ptr(), x.data2.data_ptr() if x.ternary else None,
+                out.data_ptr(), kind, batch, M, N, K,
+                w.words if w.batch > 1 else 0, x.words if x.batch > 1 else 0, N * M, splitK, variant,
+                ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0,
+                cnt.data_ptr() if cnt is not None else None, cnt.numel() if cnt is not None else 0)
+        if scale is None:
+            _b.check(L.bgemm_packed_forward(*args, _stream()))
+        else:
+            _b.check(L.bgemm_packed_forward_scaled(*args, sw.data_ptr(), sa.data_ptr(),
+                                                   bias.data_ptr() if bias is not None else None, _stream()))
     return out
 
 

@@ -35,7 +35,12 @@ extern "C" {
 /* INSTR values 0..2 are the reference's API (configs.h:70-72); 3 and 4 are supersets. */
 enum { BGEMM_MODE_AND = 0, BGEMM_MODE_XOR = 1, BGEMM_MODE_ATTN = 2, BGEMM_MODE_BWTA = 3,
        BGEMM_MODE_ATTN_X = 4 };
-enum { BGEMM_OUT_I32 = 0, BGEMM_OUT_F16 = 1 };
+/* Output kinds.  I32 = the accumulator; F16 = the integer rounded to nearest even.
+ * F32_SCALED / F16_SCALED = the binary Linear's scaling fused into the store (see
+ * bgemm_packed_forward_scaled): fp32 resp. fp16 output, parameters of the same type. */
+enum { BGEMM_OUT_I32 = 0, BGEMM_OUT_F16 = 1, BGEMM_OUT_F32_SCALED = 2, BGEMM_OUT_F16_SCALED = 3 };
+/* Element type of a floating-point source operand. */
+enum { BGEMM_SRC_F16 = 0, BGEMM_SRC_F32 = 1 };
 /* Kernel family: AUTO picks per shape; VALU = and + popcount on the vector ALU;
  * MFMA = bit planes expanded to int8 in registers feeding v_mfma_i32_32x32x32_i8;
  * MFMA_F4 = bit planes expanded to E2M1 nibbles feeding v_mfma_f32_32x32x64_f8f6f4
@@ -80,6 +85,14 @@ int bgemm_pack_sign_f16_logical(const void* src, int64_t rows, int64_t K, int64_
  * tests/python/bgemm_linear.py:222-241). */
 int bgemm_pack_ternary_f16(const void* src, int64_t rows, int64_t K, int64_t ld,
                            void* nz_tiled, void* sg_tiled, void* stream);
+/* Centre-and-pack in one pass: bit = sign bit of half_rn(src[r][k] - *zero_point), the
+ * operand the binary Linear layers hand to the kernel (tests/python/bgemm_linear.py:479-482:
+ * `x - zpa` resp. `weight - zpw`, then `.to(torch.half)`, then the sign pack of
+ * ptx_mma.cuh:341-380).  src is fp16 or fp32 (BGEMM_SRC_*) with row stride ld elements;
+ * zero_point is a DEVICE pointer to one scalar of the source type (so a zero point that
+ * was computed on the GPU needs no host read-back), or NULL for 0. */
+int bgemm_pack_sign_centered(const void* src, int src_dtype, int64_t rows, int64_t K, int64_t ld,
+                             const void* zero_point, void* dst_tiled, void* stream);
 /* logical <-> tiled re-layout of already packed bits (device buffers). */
 int bgemm_tile_from_logical(const uint32_t* logical, int64_t rows, int64_t K,
                             void* dst_tiled, void* stream);
@@ -111,6 +124,21 @@ int bgemm_packed_forward(int mode, const void* W_tiled, const void* X_tiled, con
                          int64_t strideW, int64_t strideX, int64_t strideC,
                          int splitK, int variant, void* ws, size_t ws_bytes,
                          void* counters, size_t counter_bytes, void* stream);
+
+/* The same GEMM with the binary Linear's output scaling fused into the store, replacing the
+ * separate elementwise kernels of `bgemm(...) * sw * sa (+ bias)`
+ * (tests/python/bgemm_linear.py:482-484).  Every step is evaluated and rounded exactly as
+ * torch evaluates that expression: h = fp16_rn(C[n,m]); then, for BGEMM_OUT_F32_SCALED
+ * (fp32 parameters, fp32 output) out = (float(h) * sw[m]) * sa + bias[m] in fp32; for
+ * BGEMM_OUT_F16_SCALED (fp16 parameters, fp16 output) the same with every step rounded to
+ * fp16.  sw: M per-output-channel scales; sa: one scalar; bias: M values or NULL; all are
+ * DEVICE pointers of the output's element type. */
+int bgemm_packed_forward_scaled(int mode, const void* W_tiled, const void* X_tiled, const void* X2_tiled,
+                                void* out, int out_dtype, int64_t batch, int64_t M, int64_t N, int64_t K,
+                                int64_t strideW, int64_t strideX, int64_t strideC,
+                                int splitK, int variant, void* ws, size_t ws_bytes,
+                                void* counters, size_t counter_bytes,
+                                const void* sw, const void* sa, const void* bias, void* stream);
 
 /* ---- fp16-operand call, the drop-in for the reference launcher -----------------------
  * Same argument meaning as bin_pack_linear_kernel (fp6_linear.cu:275-286):

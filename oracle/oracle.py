@@ -177,6 +177,38 @@ def bits_to_f16(bits, zero_mask=None):
     return v
 
 
+# ---------------------------------------------------------------- layer prologue / epilogue
+def np_center_to_f16(x, zero_point):
+    """What the binary Linear layers hand to the kernel (bgemm_linear.py:479-482, :140-141):
+    ``(x - zp)`` in the tensor's own type (fp32, or fp16 evaluated through fp32 and rounded),
+    then ``.to(torch.half)``.  Returns the fp16 array whose sign bits get packed."""
+    x = np.asarray(x)
+    if x.dtype == np.float32:
+        return (x - np.float32(zero_point)).astype(np.float16)
+    assert x.dtype == np.float16
+    return (x.astype(np.float32) - np.float32(np.float16(zero_point))).astype(np.float16)
+
+
+def np_scale_epilogue(acc_i32, sw, sa, bias=None):
+    """``half(acc) * sw * sa (+ bias)`` (bgemm_linear.py:482-484) with torch's type promotion:
+    fp32 parameters -> every step is an fp32 operation and the result is fp32; fp16 parameters ->
+    every step is evaluated in fp32 and rounded to fp16.  acc: int32 [N,M]; sw: [M]; sa: scalar."""
+    with np.errstate(over="ignore"):
+        h = np.asarray(acc_i32).astype(np.float32).astype(np.float16)
+    sw = np.asarray(sw)
+    if sw.dtype == np.float32:
+        r = h.astype(np.float32) * sw[None, :]
+        r = r * np.float32(sa)
+        return r + np.asarray(bias, dtype=np.float32)[None, :] if bias is not None else r
+    assert sw.dtype == np.float16
+    with np.errstate(over="ignore", invalid="ignore"):
+        r = (h.astype(np.float32) * sw.astype(np.float32)[None, :]).astype(np.float16)
+        r = (r.astype(np.float32) * np.float32(np.float16(sa))).astype(np.float16)
+        if bias is not None:
+            r = (r.astype(np.float32) + np.asarray(bias, dtype=np.float16).astype(np.float32)[None, :]).astype(np.float16)
+    return r
+
+
 # ---------------------------------------------------------------- reference CPU path
 def cpu_path_linear(x_vals, w_vals):
     """torch matmul on +-1/0 tensors: out = x @ w.T  (bgemm_linear.py:270-272)."""

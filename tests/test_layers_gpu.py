@@ -71,6 +71,36 @@ def test_bgemm_linear_module_vs_bnn(oracle, cls):
     assert torch.equal(lin(x[:5]), want[:5])
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.half])
+@pytest.mark.parametrize("bias", [True, False])
+def test_fused_inference_forward_equals_composed_ops(dtype, bias):
+    """Under no_grad the module centres+packs x in one pass, reuses the packed weight and scales in
+    the GEMM's store; the result must equal the op-by-op forward (bgemm_linear.py:479-484) bit for bit."""
+    torch.manual_seed(7)
+    lin = bl.BGEMMLinear(784, 300, bias=bias).to(DEV).to(dtype)
+    x = torch.randn(3, 50, 784, device=DEV).to(dtype)
+    y_ops = lin(x)                                   # grad mode: separate torch kernels around the GEMM
+    assert y_ops.requires_grad
+    with torch.no_grad():
+        assert lin._fusable(x)
+        y_fused = lin(x)
+        lin.fuse_inference = False
+        y_plain = lin(x)
+        lin.fuse_inference = True
+    assert y_fused.dtype == y_ops.dtype == dtype and y_fused.shape == y_ops.shape
+    assert torch.equal(y_fused, y_ops.detach()) and torch.equal(y_fused, y_plain)
+    # the packed weight is cached until the weight changes
+    wp = lin._packed_weight()
+    assert lin._packed_weight() is wp
+    with torch.no_grad():
+        lin.weight.neg_()
+        assert lin._packed_weight() is not wp
+        lin.fuse_inference = False
+        want = lin(x)
+        lin.fuse_inference = True
+        assert torch.equal(lin(x), want)
+
+
 def test_elastic_module_matches_cpu_twin():
     torch.manual_seed(4)
     x = torch.randn(64, 256, device=DEV)

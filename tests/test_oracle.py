@@ -156,3 +156,56 @@ def test_config1_cpu_reference_path(oracle):
     assert (got.T == want).all()
     assert (oracle.cpu_path_linear(torch.from_numpy(x16.astype(np.float32)),
                                    torch.from_numpy(w16.astype(np.float32))).numpy() == got).all()
+
+
+# ---------------------------------------------------------------- layer prologue / epilogue
+@pytest.mark.parametrize("dtype", ["float32", "float16"])
+def test_scale_epilogue_matches_torch_ops(oracle, dtype):
+    """np_scale_epilogue against the expression the layers evaluate with torch's own elementwise
+    kernels, `half(acc) * sw * sa + bias` (bgemm_linear.py:482-484), bit for bit."""
+    import torch
+    rng = np.random.default_rng(11)
+    acc = rng.integers(-70000, 70000, size=(37, 53)).astype(np.int32)       # beyond fp16 range too
+    acc[0, :8] = [2049, 2051, -2049, 4099, 65519, 65520, -65520, 0]         # ties, overflow
+    tdt = getattr(torch, dtype)
+    sw = torch.from_numpy(rng.uniform(1e-4, 3e-3, 53).astype(np.float32)).to(tdt)
+    bias = torch.from_numpy(rng.standard_normal(53).astype(np.float32)).to(tdt)
+    sa = torch.tensor(1.7371, dtype=tdt)
+    h = torch.from_numpy(acc).to(torch.float32).to(torch.half)
+    want = h * sw * sa
+    got = oracle.np_scale_epilogue(acc, sw.numpy(), sa.item(), None)
+    assert got.dtype == want.numpy().dtype
+    assert (got.view(np.uint32 if dtype == "float32" else np.uint16) ==
+            want.numpy().view(np.uint32 if dtype == "float32" else np.uint16)).all()
+    want += bias.view(1, -1).expand_as(want)
+    got = oracle.np_scale_epilogue(acc, sw.numpy(), sa.item(), bias.numpy())
+    assert (got.view(np.uint32 if dtype == "float32" else np.uint16) ==
+            want.numpy().view(np.uint32 if dtype == "float32" else np.uint16)).all()
+
+
+def test_scale_epilogue_hand_values(oracle):
+    # 2049 rounds to fp16 2048 (tie to even); 2048 * 0.5 * 3 + 1 = 3073 exactly in fp32,
+    # and 3073 is not an fp16 value: it rounds to 3072 (spacing 2 above 2048)
+    acc = np.array([[2049]], dtype=np.int32)
+    r32 = oracle.np_scale_epilogue(acc, np.array([0.5], np.float32), 3.0, np.array([1.0], np.float32))
+    assert r32.dtype == np.float32 and r32[0, 0] == 3073.0
+    r16 = oracle.np_scale_epilogue(acc, np.array([0.5], np.float16), 3.0, np.array([1.0], np.float16))
+    assert r16.dtype == np.float16 and r16[0, 0] == 3072.0
+    # 70000 overflows to inf at the first step, and stays inf whatever the scale
+    assert np.isinf(oracle.np_scale_epilogue(np.array([[70000]], np.int32), np.array([1e-4], np.float32), 1.0)[0, 0])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float16"])
+def test_center_to_f16_matches_torch_ops(oracle, dtype):
+    """np_center_to_f16 against `(x - zp).to(torch.half)` and its sign bit against `x < zp`."""
+    import torch
+    rng = np.random.default_rng(12)
+    x = rng.standard_normal((9, 300)).astype(dtype)
+    zp = np.asarray(x.mean(), dtype=dtype)
+    x[0, :4] = [zp, np.nextafter(zp, np.asarray(-9, dtype)), np.nextafter(zp, np.asarray(9, dtype)), 0.0]
+    tx = torch.from_numpy(x)
+    want = (tx - torch.tensor(zp.item(), dtype=tx.dtype)).to(torch.half).numpy()
+    got = oracle.np_center_to_f16(x, zp)
+    assert (got.view(np.uint16) == want.view(np.uint16)).all()
+    # x == zp gives +0.0 (bit clear); anything below gives a set sign bit even when it underflows in fp16
+    assert ((got.view(np.uint16) >> 15) == (x < zp)).all()

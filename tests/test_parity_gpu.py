@@ -321,3 +321,59 @@ def test_split_k_workspace_left_clean():
     assert lk._counters
     for buf in lk._counters.values():
         assert int(buf.count_nonzero()) == 0
+
+
+# ------------------------------------------------------------------ fused layer prologue / epilogue
+def _bits(a):
+    return a.view(np.uint32 if a.dtype == np.float32 else np.uint16)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("rows,K", [(5, 33), (64, 784), (33, 1000), (128, 4096)])
+def test_pack_centered_matches_oracle(oracle, dtype, rows, K):
+    rng = np.random.default_rng(rows * 7 + K)
+    x = rng.standard_normal((rows, K)).astype(dtype)
+    zp = np.asarray(x.mean(), dtype=dtype)
+    x[0, 0], x[-1, -1] = zp, np.nextafter(zp, np.asarray(-9, dtype))       # exactly at / just below the zero point
+    want = oracle.c_pack_sign(oracle.np_center_to_f16(x, zp))
+    got = lk.logical_from_tiled(lk.pack_sign(to_dev(x), zero_point=to_dev(zp.reshape(1))))
+    assert (got.cpu().numpy().view(np.uint32) == want).all()
+    # zero_point = 0 is the plain sign pack of the rounded source
+    got0 = lk.logical_from_tiled(lk.pack_sign(to_dev(x), zero_point=torch.zeros(1, device=DEV)))
+    assert (got0.cpu().numpy().view(np.uint32) == oracle.c_pack_sign(x.astype(np.float16))).all()
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("M,N,K,splitK,with_bias", [(96, 40, 784, 1, True), (10, 128, 4096, 3, True),
+                                                    (4096, 128, 784, 1, False), (260, 7, 300, 2, True),
+                                                    (130, 70, 2500, 1, True)])
+def test_scaled_epilogue_matches_oracle(oracle, variant, dtype, M, N, K, splitK, with_bias):
+    rng = np.random.default_rng(M + N + K)
+    w, x = rand_f16(rng, M, K), rand_f16(rng, N, K)
+    sw = rng.uniform(1e-4, 3e-3, M).astype(dtype)
+    sa = np.asarray(1.7371, dtype=dtype)
+    bias = rng.standard_normal(M).astype(dtype) if with_bias else None
+    acc = oracle.c_bgemm_packed(1, oracle.c_pack_sign(w), oracle.c_pack_sign(x), K)
+    want = oracle.np_scale_epilogue(acc, sw, sa, bias)
+    got = lk.bgemm_packed_forward(lk.pack_sign(to_dev(w)), lk.pack_sign(to_dev(x)), MODE_XOR, splitK=splitK,
+                                  variant=variant,
+                                  scale=(to_dev(sw), to_dev(sa.reshape(1)), to_dev(bias) if with_bias else None))
+    got = got[0].cpu().numpy()
+    assert got.dtype == want.dtype and (_bits(got) == _bits(want)).all()
+
+
+def test_scaled_epilogue_empty_k_and_errors():
+    sw, sa, b = torch.full((8,), 0.5, device=DEV), torch.ones(1, device=DEV), torch.arange(8.0, device=DEV)
+    w0 = lk.PackedBits(torch.empty((1, 0), dtype=torch.int32, device=DEV), None, 1, 8, 0)
+    x0 = lk.PackedBits(torch.empty((1, 0), dtype=torch.int32, device=DEV), None, 1, 3, 0)
+    out = lk.bgemm_packed_forward(w0, x0, MODE_XOR, scale=(sw, sa, b))
+    assert torch.equal(out[0], b.expand(3, 8))                         # 0 * sw * sa + bias
+    out = lk.bgemm_packed_forward(w0, x0, MODE_XOR, out_dtype=torch.half)
+    assert torch.equal(out, torch.zeros_like(out))
+    w = lk.pack_sign(torch.randn(8, 64, device=DEV))
+    x = lk.pack_sign(torch.randn(3, 64, device=DEV))
+    with pytest.raises(ValueError):
+        lk.bgemm_packed_forward(w, x, MODE_XOR, scale=(sw[:4], sa, b))
+    with pytest.raises(ValueError):
+        lk.bgemm_packed_forward(w, x, MODE_XOR, scale=(sw, sa, b.half()))
