@@ -1,38 +1,63 @@
 // Skinny GEMM for decode-like shapes: the activation side fits one 32-row MFMA operand
 // (N <= 32 binary rows, or N <= 16 ternary rows whose two planes share the operand), so the
-// work is one pass over the packed weights and the kernel is HBM-bound.
+// work is one pass over the packed weights and the kernels are HBM-bound.  Weight tiles are
+// read once and streamed past the caches (non-temporal loads); the activation tiles are
+// re-read by every wave and stay cached.
 //
-// A block owns RT weight row tiles; its KW waves split K between them (the in-kernel split-K:
-// no workspace, no second launch, no atomics on global memory) and meet in LDS, where the
-// partial accumulators are summed, the rank-one terms applied and the rows stored.
+// Two kernels:
+//  * gemm_skinny_stream_kernel: every wave owns RT weight row tiles over the whole K and keeps
+//    its accumulators to the end: no LDS, no barriers, nothing shared between waves.  Used when
+//    there are enough row tiles (a batch of weight matrices, a very tall one) to fill the chip.
+//  * gemm_skinny_splitk_kernel: a block owns one row tile and its KW waves split K between them
+//    (the in-kernel split-K: no workspace, no second launch, no atomics on global memory); the
+//    partial sums meet in LDS through ds_add.  Used for a single decode-size matrix, which has
+//    too few row tiles to occupy every SIMD otherwise.
 #include "common.h"
 #include "mfma_engines.h"
 
 namespace bgemm {
 
-template <typename Eng, int RT, int KW>
-__global__ __launch_bounds__(KW * 64) void gemm_skinny_kernel(const GemmArgs a, const int groups)
-{
-    __shared__ int sAcc[KW][RT][16][64];
-    __shared__ int sPa[RT][32], sPb[32];
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+// Weight tiles are used exactly once: keep them out of the way of the activation tiles.
+__device__ __forceinline__ uint4 load_stream(const uint4* p)
+{
+    const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+
+// Pointer to this lane's slot of the activation operand's first K-tile.  With two planes, rows
+// 0..15 of the operand come from the nonzero plane and rows 16..31 from the sign&nonzero plane
+// (both hold at most 16 real rows), so one MFMA yields both dots.
+__device__ __forceinline__ const uint4* skinny_x_ptr(const GemmArgs& a, const int b, const int lane)
+{
     const int h = lane >> 5, r = lane & 31;
-    const int b = blockIdx.x / groups, grp = blockIdx.x % groups;
+    const bool two = a.mc.planes == 2;
+    return (two && r >= 16 ? a.X2 + (h * 32 + r - 16) : a.X + lane) + (int64_t)b * a.strideX;
+}
+
+// Output of one (activation row, weight row) pair from the AND-dots d (and d2 of the second plane).
+__device__ __forceinline__ int skinny_value(const ModeCoef& mc, const bool two, const int kbits, const int pa,
+                                            const int pb, const int pb2, const int d, const int d2)
+{
+    int val = __mul24(mc.c0, kbits) + __mul24(mc.ca, pa) + __mul24(mc.cb, pb) + __mul24(mc.cd, d);
+    if (two) val += __mul24(mc.cb2, pb2) + __mul24(mc.cd2, d2);
+    return val;
+}
+
+// ---- streaming kernel --------------------------------------------------------------------------
+template <typename Eng, int RT>
+__global__ __launch_bounds__(256) void gemm_skinny_stream_kernel(const GemmArgs a, const int groups)
+{
+    constexpr int CH = 4;                        // K-tiles per chunk; two chunks are in flight
+    const int lane = threadIdx.x & 63;
+    const int h = lane >> 5, r = lane & 31;
+    const int64_t gid = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int b = (int)(gid / groups), grp = (int)(gid % groups);
+    if (b >= a.batch) return;                    // whole wave leaves together
     const bool two = a.mc.planes == 2;
 
-    if (threadIdx.x < 32) {
-        sPb[threadIdx.x] = 0;
-#pragma unroll
-        for (int t = 0; t < RT; t++) sPa[t][threadIdx.x] = 0;
-    }
-
-    int kt0, kt1;
-    split_range(a.KT, KW, wave, &kt0, &kt1);
-
-    // activation operand: one tile row; with two planes rows 0..15 come from the nonzero plane
-    // and rows 16..31 from the sign&nonzero plane (both hold at most 16 real rows)
-    const uint4* xp = (two && r >= 16 ? a.X2 + (h * 32 + r - 16) : a.X + lane) + (int64_t)b * a.strideX;
+    const uint4* xp = skinny_x_ptr(a, b, lane);
     const uint4* wp[RT];
 #pragma unroll
     for (int t = 0; t < RT; t++) {
@@ -49,21 +74,24 @@ __global__ __launch_bounds__(KW * 64) void gemm_skinny_kernel(const GemmArgs a, 
 #pragma unroll
     for (int t = 0; t < RT; t++) pa[t] = 0;
 
-    // all of this wave's K range is requested up front: the ranges are short (K/KW) and the
-    // kernel lives on memory-level parallelism
-    constexpr int MAXT = 4;                      // K-tiles kept in flight per wave
-    for (int kb = kt0; kb < kt1; kb += MAXT) {
-        uint4 xq[MAXT], wq[MAXT][RT];
+    // a chunk that starts inside K is fetched whole: K-tiles past the end are read again from the
+    // last one and skipped when the chunk is consumed
+    const int kt_last = a.KT - 1;
+    uint4 xq0[CH], xq1[CH], wq0[CH][RT], wq1[CH][RT];
+    auto fetch = [&](uint4 (&xq)[CH], uint4 (&wq)[CH][RT], const int kb) {
+        if (kb > kt_last) return;
 #pragma unroll
-        for (int q = 0; q < MAXT; q++) {
-            const int64_t off = (int64_t)min(kb + q, kt1 - 1) * TILE_U4;
+        for (int q = 0; q < CH; q++) {
+            const int64_t off = (int64_t)min(kb + q, kt_last) * TILE_U4;
             xq[q] = xp[off];
 #pragma unroll
-            for (int t = 0; t < RT; t++) wq[q][t] = wp[t][off];
+            for (int t = 0; t < RT; t++) wq[q][t] = load_stream(wp[t] + off);
         }
+    };
+    auto consume = [&](const uint4 (&xq)[CH], const uint4 (&wq)[CH][RT], const int kb) {
 #pragma unroll
-        for (int q = 0; q < MAXT; q++) {
-            if (kb + q >= kt1) break;
+        for (int q = 0; q < CH; q++) {
+            if (kb + q > kt_last) break;
             pb += popc4(xq[q]);
 #pragma unroll
             for (int t = 0; t < RT; t++) pa[t] += popc4(wq[q][t]);
@@ -74,41 +102,118 @@ __global__ __launch_bounds__(KW * 64) void gemm_skinny_kernel(const GemmArgs a, 
                 for (int t = 0; t < RT; t++) acc[t] = Eng::mma(ax, Eng::expand(wq[q][t], s), acc[t]);
             }
         }
+    };
+    fetch(xq0, wq0, 0);
+    for (int kb = 0; kb < a.KT; kb += 2 * CH) {
+        fetch(xq1, wq1, kb + CH);
+        consume(xq0, wq0, kb);
+        fetch(xq0, wq0, kb + 2 * CH);
+        consume(xq1, wq1, kb + CH);
     }
 
-    // ---- meet in LDS ---------------------------------------------------------------------------
-    pb += __shfl_xor(pb, 32);
+    // ---- rank-one terms and store, straight from the accumulators ---------------------------------
+    pb += __shfl_xor(pb, 32);                    // lane r (either half) now holds the popcount of operand row r
 #pragma unroll
     for (int t = 0; t < RT; t++) pa[t] += __shfl_xor(pa[t], 32);
-    __syncthreads();                 // popcount arrays are zeroed
+    const ModeCoef mc = a.mc;
+    const int kbits = (int)a.K;
+    const int64_t out_row0 = (int64_t)b * a.strideC;
 #pragma unroll
-    for (int t = 0; t < RT; t++)
+    for (int v = 0; v < 16; v++) {
+        const int n = 8 * (v >> 2) + 4 * h + (v & 3);
+        const int pbn = __shfl(pb, n), pbn2 = __shfl(pb, (n + 16) & 31);
+        if (n >= a.N || (two && v >= 8)) continue;      // rows 16..31 of a two-plane operand are the second plane
 #pragma unroll
-        for (int v = 0; v < 16; v++) sAcc[wave][t][v][lane] = Eng::to_int(acc[t], v);
-    if (lane < 32) {
-        atomicAdd(&sPb[lane], pb);
+        for (int t = 0; t < RT; t++) {
+            const int64_t m = ((int64_t)grp * RT + t) * 32 + r;
+            const int val = skinny_value(mc, two, kbits, pa[t], pbn, pbn2, Eng::to_int(acc[t], v),
+                                         Eng::to_int(acc[t], (v + 8) & 15));
+            if (m < a.M) store_out(a, out_row0 + (int64_t)n * a.M, m, val);
+        }
+    }
+}
+
+// ---- split-K kernel ----------------------------------------------------------------------------
+template <typename Eng, int KW>
+__global__ __launch_bounds__(KW * 64) void gemm_skinny_splitk_kernel(const GemmArgs a)
+{
+    constexpr int NT = KW * 64;
+    __shared__ int sAcc[16][64];                 // accumulator layout of the MFMA: [v][lane]
+    __shared__ int sPa[32], sPb[32];
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int h = lane >> 5;
+    const int b = blockIdx.x / a.MT, rt = blockIdx.x % a.MT;
+    const bool two = a.mc.planes == 2;
+
+    int kt0, kt1;
+    split_range(a.KT, KW, wave, &kt0, &kt1);
+
+    const uint4* xp = skinny_x_ptr(a, b, lane);
+    const uint4* wp = a.W + (int64_t)b * a.strideW + (int64_t)rt * a.KT * TILE_U4 + lane;
+
+    typename Eng::Acc acc;
 #pragma unroll
-        for (int t = 0; t < RT; t++) atomicAdd(&sPa[t][lane], pa[t]);
+    for (int v = 0; v < 16; v++) acc[v] = 0;
+    int pa = 0, pb = 0;
+
+    // the wave's K range is short (K / KW) and requested four K-tiles at a time: the kernel lives
+    // on memory-level parallelism
+    constexpr int MAXT = 4;
+    for (int kb = kt0; kb < kt1 || kb == kt0; kb += MAXT) {
+        uint4 xq[MAXT], wq[MAXT];
+        if (kb < kt1) {
+#pragma unroll
+            for (int q = 0; q < MAXT; q++) {
+                const int64_t off = (int64_t)min(kb + q, kt1 - 1) * TILE_U4;
+                xq[q] = xp[off];
+                wq[q] = load_stream(wp + off);
+            }
+        }
+        if (kb == kt0) {
+            // clear the meeting area while the first loads are in flight: every wave gets here at
+            // once, so this barrier costs next to nothing
+            for (int i = threadIdx.x; i < 16 * 64; i += NT) (&sAcc[0][0])[i] = 0;
+            if (threadIdx.x < 32) { sPb[threadIdx.x] = 0; sPa[threadIdx.x] = 0; }
+            __syncthreads();
+        }
+        if (kb < kt1) {
+#pragma unroll
+            for (int q = 0; q < MAXT; q++) {
+                if (kb + q >= kt1) break;
+                pb += popc4(xq[q]);
+                pa += popc4(wq[q]);
+#pragma unroll
+                for (int s = 0; s < Eng::STEPS; s++) acc = Eng::mma(Eng::expand(xq[q], s), Eng::expand(wq[q], s), acc);
+            }
+        }
+    }
+
+    // ---- meet in LDS: integer adds of the accumulator rows that carry outputs ------------------------
+    pb += __shfl_xor(pb, 32);
+    pa += __shfl_xor(pa, 32);
+    if (kt0 < kt1) {
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            const int n = 8 * (v >> 2) + 4 * h + (v & 3);
+            if ((two ? (n & 15) : n) < a.N) atomicAdd(&sAcc[v][lane], Eng::to_int(acc, v));
+        }
+        if (lane < 32) { atomicAdd(&sPb[lane], pb); atomicAdd(&sPa[lane], pa); }
     }
     __syncthreads();
 
-    // ---- reduce, apply the mode's rank-one terms, store -------------------------------------------
+    // ---- rank-one terms and store: one output per thread and step, consecutive threads on one row ----
     const ModeCoef mc = a.mc;
-    const int out_rows = two ? 8 : 16;           // accumulator rows that carry outputs
     const int kbits = (int)a.K;
-    for (int job = wave; job < RT * out_rows; job += KW) {
-        const int t = job / out_rows, v = job % out_rows;
-        int d = 0, d2 = 0;
-#pragma unroll
-        for (int w = 0; w < KW; w++) {
-            d += sAcc[w][t][v][lane];
-            if (two) d2 += sAcc[w][t][v + 8][lane];
-        }
-        const int n = 8 * (v >> 2) + 4 * h + (v & 3);
-        const int64_t m = ((int64_t)grp * RT + t) * 32 + r;
-        int val = __mul24(mc.c0, kbits) + __mul24(mc.ca, sPa[t][r]) + __mul24(mc.cb, sPb[n]) + __mul24(mc.cd, d);
-        if (two) val += __mul24(mc.cb2, sPb[n + 16]) + __mul24(mc.cd2, d2);
-        if (n < a.N && m < a.M) store_out(a, (int64_t)b * a.strideC + (int64_t)n * a.M, m, val);
+    const int nout = (int)a.N * 32;
+    for (int o = threadIdx.x; o < nout; o += NT) {
+        const int n = o >> 5, c = o & 31;
+        const int v = 4 * (n >> 3) + (n & 3), hh = (n >> 2) & 1;      // accumulator slot of operand row n
+        const int d = sAcc[v][hh * 32 + c];
+        const int d2 = two ? sAcc[v + 8][hh * 32 + c] : 0;
+        const int64_t m = (int64_t)rt * 32 + c;
+        const int val = skinny_value(mc, two, kbits, sPa[c], sPb[n], two ? sPb[n + 16] : 0, d, d2);
+        if (m < a.M) store_out(a, (int64_t)b * a.strideC + (int64_t)n * a.M, m, val);
     }
 }
 
@@ -117,32 +222,41 @@ bool gemm_skinny_eligible(const GemmArgs& a)
     return a.mc.planes == 2 ? a.N <= 16 : a.N <= 32;
 }
 
-template <typename Eng, int RT>
-static int launch_rt(const GemmArgs& a, hipStream_t st)
+template <typename Eng>
+static int launch_splitk(const GemmArgs& a, hipStream_t st)
 {
-    const int groups = (int)cdiv(a.MT, RT);
-    const int64_t blocks = (int64_t)a.batch * groups;
+    const int64_t blocks = (int64_t)a.batch * a.MT;
     if (blocks > 0x7fffffffLL) return fail(BGEMM_EINVAL, "gemm_skinny: grid of %lld blocks", (long long)blocks);
     // K ways per block: at least what the caller asked for, more when the grid alone would leave the
     // chip mostly idle (about four waves per SIMD wanted), never more than there are K-tiles
-    constexpr int KW_MAX = 8 / RT;               // the LDS meeting area is KW * RT * 4 KiB
     int kw = 1;
-    while (kw < KW_MAX && (kw < a.splitK || blocks * kw < 4096) && kw * 2 <= a.KT) kw *= 2;
+    while (kw < 8 && (kw < a.splitK || blocks * kw < 4096) && kw * 2 <= a.KT) kw *= 2;
     const dim3 g((unsigned)blocks);
-    if (kw == 1) hipLaunchKernelGGL((gemm_skinny_kernel<Eng, RT, 1>), g, dim3(64), 0, st, a, groups);
-    else if (kw == 2) hipLaunchKernelGGL((gemm_skinny_kernel<Eng, RT, 2>), g, dim3(128), 0, st, a, groups);
-    else if (kw == 4) hipLaunchKernelGGL((gemm_skinny_kernel<Eng, RT, 4>), g, dim3(256), 0, st, a, groups);
-    else if constexpr (KW_MAX >= 8) hipLaunchKernelGGL((gemm_skinny_kernel<Eng, RT, 8>), g, dim3(512), 0, st, a, groups);
+    if (kw == 1) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 1>), g, dim3(64), 0, st, a);
+    else if (kw == 2) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 2>), g, dim3(128), 0, st, a);
+    else if (kw == 4) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 4>), g, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 8>), g, dim3(512), 0, st, a);
+    return check_launch("gemm_skinny");
+}
+
+template <typename Eng, int RT>
+static int launch_stream(const GemmArgs& a, hipStream_t st)
+{
+    const int groups = (int)cdiv(a.MT, RT);
+    const int64_t blocks = cdiv((int64_t)a.batch * groups, 4);
+    if (blocks > 0x7fffffffLL) return fail(BGEMM_EINVAL, "gemm_skinny: grid of %lld blocks", (long long)blocks);
+    hipLaunchKernelGGL((gemm_skinny_stream_kernel<Eng, RT>), dim3((unsigned)blocks), dim3(256), 0, st, a, groups);
     return check_launch("gemm_skinny");
 }
 
 int launch_gemm_skinny(const GemmArgs& a, hipStream_t st, bool fp4)
 {
-    // two row tiles per block share one expansion of the activation fragment once there are
-    // enough row tiles to keep every CU busy anyway
-    const bool rt2 = (int64_t)a.batch * a.MT >= 2048;
-    if (fp4) return rt2 ? launch_rt<EngF4, 2>(a, st) : launch_rt<EngF4, 1>(a, st);
-    return rt2 ? launch_rt<EngI8, 2>(a, st) : launch_rt<EngI8, 1>(a, st);
+    // Enough row tiles for about four waves on every SIMD: no K split needed (the result does not
+    // depend on it).  Two row tiles per wave share one expansion of the activation tiles.
+    const int64_t row_tiles = (int64_t)a.batch * a.MT;
+    if (row_tiles >= 8192) return fp4 ? launch_stream<EngF4, 2>(a, st) : launch_stream<EngI8, 2>(a, st);
+    if (row_tiles >= 4096) return fp4 ? launch_stream<EngF4, 1>(a, st) : launch_stream<EngI8, 1>(a, st);
+    return fp4 ? launch_splitk<EngF4>(a, st) : launch_splitk<EngI8>(a, st);
 }
 
 }  // namespace bgemm

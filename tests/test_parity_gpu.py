@@ -377,3 +377,30 @@ def test_scaled_epilogue_empty_k_and_errors():
         lk.bgemm_packed_forward(w, x, MODE_XOR, scale=(sw[:4], sa, b))
     with pytest.raises(ValueError):
         lk.bgemm_packed_forward(w, x, MODE_XOR, scale=(sw, sa, b.half()))
+
+
+# ------------------------------------------------------------------ skinny shapes with many row tiles
+@pytest.mark.parametrize("B,M,N,K", [(40, 4100, 5, 300),      # 5160 row tiles: one per wave, ragged M and K
+                                     (70, 4000, 16, 2304),    # 8750 row tiles: two per wave, nine K-tiles
+                                     (1, 262144 + 40, 1, 256),# one tall matrix, odd number of row tiles
+                                     (33, 8000, 32, 1000)])   # 32 binary activation rows
+def test_skinny_streaming_batched(B, M, N, K):
+    g = torch.Generator(device=DEV).manual_seed(B * 31 + N)
+    w = torch.randn((B, M, K), generator=g, device=DEV, dtype=torch.half)
+    x = torch.randn((N, K), generator=g, device=DEV, dtype=torch.half)
+    x[:, ::5] = 0
+    wp, xp, xt = lk.pack_sign(w), lk.pack_sign(x), lk.pack_ternary(x)
+    ws, xs = torch.where(torch.signbit(w), -1.0, 1.0), torch.where(torch.signbit(x), -1.0, 1.0)
+    want = {
+        MODE_XOR: xs @ ws.transpose(1, 2),
+        MODE_AND: (xs < 0).float() @ (ws < 0).float().transpose(1, 2),
+        MODE_ATTN: xs @ (ws > 0).float().transpose(1, 2),
+        MODE_ATTN_X: (xs > 0).float() @ ws.transpose(1, 2),
+        MODE_BWTA: torch.sign(x.float()) @ ws.transpose(1, 2),
+    }
+    for mode in ([MODE_XOR, MODE_AND, MODE_ATTN, MODE_ATTN_X] + ([MODE_BWTA] if N <= 16 else [])):
+        got = lk.bgemm_packed_forward(wp, xt if mode == MODE_BWTA else xp, mode, torch.int32)
+        assert tuple(got.shape) == (B, N, M) and torch.equal(got, want[mode].to(torch.int32)), mode
+    variants = {v: lk.bgemm_packed_forward(wp, xp, MODE_XOR, torch.half, 1, v) for v in (VARIANT_MFMA, VARIANT_MFMA_F4)}
+    for v, got in variants.items():
+        assert torch.equal(got, want[MODE_XOR].half()), v
