@@ -101,16 +101,15 @@ __device__ __forceinline__ bool splitk_arrive(unsigned* counter, const unsigned 
     return *s_flag != 0;
 }
 
-// Device-scope load of one partial-tile vector (bypasses the reader's L1).
-__device__ __forceinline__ int4 load_partial(const int4* p)
+// Device-scope 16-byte load of one partial-tile vector: `sc1` makes it miss the reader's L1 and
+// take the line from the L2 the writer's stores went to.  `base` is uniform across the wave
+// (a buffer resource is built from it), `byte_off` is this lane's offset from it.
+__device__ __forceinline__ int4 load_partial(const void* base, const unsigned byte_off)
 {
-    const int* q = reinterpret_cast<const int*>(p);
-    int4 v;
-    v.x = __hip_atomic_load(q + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    v.y = __hip_atomic_load(q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    v.z = __hip_atomic_load(q + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    v.w = __hip_atomic_load(q + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    return v;
+    typedef int v4i __attribute__((ext_vector_type(4)));
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0x7fffffff, 0x00020000);
+    const v4i v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)byte_off, 0, 16 /* sc1 */);
+    return make_int4(v.x, v.y, v.z, v.w);
 }
 
 // Split-K grids are padded to a multiple of 8 * splitK blocks and numbered split-fastest, so
@@ -119,12 +118,13 @@ static inline int64_t splitk_grid(int64_t real_blocks, int splitK)
 {
     return splitK > 1 ? cdiv(real_blocks, 8 * (int64_t)splitK) * 8 * splitK : real_blocks;
 }
-// More K ranges than needed to give every CU a few blocks only add hand-over traffic: the
-// result does not depend on the split, so the caller's value is treated as an upper bound.
+// More K ranges than it takes to give every compute unit a block only add hand-over traffic (a
+// grid that already has one block per unit gets slower when split): the result does not depend
+// on the split, so the caller's value is treated as an upper bound.
 static inline int effective_split(int64_t tiles, int splitK, int KT)
 {
     int s = splitK;
-    while (s > 1 && (tiles * s > 512 || s > KT)) s--;
+    while (s > 1 && (tiles * s > 384 || s > KT)) s--;
     return s;
 }
 

@@ -230,9 +230,8 @@ __global__ __launch_bounds__(WGN* WGM * 64) void gemm_mfma_kernel(const GemmArgs
     constexpr int TILE_I4 = WGN * WN * WGM * WM * 256;          // int4 per block tile
     int4* tile_base = nullptr;
     if (a.splitK > 1) {
-        tile_base = reinterpret_cast<int4*>(a.ws_part) + ((int64_t)b * per_gemm + tile_id) * a.splitK * TILE_I4 +
-                    (int64_t)wave * (WN * WM * 256) + lane;
-        int4* mine = tile_base + (int64_t)split * TILE_I4;
+        tile_base = reinterpret_cast<int4*>(a.ws_part) + ((int64_t)b * per_gemm + tile_id) * a.splitK * TILE_I4;
+        int4* mine = tile_base + (int64_t)split * TILE_I4 + wave * (WN * WM * 256) + lane;
 #pragma unroll
         for (int i = 0; i < WN; i++) {
             int val[WM][16];
@@ -268,12 +267,12 @@ __global__ __launch_bounds__(WGN* WGM * 64) void gemm_mfma_kernel(const GemmArgs
         if (a.splitK > 1) {
             for (int s = 0; s < a.splitK; s++) {
                 if (s == split) continue;
-                const int4* other = tile_base + (int64_t)s * TILE_I4;
+                const int4* other = tile_base + (int64_t)s * TILE_I4;       // uniform: one split's tile
 #pragma unroll
                 for (int j = 0; j < WM; j++)
 #pragma unroll
                     for (int g = 0; g < 4; g++) {
-                        const int4 o = load_partial(other + ((i * WM + j) * 4 + g) * 64);
+                        const int4 o = load_partial(other, (unsigned)(wave * (WN * WM * 256) + lane + ((i * WM + j) * 4 + g) * 64) * 16u);
                         val[j][4 * g] += o.x; val[j][4 * g + 1] += o.y;
                         val[j][4 * g + 2] += o.z; val[j][4 * g + 3] += o.w;
                     }
@@ -342,8 +341,11 @@ struct MfmaCfg { int id, bn, bm; };
 // Tile choice: the largest tile that still yields about two blocks per CU.
 static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int splitK, int planes)
 {
+    // The tile is chosen for the output alone: K ranges are only added (effective_split) where
+    // the tiles of the smallest efficient size still leave compute units idle.
+    (void)splitK;
     const int64_t want = 512;
-    auto blocks = [&](int bn, int bm) { return batch * splitK * cdiv(N, bn) * cdiv(M, bm); };
+    auto blocks = [&](int bn, int bm) { return batch * cdiv(N, bn) * cdiv(M, bm); };
     if (M <= 64) return blocks(128, 64) >= want ? MfmaCfg{7, 128, 64} : MfmaCfg{6, 64, 64};   // narrow outputs
     if (planes == 1 && blocks(256, 256) >= want) return {0, 256, 256};
     if (blocks(128, 128) >= want) return {1, 128, 128};

@@ -49,7 +49,7 @@ __device__ __forceinline__ int skinny_value(const ModeCoef& mc, const bool two, 
 template <typename Eng, int RT>
 __global__ __launch_bounds__(256) void gemm_skinny_stream_kernel(const GemmArgs a, const int groups)
 {
-    constexpr int CH = 4;                        // K-tiles per chunk; two chunks are in flight
+    constexpr int CH = 2;                        // K-tiles per chunk; two chunks are in flight
     const int lane = threadIdx.x & 63;
     const int h = lane >> 5, r = lane & 31;
     const int64_t gid = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);

@@ -119,8 +119,8 @@ __global__ __launch_bounds__(256) void gemm_valu_kernel(const GemmArgs a, const 
         }
     if (a.splitK > 1) {
         // partial tiles in register order; the last split to arrive adds the others to its own
-        int4* tile_base = reinterpret_cast<int4*>(a.ws_part) + ((int64_t)b * per_gemm + tile_id) * a.splitK * 1024 + tid;
-        int4* mine = tile_base + (int64_t)split * 1024;
+        int4* tile_base = reinterpret_cast<int4*>(a.ws_part) + ((int64_t)b * per_gemm + tile_id) * a.splitK * 1024;
+        int4* mine = tile_base + (int64_t)split * 1024 + tid;
 #pragma unroll
         for (int i = 0; i < 4; i++) mine[i * 256] = make_int4(val[i][0], val[i][1], val[i][2], val[i][3]);
         if (!splitk_arrive(a.ws_cnt + (int64_t)b * per_gemm + tile_id, (unsigned)a.splitK, &s_last)) return;
@@ -129,7 +129,7 @@ __global__ __launch_bounds__(256) void gemm_valu_kernel(const GemmArgs a, const 
             const int4* other = tile_base + (int64_t)s * 1024;
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                const int4 o = load_partial(other + i * 256);
+                const int4 o = load_partial(other, (unsigned)(tid + i * 256) * 16u);
                 val[i][0] += o.x; val[i][1] += o.y; val[i][2] += o.z; val[i][3] += o.w;
             }
         }
