@@ -211,7 +211,7 @@ def bench_c2(steps, warmup):
     def fwd_fused(i):
         h = x
         for Wp, sw in zip(Wps, sws):
-            h = lk.bgemm_packed_forward(Wp, lk.pack_sign(h), lk.MODE_XOR, scale=(sw, sa, None))[0]
+            h = lk.bgemm_packed_forward(Wp, lk.pack_sign(h), lk.MODE_XOR, splitK=8, scale=(sw, sa, None))[0]
         return h
     same = bool(torch.equal(fwd_ops(0), fwd_fused(0)))
     ms_ops = time_gpu(fwd_ops, warmup, steps)

@@ -231,7 +231,8 @@ class BGEMMLinear(_ScaledBinaryLinear):
         lead = x.shape[:-1]
         xp = lowbit_kernel.pack_sign(x.reshape(-1, x.shape[-1]), zero_point=self.zpa)
         bias = None if self.bias is None else self.bias.detach()
-        out = lowbit_kernel.bgemm_packed_forward(self._packed_weight(), xp, lowbit_kernel.MODE_XOR,
+        # splitK is an upper bound: the library only splits K where the output tiles alone leave CUs idle
+        out = lowbit_kernel.bgemm_packed_forward(self._packed_weight(), xp, lowbit_kernel.MODE_XOR, splitK=8,
                                                  scale=(self.sw.detach(), self.sa.detach().reshape(1), bias))
         return out.reshape(*lead, self.weight.shape[0])
 

@@ -32,13 +32,11 @@ static int pick_variant(int mode, int64_t batch, int64_t M, int64_t N, int64_t K
     return BGEMM_VARIANT_MFMA_F4;
 }
 
-static bool skinny_shape(int planes, int64_t N) { return planes == 2 ? N <= 16 : N <= 32; }
-
-static void ws_needs(int variant, int planes, int64_t batch, int64_t M, int64_t N, int splitK,
+static void ws_needs(int variant, int planes, int64_t batch, int64_t M, int64_t N, int64_t K, int splitK,
                      size_t* part, size_t* counters)
 {
     *part = *counters = 0;
-    if (variant != BGEMM_VARIANT_VALU && skinny_shape(planes, N)) return;      // split inside the block
+    if (variant != BGEMM_VARIANT_VALU && gemm_skinny_shape(planes, batch, M, N, K)) return;      // split inside the block
     if (variant == BGEMM_VARIANT_VALU) gemm_valu_ws(batch, M, N, splitK, planes, part, counters);
     else gemm_mfma_ws(batch, M, N, splitK, planes, part, counters);
 }
@@ -65,7 +63,7 @@ static bool ws_query(int mode, int64_t batch, int64_t M, int64_t N, int64_t K, i
     if (!mode_coef(mode, &mc) || splitK <= 1 || batch <= 0 || M <= 0 || N <= 0 || K <= 0) return false;
     if (variant < BGEMM_VARIANT_AUTO || variant > BGEMM_VARIANT_MFMA_F4) return false;
     const int v = variant == BGEMM_VARIANT_AUTO ? pick_variant(mode, batch, M, N, K) : variant;
-    ws_needs(v, mc.planes, batch, M, N, splitK, part, counters);
+    ws_needs(v, mc.planes, batch, M, N, K, splitK, part, counters);
     return true;
 }
 
@@ -146,10 +144,10 @@ static int packed_forward(int mode, const void* W_tiled, const void* X_tiled, co
     a.batch = (int)batch; a.splitK = splitK;
     a.vec_store = (M % 4 == 0) && (strideC % 4 == 0) && (((uintptr_t)out & 15) == 0);
     const int v = variant == BGEMM_VARIANT_AUTO ? pick_variant(mode, batch, M, N, K) : variant;
-    const bool skinny = v != BGEMM_VARIANT_VALU && gemm_skinny_eligible(a);
+    const bool skinny = v != BGEMM_VARIANT_VALU && gemm_skinny_shape(a.mc.planes, batch, M, N, K);
     if (splitK > 1 && !skinny) {
         size_t part, cnt;
-        ws_needs(v, a.mc.planes, batch, M, N, splitK, &part, &cnt);
+        ws_needs(v, a.mc.planes, batch, M, N, K, splitK, &part, &cnt);
         if (!ws || !counters)
             return fail(BGEMM_EWORKSPACE, "bgemm_packed_forward: splitK=%d needs %zu workspace and %zu counter bytes",
                         splitK, round256(part), round256(cnt * 4));

@@ -118,13 +118,15 @@ static inline int64_t splitk_grid(int64_t real_blocks, int splitK)
 {
     return splitK > 1 ? cdiv(real_blocks, 8 * (int64_t)splitK) * 8 * splitK : real_blocks;
 }
+// The result does not depend on the split, so the caller's value is treated as an upper bound.
 // More K ranges than it takes to give every compute unit a block only add hand-over traffic (a
-// grid that already has one block per unit gets slower when split): the result does not depend
-// on the split, so the caller's value is treated as an upper bound.
+// grid that already has one block per unit gets slower when split), and a hand-over costs three
+// dependent trips to the L2 (store, ticket, load: about 4 us), as much as a few dozen K-tiles of
+// main loop: shorter ranges are not worth it.
 static inline int effective_split(int64_t tiles, int splitK, int KT)
 {
     int s = splitK;
-    while (s > 1 && (tiles * s > 384 || s > KT)) s--;
+    while (s > 1 && (tiles * s > 384 || KT / s < 24)) s--;
     return s;
 }
 
@@ -176,8 +178,8 @@ int pack_sign_pair(const void* srcA, int64_t rowsA, void* dstA, const void* srcB
 // Kernel families (each in its own translation unit).
 int launch_gemm_mfma(const GemmArgs& a, hipStream_t st, bool fp4);
 int launch_gemm_valu(const GemmArgs& a, hipStream_t st);
-// Skinny shapes (activation side fits one 32-row operand): in-block split-K, no workspace.
-bool gemm_skinny_eligible(const GemmArgs& a);
+// Skinny shapes (few activation rows): K is split inside the block, no workspace.
+bool gemm_skinny_shape(int planes, int64_t batch, int64_t M, int64_t N, int64_t K);
 int launch_gemm_skinny(const GemmArgs& a, hipStream_t st, bool fp4);
 // Split-K needs of each family for a shape: bytes of partial-tile scratch, number of counters.
 void gemm_mfma_ws(int64_t batch, int64_t M, int64_t N, int splitK, int planes, size_t* part_bytes, size_t* counters);

@@ -11,7 +11,8 @@
 //  * gemm_skinny_splitk_kernel: a block owns one row tile and its KW waves split K between them
 //    (the in-kernel split-K: no workspace, no second launch, no atomics on global memory); the
 //    partial sums meet in LDS through ds_add.  Used for a single decode-size matrix, which has
-//    too few row tiles to occupy every SIMD otherwise.
+//    too few row tiles to occupy every SIMD otherwise, and, with up to four activation tile rows
+//    per wave, for small batches (N <= 128) against a few thousand weight rows.
 #include "common.h"
 #include "mfma_engines.h"
 
@@ -134,71 +135,102 @@ __global__ __launch_bounds__(256) void gemm_skinny_stream_kernel(const GemmArgs 
 }
 
 // ---- split-K kernel ----------------------------------------------------------------------------
-template <typename Eng, int KW>
+// NTL = activation tile rows handled by every wave (32 activation rows each).  More than one is
+// for shapes whose output has too few tiles to occupy the chip in the general kernel (a batch of
+// 128 rows against a few thousand weight rows): all KW * (weight row tiles) waves work, each on a
+// short K range, instead of a few waves walking all of K.
+template <typename Eng, int KW, int NTL>
 __global__ __launch_bounds__(KW * 64) void gemm_skinny_splitk_kernel(const GemmArgs a)
 {
     constexpr int NT = KW * 64;
-    __shared__ int sAcc[16][64];                 // accumulator layout of the MFMA: [v][lane]
-    __shared__ int sPa[32], sPb[32];
+    __shared__ int sAcc[NTL][16][64];            // accumulator layout of the MFMA: [v][lane]
+    __shared__ int sPa[32], sPb[NTL][32];
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int h = lane >> 5;
     const int b = blockIdx.x / a.MT, rt = blockIdx.x % a.MT;
-    const bool two = a.mc.planes == 2;
+    const bool two = a.mc.planes == 2;           // only with NTL == 1
 
     int kt0, kt1;
     split_range(a.KT, KW, wave, &kt0, &kt1);
 
-    const uint4* xp = skinny_x_ptr(a, b, lane);
+    const uint4* xp[NTL];
+    if (NTL == 1) xp[0] = skinny_x_ptr(a, b, lane);
+    else {
+#pragma unroll
+        for (int i = 0; i < NTL; i++)            // tile rows past the end re-read the last one (never stored)
+            xp[i] = a.X + (int64_t)b * a.strideX + (int64_t)min(i, a.NT - 1) * a.KT * TILE_U4 + lane;
+    }
     const uint4* wp = a.W + (int64_t)b * a.strideW + (int64_t)rt * a.KT * TILE_U4 + lane;
 
-    typename Eng::Acc acc;
+    typename Eng::Acc acc[NTL];
 #pragma unroll
-    for (int v = 0; v < 16; v++) acc[v] = 0;
-    int pa = 0, pb = 0;
+    for (int i = 0; i < NTL; i++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) acc[i][v] = 0;
+    int pa = 0, pb[NTL];
+#pragma unroll
+    for (int i = 0; i < NTL; i++) pb[i] = 0;
 
-    // the wave's K range is short (K / KW) and requested four K-tiles at a time: the kernel lives
+    // the wave's K range is short (K / KW) and requested MAXT K-tiles at a time: the kernel lives
     // on memory-level parallelism
-    constexpr int MAXT = 4;
+    constexpr int MAXT = NTL == 1 ? 4 : 2;
     for (int kb = kt0; kb < kt1 || kb == kt0; kb += MAXT) {
-        uint4 xq[MAXT], wq[MAXT];
+        uint4 xq[MAXT][NTL], wq[MAXT];
         if (kb < kt1) {
 #pragma unroll
             for (int q = 0; q < MAXT; q++) {
                 const int64_t off = (int64_t)min(kb + q, kt1 - 1) * TILE_U4;
-                xq[q] = xp[off];
+#pragma unroll
+                for (int i = 0; i < NTL; i++) xq[q][i] = xp[i][off];
                 wq[q] = load_stream(wp + off);
             }
         }
         if (kb == kt0) {
             // clear the meeting area while the first loads are in flight: every wave gets here at
             // once, so this barrier costs next to nothing
-            for (int i = threadIdx.x; i < 16 * 64; i += NT) (&sAcc[0][0])[i] = 0;
-            if (threadIdx.x < 32) { sPb[threadIdx.x] = 0; sPa[threadIdx.x] = 0; }
+            for (int i = threadIdx.x; i < NTL * 16 * 64; i += NT) (&sAcc[0][0][0])[i] = 0;
+            if (threadIdx.x < 32) {
+                sPa[threadIdx.x] = 0;
+#pragma unroll
+                for (int i = 0; i < NTL; i++) sPb[i][threadIdx.x] = 0;
+            }
             __syncthreads();
         }
         if (kb < kt1) {
 #pragma unroll
             for (int q = 0; q < MAXT; q++) {
                 if (kb + q >= kt1) break;
-                pb += popc4(xq[q]);
                 pa += popc4(wq[q]);
 #pragma unroll
-                for (int s = 0; s < Eng::STEPS; s++) acc = Eng::mma(Eng::expand(xq[q], s), Eng::expand(wq[q], s), acc);
+                for (int i = 0; i < NTL; i++) pb[i] += popc4(xq[q][i]);
+#pragma unroll
+                for (int s = 0; s < Eng::STEPS; s++) {
+                    const typename Eng::Frag bw = Eng::expand(wq[q], s);
+#pragma unroll
+                    for (int i = 0; i < NTL; i++) acc[i] = Eng::mma(Eng::expand(xq[q][i], s), bw, acc[i]);
+                }
             }
         }
     }
 
     // ---- meet in LDS: integer adds of the accumulator rows that carry outputs ------------------------
-    pb += __shfl_xor(pb, 32);
     pa += __shfl_xor(pa, 32);
+#pragma unroll
+    for (int i = 0; i < NTL; i++) pb[i] += __shfl_xor(pb[i], 32);
     if (kt0 < kt1) {
 #pragma unroll
-        for (int v = 0; v < 16; v++) {
-            const int n = 8 * (v >> 2) + 4 * h + (v & 3);
-            if ((two ? (n & 15) : n) < a.N) atomicAdd(&sAcc[v][lane], Eng::to_int(acc, v));
+        for (int i = 0; i < NTL; i++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int n = 32 * i + 8 * (v >> 2) + 4 * h + (v & 3);
+                if ((two ? (n & 15) : n) < a.N) atomicAdd(&sAcc[i][v][lane], Eng::to_int(acc[i], v));
+            }
+        if (lane < 32) {
+            atomicAdd(&sPa[lane], pa);
+#pragma unroll
+            for (int i = 0; i < NTL; i++) atomicAdd(&sPb[i][lane], pb[i]);
         }
-        if (lane < 32) { atomicAdd(&sPb[lane], pb); atomicAdd(&sPa[lane], pa); }
     }
     __syncthreads();
 
@@ -207,22 +239,27 @@ __global__ __launch_bounds__(KW * 64) void gemm_skinny_splitk_kernel(const GemmA
     const int kbits = (int)a.K;
     const int nout = (int)a.N * 32;
     for (int o = threadIdx.x; o < nout; o += NT) {
-        const int n = o >> 5, c = o & 31;
-        const int v = 4 * (n >> 3) + (n & 3), hh = (n >> 2) & 1;      // accumulator slot of operand row n
-        const int d = sAcc[v][hh * 32 + c];
-        const int d2 = two ? sAcc[v + 8][hh * 32 + c] : 0;
+        const int n = o >> 5, c = o & 31, i = n >> 5, nl = n & 31;
+        const int v = 4 * (nl >> 3) + (nl & 3), hh = (nl >> 2) & 1;   // accumulator slot of operand row nl
+        const int d = sAcc[i][v][hh * 32 + c];
+        const int d2 = two ? sAcc[0][v + 8][hh * 32 + c] : 0;
         const int64_t m = (int64_t)rt * 32 + c;
-        const int val = skinny_value(mc, two, kbits, sPa[c], sPb[n], two ? sPb[n + 16] : 0, d, d2);
+        const int val = skinny_value(mc, two, kbits, sPa[c], sPb[i][nl], two ? sPb[0][nl + 16] : 0, d, d2);
         if (m < a.M) store_out(a, (int64_t)b * a.strideC + (int64_t)n * a.M, m, val);
     }
 }
 
-bool gemm_skinny_eligible(const GemmArgs& a)
+// Shapes the skinny kernels take: one activation tile row always; up to four when the general
+// kernel's 64 x 128 output tiles would number fewer than the compute units and K is long enough
+// for the split to pay for the meeting in LDS.
+bool gemm_skinny_shape(int planes, int64_t batch, int64_t M, int64_t N, int64_t K)
 {
-    return a.mc.planes == 2 ? a.N <= 16 : a.N <= 32;
+    if (planes == 2) return N <= 16;
+    if (N <= 32) return true;
+    return N <= 128 && K >= 2048 && batch * cdiv(N, 64) * cdiv(M, 128) < 256;
 }
 
-template <typename Eng>
+template <typename Eng, int NTL>
 static int launch_splitk(const GemmArgs& a, hipStream_t st)
 {
     const int64_t blocks = (int64_t)a.batch * a.MT;
@@ -232,11 +269,19 @@ static int launch_splitk(const GemmArgs& a, hipStream_t st)
     int kw = 1;
     while (kw < 8 && (kw < a.splitK || blocks * kw < 4096) && kw * 2 <= a.KT) kw *= 2;
     const dim3 g((unsigned)blocks);
-    if (kw == 1) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 1>), g, dim3(64), 0, st, a);
-    else if (kw == 2) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 2>), g, dim3(128), 0, st, a);
-    else if (kw == 4) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 4>), g, dim3(256), 0, st, a);
-    else hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 8>), g, dim3(512), 0, st, a);
+    if (kw == 1) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 1, NTL>), g, dim3(64), 0, st, a);
+    else if (kw == 2) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 2, NTL>), g, dim3(128), 0, st, a);
+    else if (kw == 4) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 4, NTL>), g, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 8, NTL>), g, dim3(512), 0, st, a);
     return check_launch("gemm_skinny");
+}
+
+template <typename Eng>
+static int launch_splitk_n(const GemmArgs& a, hipStream_t st)
+{
+    if (a.NT <= 1) return launch_splitk<Eng, 1>(a, st);
+    if (a.NT == 2) return launch_splitk<Eng, 2>(a, st);
+    return launch_splitk<Eng, 4>(a, st);
 }
 
 template <typename Eng, int RT>
@@ -254,9 +299,11 @@ int launch_gemm_skinny(const GemmArgs& a, hipStream_t st, bool fp4)
     // Enough row tiles for about four waves on every SIMD: no K split needed (the result does not
     // depend on it).  Two row tiles per wave share one expansion of the activation tiles.
     const int64_t row_tiles = (int64_t)a.batch * a.MT;
-    if (row_tiles >= 8192) return fp4 ? launch_stream<EngF4, 2>(a, st) : launch_stream<EngI8, 2>(a, st);
-    if (row_tiles >= 4096) return fp4 ? launch_stream<EngF4, 1>(a, st) : launch_stream<EngI8, 1>(a, st);
-    return fp4 ? launch_splitk<EngF4>(a, st) : launch_splitk<EngI8>(a, st);
+    if (a.NT <= 1) {
+        if (row_tiles >= 8192) return fp4 ? launch_stream<EngF4, 2>(a, st) : launch_stream<EngI8, 2>(a, st);
+        if (row_tiles >= 4096) return fp4 ? launch_stream<EngF4, 1>(a, st) : launch_stream<EngI8, 1>(a, st);
+    }
+    return fp4 ? launch_splitk_n<EngF4>(a, st) : launch_splitk_n<EngI8>(a, st);
 }
 
 }  // namespace bgemm

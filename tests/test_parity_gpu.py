@@ -111,7 +111,8 @@ def test_pack_strided_and_unaligned(oracle):
 
 # ------------------------------------------------------------------ packed GEMM, small and ragged
 SMALL = [(1, 1, 1), (8, 5, 32), (33, 7, 40), (32, 32, 128), (10, 3, 784), (64, 1, 256), (65, 17, 300),
-         (130, 70, 1000), (256, 256, 512), (40, 200, 2304)]
+         (130, 70, 1000), (256, 256, 512), (40, 200, 2304),
+         (260, 70, 2500), (100, 40, 2304), (33, 128, 4096)]      # two to four activation tile rows, K split in the block
 
 
 @pytest.mark.parametrize("variant", VARIANTS)
