@@ -164,6 +164,74 @@ def bench_c4(steps, warmup, N, splitK, variant=0, copies=64):
             "ms_eager_launch": ms_eager, "gbs": bytes_alg / ms / 1e6, "ops": ops, "bytes": bytes_alg, "bit_exact": ok}
 
 
+def bench_c4_batched(steps, N, B=64):
+    """The same decode-shape BWTA linear over B weight matrices in ONE launch (the layers of a model,
+    a set of experts): 361 MB of weights stream through once, so the launch is long enough to show the
+    bandwidth the kernel sustains rather than the latency of one 5.6 MB launch."""
+    import torch
+    import lowbit_kernel as lk
+    dev = torch.device("cuda:0")
+    M, K = 11008, 4096
+    g = torch.Generator(device=dev).manual_seed(4100 + N)
+    t = torch.randint(0, 4, (N, K), generator=g, device=dev)
+    x16 = torch.where(t == 0, -1.0, torch.where(t == 3, 1.0, 0.0)).to(torch.half)
+    xt = lk.pack_ternary(x16)
+    words = M * K // 32
+    wdata = torch.randint(-2 ** 31, 2 ** 31 - 1, (B, words), generator=g, device=dev, dtype=torch.int32)
+    wb = lk.PackedBits(wdata, None, B, M, K)
+    out = torch.empty((B, N, M), dtype=torch.int32, device=dev)
+    fn = lambda i: lk.bgemm_packed_forward(wb, xt, lk.MODE_BWTA, torch.int32, 1, 0, out=out)
+    ms = time_gpu_graph(fn, 4, 2, max(5, steps // 40))
+    # parity of three of the matrices against the fp32 closed form on unpacked bits
+    ok = True
+    for b in (0, B // 2, B - 1):
+        w_logical = lk.logical_from_tiled(lk.PackedBits(wdata[b:b + 1], None, 1, M, K))
+        shifts = torch.arange(31, -1, -1, device=dev, dtype=torch.int32)
+        bits = ((w_logical.unsqueeze(-1) >> shifts) & 1).reshape(M, K)
+        want = (torch.sign(x16.float()) @ (1 - 2 * bits).float().T).to(torch.int32)
+        ok = ok and bool(torch.equal(out[b], want))
+    ops = 2.0 * B * M * N * K
+    bytes_alg = B * (M * K / 8 + 4.0 * M * N) + 2 * N * K / 8
+    return {"name": "C4 batched: %d x BWTA W[11008,4096] N=%d in one launch" % (B, N), "ms": ms, "tops": ops / ms / 1e9,
+            "gbs": bytes_alg / ms / 1e6, "ops": ops, "bytes": bytes_alg, "bit_exact": ok}
+
+
+def bench_floor():
+    """What the hardware allows a kernel of the decode path's shape: the cost of launching an empty kernel,
+    of reading one cold 5.6 MB buffer (the packed W[11008,4096]), and the bandwidth a plain read sustains."""
+    import ctypes
+    import torch
+    so = os.path.join(ROOT, "bgemm-cuda_amd", "libbgemm_membench.so")
+    L = ctypes.CDLL(so)
+    p, i64, ci = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+    L.bgemm_membench_empty.argtypes = [ci, ci, p, p]
+    L.bgemm_membench_read.argtypes = [p, i64, ci, ci, p, p]
+    dev = torch.device("cuda:0")
+    nbytes, copies = 11008 * 4096 // 8, 64
+    buf = torch.ones(copies * nbytes // 4, dtype=torch.int32, device=dev)
+    scratch = torch.zeros(64, dtype=torch.int32, device=dev)
+    st = lambda: torch.cuda.current_stream().cuda_stream
+    res = {}
+    res["empty_kernel_us"] = 1e3 * time_gpu_graph(
+        lambda i: L.bgemm_membench_empty(344, 512, scratch.data_ptr(), st()), 64, 2, 20)
+    best = None
+    for blocks, threads in ((512, 512), (1024, 256), (1024, 512), (2048, 256)):
+        us = 1e3 * time_gpu_graph(lambda i: L.bgemm_membench_read(buf.data_ptr() + (i % copies) * nbytes, nbytes, blocks,
+                                                                  threads, scratch.data_ptr(), st()), copies, 2, 20)
+        best = us if best is None else min(best, us)
+    res["cold_read_5p6MB_us"] = best
+    res["cold_read_5p6MB_gbs"] = nbytes / best / 1e3
+    best = None
+    for blocks, threads in ((2048, 512), (4096, 512), (8192, 512)):
+        us = 1e3 * time_gpu_graph(lambda i: L.bgemm_membench_read(buf.data_ptr(), copies * nbytes, blocks, threads,
+                                                                  scratch.data_ptr(), st()), 4, 2, 10)
+        best = us if best is None else min(best, us)
+    res["sustained_read_361MB_us"] = best
+    res["sustained_read_gbs"] = copies * nbytes / best / 1e3
+    res["sustained_read_frac_of_8TBs"] = res["sustained_read_gbs"] / HBM_PEAK_GBS
+    return res
+
+
 def bench_c3(steps, warmup, variant=0):
     """192 x ([512,512] {0,1} x [512,64] {-1,1}) -> int32 [192,512,64]."""
     import torch
@@ -231,6 +299,9 @@ def run_extra(which):
             for sk in (1, 8):
                 extra.append(bench_c4(2000, 200, N, sk))
                 log(json.dumps(extra[-1]))
+        for N in (1, 4, 16):
+            extra.append(bench_c4_batched(400, N))
+            log(json.dumps(extra[-1]))
     if which in ("c3", "all"):
         extra.append(bench_c3(200, 20))
         log(json.dumps(extra[-1]))
@@ -259,6 +330,8 @@ def main():
     ap.add_argument("--only", choices=["c2", "c3", "c4", "sweep"], help="time just that configuration (for profiling)")
     ap.add_argument("--variant", type=int, default=0, help="0 auto, 1 VALU, 2 MFMA int8, 3 MFMA fp4")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--floor", action="store_true",
+                    help="print the hardware floors for the decode shape (empty launch, cold 5.6 MB read, sustained read)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run a 256 MiB device-to-device copy (known traffic, for scaling rocprof counters)")
     args = ap.parse_args()
@@ -276,6 +349,9 @@ def main():
         dst = torch.empty_like(src)
         ms = time_gpu(lambda i: dst.copy_(src), 2, 5)
         log("calibration copy: 256 MiB read + 256 MiB written per launch, %.4f ms" % ms)
+    if args.floor:
+        print(json.dumps({"floor": bench_floor()}), flush=True)
+        return
     if args.only:
         print(json.dumps({"configs": run_extra(args.only)}), flush=True)
         return

@@ -7,6 +7,9 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 SO = os.path.join(HERE, "libbgemm_mi355x.so")
 SOURCES = ["api.hip", "pack.hip", "gemm_mfma.hip", "gemm_valu.hip", "gemm_skinny.hip"]
+# measurement probes for bench.py --floor, kept out of the library proper
+MEMBENCH_SO = os.path.join(HERE, "libbgemm_membench.so")
+MEMBENCH_SOURCE = "membench.hip"
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
          # keep the compiler from forming packed-fp32 VALU ops
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
@@ -17,9 +20,10 @@ def build(verbose=True):
     objs = []
     procs = []
     os.makedirs(os.path.join(HERE, "build"), exist_ok=True)
-    for s in SOURCES:
+    for s in SOURCES + [MEMBENCH_SOURCE]:
         o = os.path.join(HERE, "build", s.replace(".hip", ".o"))
-        objs.append(o)
+        if s != MEMBENCH_SOURCE:
+            objs.append(o)
         cmd = [hipcc] + FLAGS + ["-c", os.path.join(CSRC, s), "-o", o]
         if verbose:
             print(" ".join(cmd), flush=True)
@@ -28,6 +32,11 @@ def build(verbose=True):
         if p.wait() != 0:
             raise RuntimeError("hipcc failed on %s" % s)
     cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", SO] + objs
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", MEMBENCH_SO,
+           os.path.join(HERE, "build", MEMBENCH_SOURCE.replace(".hip", ".o"))]
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)
