@@ -40,18 +40,38 @@ def _linear_grads(grad_out, x_sign, w_sign):
     return grad_x, grad_w
 
 
+def _batched_packed(x_rows, w_rows, mode):
+    """x_rows [..., N, K], w_rows [..., M, K] with equal leading dimensions -> fp16 [..., N, M]: one launch
+    over all leading dimensions on the batched packed entry point (no per-matrix Python loop)."""
+    lead = x_rows.shape[:-2]
+    if w_rows.shape[:-2] != lead:
+        raise ValueError("leading dimensions differ: %s vs %s" % (tuple(x_rows.shape), tuple(w_rows.shape)))
+    xp = lowbit_kernel.pack_sign(x_rows.reshape(-1, *x_rows.shape[-2:]))
+    wp = lowbit_kernel.pack_sign(w_rows.reshape(-1, *w_rows.shape[-2:]))
+    out = lowbit_kernel.bgemm_packed_forward(wp, xp, mode, torch.half)
+    return out.reshape(*lead, x_rows.shape[-2], w_rows.shape[-2])
+
+
 class bgemm_matmul(torch.autograd.Function):
-    """matA [.., N, K] @ matB [K, M] with both operands binarised by sign (bgemm_linear.py:9-42)."""
+    """matA [.., N, K] @ matB [K, M] with both operands binarised by sign (bgemm_linear.py:9-42).
+    A matB with leading dimensions ([B, H, K, M], as K^T in attention) is a batched matmul."""
 
     @staticmethod
     def forward(ctx, matA, matB, instruction='xor'):
         matA, matB = matA.to(torch.half), matB.to(torch.half)
         ctx.save_for_backward(matA, matB)
-        return _kernel_2d(matA, matB.transpose(-1, -2).contiguous(), _instr(instruction))
+        bt = matB.transpose(-1, -2).contiguous()
+        if matB.dim() > 2:
+            mode = lowbit_kernel.MODE_AND if instruction == 'and' else lowbit_kernel.MODE_XOR
+            return _batched_packed(matA, bt, mode)
+        return _kernel_2d(matA, bt, _instr(instruction))
 
     @staticmethod
     def backward(ctx, grad_output):
         matA, matB = ctx.saved_tensors
+        if matB.dim() > 2:
+            g = grad_output.to(matA.dtype)
+            return g @ matB.sign().transpose(-1, -2), matA.sign().transpose(-1, -2) @ g, None
         grad_a, grad_bt = _linear_grads(grad_output, matA.sign(), matB.sign().transpose(-1, -2))
         return grad_a, grad_bt.transpose(-1, -2), None
 
@@ -65,6 +85,10 @@ class bgemm_attn_matmul(torch.autograd.Function):
         input1, input2 = input1.to(torch.half), input2.to(torch.half)
         ctx.save_for_backward(input1, input2)
         vt = input2.transpose(-1, -2).contiguous()
+        if input1.dim() > 2:
+            # [B, H, S_q, S_k] x [B, H, S_k, d]: attn stays as it lies (activation side, {0,1}), only the
+            # small value operand is transposed; the result comes out as [B, H, S_q, d] directly
+            return _batched_packed(input1, vt, lowbit_kernel.MODE_ATTN_X)
         return lowbit_kernel.bgemm_linear_forward_cuda(vt, input1, 1, lowbit_kernel.ATTN_MM).T
 
     @staticmethod
@@ -74,7 +98,7 @@ class bgemm_attn_matmul(torch.autograd.Function):
         a01 = torch.where(a01 == 0, torch.ones_like(a01), a01)     # as the reference does (:70-71)
         v = value.sign()
         g = grad_output.to(v.dtype)
-        return (g @ v.T) / 2, a01.T @ g, None
+        return (g @ v.transpose(-1, -2)) / 2, a01.transpose(-1, -2) @ g, None
 
 
 class bgemm_linear(torch.autograd.Function):

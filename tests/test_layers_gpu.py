@@ -37,6 +37,33 @@ def test_bgemm_matmul_and_attn_matmul():
     assert tuple(out.shape) == (128, 64) and torch.equal(out.float(), want.half().float())
 
 
+def test_batched_attention_pair_bert_shape():
+    """Q K^T then A V over [batch, heads, seq, head_dim] in one launch each (the reference is 2-D only)."""
+    torch.manual_seed(5)
+    B, H, S, D = 2, 12, 512, 64
+    q, k, v = (torch.randn(B, H, S, D, device=DEV) for _ in range(3))
+    scores = bl.bgemm_matmul.apply(q, k.transpose(-1, -2))
+    pm = lambda t: torch.where(torch.signbit(t.half()), -1.0, 1.0)
+    want = torch.matmul(pm(q), pm(k).transpose(-1, -2))
+    assert scores.dtype == torch.half and tuple(scores.shape) == (B, H, S, S)
+    assert torch.equal(scores.float(), want.half().float())
+    attn = torch.randn(B, H, S, S, device=DEV)                    # zero-centred: "1" where the sign bit is clear
+    ctx = bl.bgemm_attn_matmul.apply(attn, v)
+    # operands are read off the sign bit, as the kernel does: among millions of halves a few round to +-0.0,
+    # which torch.sign would map to 0
+    want = torch.matmul((~torch.signbit(attn.half())).float(), torch.where(torch.signbit(v.half()), -1.0, 1.0))
+    assert tuple(ctx.shape) == (B, H, S, D) and torch.equal(ctx.float(), want.half().float())
+    # each slice equals the 2-D call
+    assert torch.equal(ctx[1, 3], bl.bgemm_attn_matmul.apply(attn[1, 3], v[1, 3]))
+    # gradients flow with batched shapes
+    qg = q.clone().requires_grad_(True)
+    kt = k.transpose(-1, -2).clone().requires_grad_(True)
+    bl.bgemm_matmul.apply(qg, kt).float().sum().backward()
+    assert qg.grad.shape == q.shape and kt.grad.shape == kt.shape
+    g = torch.ones(S, S, device=DEV)
+    assert torch.allclose(qg.grad[0, 0].float(), g @ k[0, 0].half().sign().float(), atol=0)   # backward uses torch.sign
+
+
 def test_bgemm_linear_backward_shapes_and_values():
     torch.manual_seed(2)
     x = torch.randn(32, 128, device=DEV, requires_grad=True)
