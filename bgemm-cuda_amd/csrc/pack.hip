@@ -1,6 +1,8 @@
-// fp16 -> bit-plane packing and logical <-> tiled re-layout.  HBM-bound byte work:
-// one 16-byte load per lane, eight sign (and nonzero) bits extracted per lane, four
-// lanes merged into a 32-bit word, 16-byte-contiguous stores into the tiled layout.
+// fp16 / fp32 -> bit-plane packing and logical <-> tiled re-layout.  HBM-bound byte work.
+// Tiled output: a wave packs one 32-row x 256-bit tile, with all of its 16-byte loads in
+// flight at once; each lane turns eight elements into a byte of sign (and nonzero) bits, the
+// bytes are put in tile order through LDS, and the tile leaves as one 16-byte store per lane.
+// Logical output (the reference's row-major words): a wave packs 512 elements of one row.
 #include "common.h"
 #include <string.h>
 
@@ -29,7 +31,7 @@ __device__ __forceinline__ uint16_t half_bits(const float f)
     return __half_as_ushort(__float2half_rn(f));
 }
 
-// One wave packs 512 consecutive K elements of one row (16 words).
+// Logical output: one wave packs 512 consecutive K elements of one row (16 words).
 __device__ __forceinline__ void pack_wave(const PackJob& j, const int64_t gw, const int lane)
 {
     const int64_t row = gw / j.nseg, seg = gw - row * j.nseg;
@@ -93,13 +95,118 @@ __device__ __forceinline__ void pack_wave(const PackJob& j, const int64_t gw, co
     }
 }
 
+// Sign (and nonzero) bits of eight fp16 bit patterns, element e at bit 7 - e.
+__device__ __forceinline__ void bits8(const uint16_t (&h)[8], uint32_t& sg, uint32_t& nz)
+{
+    sg = 0; nz = 0;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        sg |= (uint32_t)(h[e] >> 15) << (7 - e);
+        nz |= (uint32_t)((h[e] & 0x7fff) != 0) << (7 - e);
+    }
+}
+
+// One wave packs tile (rt, kt) = gw of the tiled layout.  Lane (c = lane & 31, lane >> 5) takes
+// elements 256 kt + 8c .. + 7 of rows 2 jj + (lane >> 5), jj = 0..15.  lds: 2 KiB of this wave's own.
+__device__ __forceinline__ void pack_tile(const PackJob& j, const int64_t gw, const int lane, unsigned char* lds)
+{
+    const int64_t rt = gw / j.KT, kt = gw - rt * j.KT;
+    if (rt * TILE_ROWS >= j.rows_out) return;              // whole wave leaves together
+    const int c = lane & 31, rsub = lane >> 5;
+    const int64_t row0 = rt * TILE_ROWS + rsub, k0 = kt * TILE_KBITS + 8 * c;
+    const bool ternary = j.mode & 1, f32 = j.mode & 4;
+    // byte of (row r, lane c) inside the tile: word c >> 2 of the row goes to slot h * 32 + r, position q;
+    // the row's first element is the word's most significant bit, i.e. byte 3 of the little-endian word
+    const int byte0 = (((c >> 4) * 32) * 4 + ((c >> 2) & 3)) * 4 + (3 - (c & 3));
+    float zf = 0.f;
+    if (j.zp) zf = f32 ? *reinterpret_cast<const float*>(j.zp) : __half2float(*reinterpret_cast<const __half*>(j.zp));
+    auto emit = [&](const int r, uint16_t (&h)[8], const int valid) {
+        if (j.zp && !f32) {
+#pragma unroll
+            for (int e = 0; e < 8; e++)
+                if (e < valid) h[e] = half_bits(__fsub_rn(__half2float(__ushort_as_half(h[e])), zf));
+        }
+        uint32_t sg, nz;
+        bits8(h, sg, nz);
+        lds[byte0 + r * 16] = (unsigned char)(ternary ? nz : sg);
+        if (ternary) lds[1024 + byte0 + r * 16] = (unsigned char)(sg & nz);
+    };
+    // the whole tile lies inside the source and every row is 16-byte aligned: plain vector loads, all in flight
+    const int64_t esz = f32 ? 4 : 2;
+    const bool interior = rt * TILE_ROWS + TILE_ROWS <= j.rows && kt * TILE_KBITS + TILE_KBITS <= j.K &&
+                          ((((uintptr_t)j.src) | (uintptr_t)(j.ld * esz)) & 15) == 0;
+    if (interior && !f32) {
+        const uint16_t* p = reinterpret_cast<const uint16_t*>(j.src) + row0 * j.ld + k0;
+        uint4 raw[16];
+#pragma unroll
+        for (int jj = 0; jj < 16; jj++) raw[jj] = *reinterpret_cast<const uint4*>(p + (int64_t)(2 * jj) * j.ld);
+#pragma unroll
+        for (int jj = 0; jj < 16; jj++) {
+            const uint4 v = raw[jj];
+            uint16_t h[8] = {(uint16_t)(v.x & 0xffff), (uint16_t)(v.x >> 16), (uint16_t)(v.y & 0xffff), (uint16_t)(v.y >> 16),
+                             (uint16_t)(v.z & 0xffff), (uint16_t)(v.z >> 16), (uint16_t)(v.w & 0xffff), (uint16_t)(v.w >> 16)};
+            emit(2 * jj + rsub, h, 8);
+        }
+    } else if (interior) {
+        const float* p = reinterpret_cast<const float*>(j.src) + row0 * j.ld + k0;
+#pragma unroll
+        for (int g = 0; g < 2; g++) {
+            float4 lo[8], hi[8];
+#pragma unroll
+            for (int jj = 0; jj < 8; jj++) {
+                const float* q = p + (int64_t)(2 * (8 * g + jj)) * j.ld;
+                lo[jj] = *reinterpret_cast<const float4*>(q);
+                hi[jj] = *reinterpret_cast<const float4*>(q + 4);
+            }
+#pragma unroll
+            for (int jj = 0; jj < 8; jj++) {
+                const float f[8] = {lo[jj].x, lo[jj].y, lo[jj].z, lo[jj].w, hi[jj].x, hi[jj].y, hi[jj].z, hi[jj].w};
+                uint16_t h[8];
+#pragma unroll
+                for (int e = 0; e < 8; e++) h[e] = half_bits(j.zp ? __fsub_rn(f[e], zf) : f[e]);
+                emit(2 * (8 * g + jj) + rsub, h, 8);
+            }
+        }
+    } else {
+        // edge tiles and unaligned sources: element loads, rows and columns past the end read as +0.0
+        for (int jj = 0; jj < 16; jj++) {
+            const int64_t row = row0 + 2 * jj;
+            uint16_t h[8];
+#pragma unroll
+            for (int e = 0; e < 8; e++) h[e] = 0;
+            int valid = 0;
+            if (row < j.rows && k0 < j.K) {
+                valid = (int)(j.K - k0 < 8 ? j.K - k0 : 8);
+                if (f32) {
+                    const float* q = reinterpret_cast<const float*>(j.src) + row * j.ld + k0;
+#pragma unroll
+                    for (int e = 0; e < 8; e++) if (e < valid) h[e] = half_bits(j.zp ? __fsub_rn(q[e], zf) : q[e]);
+                } else {
+                    const uint16_t* q = reinterpret_cast<const uint16_t*>(j.src) + row * j.ld + k0;
+#pragma unroll
+                    for (int e = 0; e < 8; e++) if (e < valid) h[e] = q[e];
+                }
+            }
+            emit(2 * jj + rsub, h, valid);
+        }
+    }
+    __builtin_amdgcn_wave_barrier();       // the tile was written by this wave alone: LDS keeps its order
+    reinterpret_cast<uint4*>(j.dst0)[gw * TILE_U4 + lane] = reinterpret_cast<const uint4*>(lds)[lane];
+    if (ternary) reinterpret_cast<uint4*>(j.dst1)[gw * TILE_U4 + lane] = reinterpret_cast<const uint4*>(lds + 1024)[lane];
+}
+
 // Up to two operands per launch (the fp16 entry point packs weights and activations together).
 __global__ __launch_bounds__(256) void pack_f16_kernel(const PackJob j0, const PackJob j1)
 {
-    const int lane = threadIdx.x & 63;
-    const int64_t gw = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (gw < j0.waves) pack_wave(j0, gw, lane);
-    else if (gw - j0.waves < j1.waves) pack_wave(j1, gw - j0.waves, lane);
+    __shared__ __align__(16) unsigned char s_tile[4][2048];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int64_t gw = (int64_t)blockIdx.x * 4 + wave;
+    const bool first = gw < j0.waves;
+    const PackJob& j = first ? j0 : j1;
+    if (!first) gw -= j0.waves;
+    if (gw >= j.waves) return;
+    if (j.mode & 2) pack_wave(j, gw, lane);
+    else pack_tile(j, gw, lane, s_tile[wave]);
 }
 
 // dir 0: logical -> tiled (zero padding), dir 1: tiled -> logical.  One thread per tiled word.
@@ -132,7 +239,7 @@ static int make_job(PackJob* j, const void* src, int64_t rows, int64_t K, int64_
     j->KT = k_tiles(K); j->Kw = cdiv(K, 32);
     j->rows_out = (mode & 2) ? rows : row_tiles(rows) * TILE_ROWS;
     j->nseg = cdiv(j->KT * TILE_KBITS, 512);
-    j->waves = j->rows_out * j->nseg;
+    j->waves = (mode & 2) ? j->rows_out * j->nseg : row_tiles(rows) * j->KT;
     return BGEMM_OK;
 }
 
