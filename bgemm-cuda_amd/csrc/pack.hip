@@ -15,7 +15,8 @@ __host__ __device__ static inline int64_t tiled_word_offset(int64_t row, int64_t
     return ((rt * KT + kt) * TILE_U4 + h * 32 + r) * 4 + q;
 }
 
-// One operand to pack.  mode bit0: also write the (sign & nonzero) plane and make plane 0 the
+// One operand to pack.  mode bit3: tiled output written by the row-segment waves (small operands:
+// sixteen times as many, shorter waves).  mode bit0: also write the (sign & nonzero) plane and make plane 0 the
 // nonzero plane.  mode bit1: write the logical layout instead of the tiled one.  mode bit2: the
 // source is fp32 (rounded to fp16 first, as the layers' `.to(torch.half)` does).
 // zp: device scalar of the source type subtracted before that rounding, or null.
@@ -205,7 +206,7 @@ __global__ __launch_bounds__(256) void pack_f16_kernel(const PackJob j0, const P
     const PackJob& j = first ? j0 : j1;
     if (!first) gw -= j0.waves;
     if (gw >= j.waves) return;
-    if (j.mode & 2) pack_wave(j, gw, lane);
+    if (j.mode & (2 | 8)) pack_wave(j, gw, lane);
     else pack_tile(j, gw, lane, s_tile[wave]);
 }
 
@@ -239,7 +240,9 @@ static int make_job(PackJob* j, const void* src, int64_t rows, int64_t K, int64_
     j->KT = k_tiles(K); j->Kw = cdiv(K, 32);
     j->rows_out = (mode & 2) ? rows : row_tiles(rows) * TILE_ROWS;
     j->nseg = cdiv(j->KT * TILE_KBITS, 512);
-    j->waves = (mode & 2) ? j->rows_out * j->nseg : row_tiles(rows) * j->KT;
+    // a wave per tile streams best, but an operand of a few hundred tiles would leave most SIMDs without one
+    if (!(mode & 2) && row_tiles(rows) * j->KT < 2048) j->mode |= 8;
+    j->waves = (j->mode & (2 | 8)) ? j->rows_out * j->nseg : row_tiles(rows) * j->KT;
     return BGEMM_OK;
 }
 

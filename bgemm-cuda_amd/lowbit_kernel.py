@@ -9,6 +9,9 @@ else here is the packed-operand surface the reference only stubbed
 All work is enqueued on the current torch stream through the C ABI in
 include/bgemm_mi355x.h; torch supplies device memory and streams only.
 """
+import contextlib
+import struct
+
 import torch
 
 import _lib as _b
@@ -18,11 +21,33 @@ from _lib import (MODE_AND, MODE_XOR, MODE_ATTN, MODE_BWTA, MODE_ATTN_X, OUT_I32
 AND_POP, XOR_POP, ATTN_MM = 0, 1, 2   # lowbit_kernel/csrc/include/configs.h:70-72
 
 __all__ = ["bgemm_linear_forward_cuda", "binary_weight_prepacking", "pack_sign", "pack_ternary",
-           "bgemm_packed_forward", "PackedBits", "AND_POP", "XOR_POP", "ATTN_MM"]
+           "bgemm_packed_forward", "PackedBits", "save_packed", "load_packed", "AND_POP", "XOR_POP", "ATTN_MM"]
+
+
+_NULL_CTX = contextlib.nullcontext()
 
 
 def _stream():
     return torch.cuda.current_stream().cuda_stream
+
+
+def _on(device):
+    """Context that makes `device` current; free when it already is (the usual case)."""
+    if device.index is None or device.index == torch.cuda.current_device():
+        return _NULL_CTX
+    return torch.cuda.device(device)
+
+
+# workspace needs per (mode, batch, M, N, K, splitK, variant): two C calls saved per launch
+_ws_needs = {}
+
+
+def _split_k_needs(L, key):
+    need = _ws_needs.get(key)
+    if need is None:
+        need = (L.bgemm_packed_workspace_bytes(*key), L.bgemm_packed_counter_bytes(*key))
+        _ws_needs[key] = need
+    return need
 
 
 def _need_cuda(t, name):
@@ -96,7 +121,7 @@ def _pack(x, ternary, zero_point=None):
     words = L.bgemm_tiled_words(rows, K)
     d0 = torch.empty((batch, words), dtype=torch.int32, device=x.device)
     d1 = torch.empty_like(d0) if ternary else None
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         st = _stream()
         if batch > 1 and rows % 32 == 0:
             # whole tiles per matrix: the batch is one tall matrix in the tiled layout
@@ -139,7 +164,7 @@ def binary_weight_prepacking(weights):
     w = weights.to(torch.half).contiguous()
     OC, IC = w.shape
     out = torch.empty((OC, (IC + 31) // 32), dtype=torch.int32, device=w.device)
-    with torch.cuda.device(w.device):
+    with _on(w.device):
         _b.check(_b.lib().bgemm_pack_sign_f16_logical(w.data_ptr(), OC, IC, IC, out.data_ptr(), _stream()))
     return out
 
@@ -151,7 +176,7 @@ def tile_from_logical(logical, K):
     R = logical.shape[0]
     L = _b.lib()
     d0 = torch.empty((1, L.bgemm_tiled_words(R, K)), dtype=torch.int32, device=logical.device)
-    with torch.cuda.device(logical.device):
+    with _on(logical.device):
         _b.check(L.bgemm_tile_from_logical(logical.data_ptr(), R, K, d0.data_ptr(), _stream()))
     return PackedBits(d0, None, 1, R, K)
 
@@ -160,7 +185,7 @@ def logical_from_tiled(packed, plane=0):
     """PackedBits (batch 1) -> int32 ``[R, ceil(K/32)]`` in the logical format."""
     src = packed.data if plane == 0 else packed.data2
     out = torch.empty((packed.rows, (packed.K + 31) // 32), dtype=torch.int32, device=src.device)
-    with torch.cuda.device(src.device):
+    with _on(src.device):
         _b.check(_b.lib().bgemm_logical_from_tiled(src.data_ptr(), packed.rows, packed.K, out.data_ptr(), _stream()))
     return out
 
@@ -203,11 +228,12 @@ def bgemm_packed_forward(w, x, mode=MODE_XOR, out_dtype=torch.int32, splitK=1, v
     if out is None:
         out = torch.empty((batch, N, M), dtype=out_dtype, device=dev)
     L = _b.lib()
-    with torch.cuda.device(dev):
+    with _on(dev):
         ws = cnt = None
         if splitK > 1:
-            ws, cnt = _split_k_buffers(L.bgemm_packed_workspace_bytes(mode, batch, M, N, K, splitK, variant),
-                                       L.bgemm_packed_counter_bytes(mode, batch, M, N, K, splitK, variant), dev)
+            part_bytes, counter_bytes = _split_k_needs(L, (mode, batch, M, N, K, splitK, variant))
+            if part_bytes:
+                ws, cnt = _split_k_buffers(part_bytes, counter_bytes, dev)
         args = (mode, w.data.data_ptr(), x.data.data_ptr(), x.data2.data_ptr() if x.ternary else None,
                 out.data_ptr(), kind, batch, M, N, K,
                 w.words if w.batch > 1 else 0, x.words if x.batch > 1 else 0, N * M, splitK, variant,
@@ -240,11 +266,61 @@ def bgemm_linear_forward_cuda(in_feats, weights, splitK=1, INSTR=1):
     M = w.shape[0]
     out = torch.empty((N, M), dtype=torch.half, device=x.device)
     L = _b.lib()
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         ws = torch.empty(max(L.bgemm_f16_workspace_bytes(M, N, K, splitK), 1), dtype=torch.uint8, device=x.device)
         _b.check(L.bgemm_f16_forward(w.data_ptr(), x.data_ptr(), out.data_ptr(), M, N, K,
                                      ws.data_ptr(), ws.numel(), int(splitK), int(INSTR), _stream()))
     return out
+
+
+# ---- prepacked operands on disk -----------------------------------------------------------------
+# The reference has no binary prepack format (its TODO list asks for one, README.md:25-33).  A file is
+# a 64-byte little-endian header followed by the tiled words of plane 0 and, for ternary operands,
+# plane 1: magic "BGEMMPK1", layout version (= the library's ABI version, which changes with the tiled
+# layout), planes, batch, rows, K, words per matrix.
+_PK_MAGIC = b"BGEMMPK1"
+_PK_HEADER = struct.Struct("<8sIIqqqq16x")
+
+
+def save_packed(path, packed):
+    """Writes a PackedBits (e.g. prepacked weights) to `path`."""
+    head = _PK_HEADER.pack(_PK_MAGIC, _b.ABI_VERSION, 2 if packed.ternary else 1, packed.batch, packed.rows,
+                           packed.K, packed.words)
+    with open(path, "wb") as f:
+        f.write(head)
+        f.write(packed.data.contiguous().cpu().numpy().tobytes())
+        if packed.ternary:
+            f.write(packed.data2.contiguous().cpu().numpy().tobytes())
+
+
+def read_packed_header(path):
+    """(planes, batch, rows, K, words) of a file written by save_packed; raises ValueError on anything else."""
+    with open(path, "rb") as f:
+        raw = f.read(_PK_HEADER.size)
+    if len(raw) != _PK_HEADER.size:
+        raise ValueError("%s: too short for a packed-operand header" % path)
+    magic, version, planes, batch, rows, K, words = _PK_HEADER.unpack(raw)
+    if magic != _PK_MAGIC:
+        raise ValueError("%s: not a packed-operand file" % path)
+    if version != _b.ABI_VERSION:
+        raise ValueError("%s: tiled layout version %d, this library reads %d: pack the weights again" %
+                         (path, version, _b.ABI_VERSION))
+    if planes not in (1, 2) or batch < 1 or rows < 1 or K < 1 or words != ((rows + 31) // 32) * ((K + 255) // 256) * 256:
+        raise ValueError("%s: inconsistent header" % path)
+    return planes, batch, rows, K, words
+
+
+def load_packed(path, device="cuda"):
+    """Reads a file written by save_packed back into a PackedBits on `device`."""
+    import numpy as np
+    planes, batch, rows, K, words = read_packed_header(path)
+    n = batch * words
+    arr = np.fromfile(path, dtype=np.int32, offset=_PK_HEADER.size)
+    if arr.size != planes * n:
+        raise ValueError("%s: %d words of payload, header says %d" % (path, arr.size, planes * n))
+    d0 = torch.from_numpy(arr[:n].reshape(batch, words).copy()).to(device)
+    d1 = torch.from_numpy(arr[n:].reshape(batch, words).copy()).to(device) if planes == 2 else None
+    return PackedBits(d0, d1, batch, rows, K)
 
 
 def _fp6_only(*_a, **_k):

@@ -135,3 +135,32 @@ def test_cpu_layers_match_reference_cpu_path(oracle):
     assert torch.equal(y2, oracle.cpu_path_linear(xs, ws) * el.sa * el.sw + el.bias)
     y2.sum().backward()
     assert el.weight.grad is not None and el.sa.grad is not None
+
+
+def test_packed_file_format_round_trip_and_rejects(tmp_path):
+    """The on-disk prepacked format is plain host code: header checks run without a GPU."""
+    import numpy as np
+    import torch
+    import lowbit_kernel as lk
+    rows, K = 40, 300
+    words = 2 * 2 * 256
+    rng = np.random.default_rng(3)
+    d0 = torch.from_numpy(rng.integers(-2 ** 31, 2 ** 31 - 1, (3, words), dtype=np.int64).astype(np.int32))
+    d1 = torch.from_numpy(rng.integers(-2 ** 31, 2 ** 31 - 1, (3, words), dtype=np.int64).astype(np.int32))
+    path = str(tmp_path / "w.bgpk")
+    lk.save_packed(path, lk.PackedBits(d0, d1, 3, rows, K))
+    assert lk.read_packed_header(path) == (2, 3, rows, K, words)
+    back = lk.load_packed(path, device="cpu")
+    assert back.batch == 3 and back.rows == rows and back.K == K and back.ternary
+    assert torch.equal(back.data, d0) and torch.equal(back.data2, d1)
+    raw = bytearray(open(path, "rb").read())
+    for mutate, what in ((lambda b: b.__setitem__(0, 0x58), "magic"), (lambda b: b.__setitem__(8, 99), "version"),
+                         (lambda b: b.__setitem__(slice(24, 32), (100).to_bytes(8, "little")), "rows vs words")):
+        bad = bytearray(raw)
+        mutate(bad)
+        open(path, "wb").write(bad)
+        with pytest.raises(ValueError):
+            lk.read_packed_header(path)
+    open(path, "wb").write(raw[:-4])          # truncated payload
+    with pytest.raises(ValueError):
+        lk.load_packed(path, device="cpu")

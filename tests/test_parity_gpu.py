@@ -405,3 +405,18 @@ def test_skinny_streaming_batched(B, M, N, K):
     variants = {v: lk.bgemm_packed_forward(wp, xp, MODE_XOR, torch.half, 1, v) for v in (VARIANT_MFMA, VARIANT_MFMA_F4)}
     for v, got in variants.items():
         assert torch.equal(got, want[MODE_XOR].half()), v
+
+
+def test_packed_file_round_trip_on_device(tmp_path):
+    """Weights prepacked once, written to disk, read back: same bits, same GEMM."""
+    rng = np.random.default_rng(77)
+    w, x = rand_f16(rng, 300, 1000), rand_f16(rng, 9, 1000)
+    wp, xt = lk.pack_sign(to_dev(w)), lk.pack_ternary(to_dev(x))
+    pw, px = str(tmp_path / "w.bgpk"), str(tmp_path / "x.bgpk")
+    lk.save_packed(pw, wp)
+    lk.save_packed(px, xt)
+    wp2, xt2 = lk.load_packed(pw, DEV), lk.load_packed(px, DEV)
+    assert torch.equal(wp2.data, wp.data) and torch.equal(xt2.data, xt.data) and torch.equal(xt2.data2, xt.data2)
+    a = lk.bgemm_packed_forward(wp, xt, MODE_BWTA, torch.int32)
+    b = lk.bgemm_packed_forward(wp2, xt2, MODE_BWTA, torch.int32)
+    assert torch.equal(a, b) and (a[0].cpu().numpy() == dense_ref(MODE_BWTA, w, x)).all()
