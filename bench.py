@@ -4,11 +4,11 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--all]
 
 A step is one pass of the hot path over one batch of synthetic input: one 8192^3
-{-1,1}x{-1,1} BGEMM on prepacked operands (BASELINE config 5, the compute-bound case the
+{-1,1}x{-1,1} BGEMM on prepacked operands (benchmark configuration 5, the compute-bound case the
 metric's target is quoted on), int32 output, operands resident in HBM before the timed
 region.  One JSON line goes to stdout; `value` is effective binary TOPS = 2*M*N*K / t
 (the reference drivers' own op count, lowbit_kernel/csrc/benchmark.cu:291).  With --all the
-line also carries the other BASELINE configurations (MLP forward, batched attention A x V,
+line also carries the other benchmark configurations (MLP forward, batched attention A x V,
 decode-shape BWTA) under "all_configs".
 """
 import argparse
@@ -292,7 +292,7 @@ def bench_c2(steps, warmup):
 
 
 def run_extra(which):
-    """The non-headline BASELINE configurations: 'c4' decode BWTA, 'c3' attention, 'c2' MLP, 'sweep'."""
+    """The non-headline benchmark configurations: 'c4' decode BWTA, 'c3' attention, 'c2' MLP, 'sweep'."""
     extra = []
     if which in ("c4", "all"):
         for N in (1, 4, 16):
@@ -326,7 +326,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--all", action="store_true", help="also time the other BASELINE configurations")
+    ap.add_argument("--all", action="store_true", help="also time the other benchmark configurations")
     ap.add_argument("--only", choices=["c2", "c3", "c4", "sweep"], help="time just that configuration (for profiling)")
     ap.add_argument("--variant", type=int, default=0, help="0 auto, 1 VALU, 2 MFMA int8, 3 MFMA fp4")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -373,7 +373,7 @@ def main():
         "ms_per_step": c5["ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "fp4" if fp4 else "int8",
         "data": "synthetic",
-        "config": {"workload": "BASELINE config 5: BGEMM M=N=K=8192, {-1,+1}x{-1,+1}, weights and activations "
+        "config": {"workload": "BASELINE.json config 5: BGEMM M=N=K=8192, {-1,+1}x{-1,+1}, weights and activations "
                                "prepacked (tiled bit layout), int32 output, splitK=1",
                    "arithmetic": ("1-bit operands expanded in registers to E2M1 (fp4) MFMA operands, fp32 accumulation "
                                   "of exact integers" if fp4 else

@@ -142,7 +142,7 @@ def test_elastic_module_matches_cpu_twin():
 
 
 def test_config2_mlp_forward_bitwise(oracle):
-    """BASELINE config 2: 784 -> 4096 -> 4096 -> 10, batch 128, fp16 outputs vs the CPU chain."""
+    """Benchmark configuration 2: 784 -> 4096 -> 4096 -> 10, batch 128, fp16 outputs vs the CPU chain."""
     g = torch.Generator().manual_seed(1002)
     dims = [784, 4096, 4096, 10]
     x = torch.randn(128, 784, generator=g).half()

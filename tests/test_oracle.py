@@ -142,7 +142,7 @@ def test_reference_call_rounds_large_sums(oracle):
 
 
 def test_config1_cpu_reference_path(oracle):
-    """BASELINE config 1: A[1024,1024] x B[1024,64], +-1 from a seed, vs fp32 torch.matmul."""
+    """Benchmark configuration 1: A[1024,1024] x B[1024,64], +-1 from a seed, vs fp32 torch.matmul."""
     import torch
     g = torch.Generator().manual_seed(1001)
     a_bits = torch.randint(0, 2, (1024, 1024), generator=g)

@@ -2,7 +2,7 @@
 
 Bar: bit-exact for int32 outputs; fp16 outputs equal the exact integer rounded to nearest
 even (tolerance 0 ulp).  Sizes the oracle finishes in seconds are compared element by element;
-BASELINE's full sizes are checked on sampled rows plus size-independent identities.
+the benchmark's full sizes are checked on sampled rows plus size-independent identities.
 """
 import json
 import os
@@ -144,7 +144,7 @@ def test_packed_golden_dense(golden_dir):
                 assert (got[0].cpu().numpy() == d["%s%d" % (nm, i)]).all(), (i, nm, variant)
 
 
-# ------------------------------------------------------------------ BASELINE configurations
+# ------------------------------------------------------------------ benchmark configurations
 def dense_ref(mode, w, x):
     """Closed forms in fp32 on the CPU (exact: K < 2^24); the reference drivers' own method."""
     a = torch.from_numpy((w.view(np.uint16) >> 15).astype(np.float32))
