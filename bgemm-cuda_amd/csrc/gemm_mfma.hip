@@ -18,7 +18,7 @@ __device__ const uint4 g_zero_tile[TILE_U4] = {};
 
 // Block = WGN x WGM waves, each wave owns WN x WM tiles of 32x32 outputs, PL activation planes.
 template <typename Eng, int WGN, int WGM, int WN, int WM, int PL, bool PIPE>
-__global__ __launch_bounds__(WGN* WGM * 64) void gemm_mfma_kernel(const GemmArgs a, const int tiles_n,
+__global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mfma_kernel(const GemmArgs a, const int tiles_n,
                                                                    const int tiles_m)
 {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -338,18 +338,22 @@ __global__ __launch_bounds__(WGN* WGM * 64) void gemm_mfma_kernel(const GemmArgs
 // ---- host side ---------------------------------------------------------------------------
 struct MfmaCfg { int id, bn, bm; };
 
-// Tile choice: the largest tile that still yields about two blocks per CU.
+// Tile choice, from timings of each configuration over a sweep of shapes: the 256 x 256 tile (one
+// block per CU, hand-pipelined loop) needs at least two rounds of blocks to pay for its long
+// epilogue; 256 x 128 (two resident blocks per CU, so one block's stores overlap the other's main
+// loop) wins from one block per CU upwards; below that the smaller tiles, down to 32 x 128, are
+// chosen so that every CU gets a block.
 static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int splitK, int planes)
 {
     // The tile is chosen for the output alone: K ranges are only added (effective_split) where
     // the tiles of the smallest efficient size still leave compute units idle.
     (void)splitK;
-    const int64_t want = 512;
     auto blocks = [&](int bn, int bm) { return batch * cdiv(N, bn) * cdiv(M, bm); };
-    if (M <= 64) return blocks(128, 64) >= want ? MfmaCfg{7, 128, 64} : MfmaCfg{6, 64, 64};   // narrow outputs
-    if (planes == 1 && blocks(256, 256) >= want) return {0, 256, 256};
-    if (blocks(128, 128) >= want) return {1, 128, 128};
-    if (blocks(64, 128) >= want || N > 32) return {2, 64, 128};
+    if (M <= 64) return blocks(128, 64) >= 512 ? MfmaCfg{7, 128, 64} : MfmaCfg{6, 64, 64};   // narrow outputs
+    if (planes == 1 && blocks(256, 256) >= 512) return {0, 256, 256};
+    if (planes == 1 && blocks(256, 128) >= 256) return {4, 256, 128};
+    if (blocks(128, 128) >= 512) return {1, 128, 128};
+    if (blocks(64, 128) >= 256) return {2, 64, 128};
     return {3, 32, 128};
 }
 
@@ -377,7 +381,7 @@ static int launch_cfg(const GemmArgs& a, hipStream_t st)
         else
             return fail(BGEMM_EINVAL, "gemm_mfma: tile not built for two planes");
     } else
-        hipLaunchKernelGGL((gemm_mfma_kernel<Eng, WGN, WGM, WN, WM, 1, (WN * WM >= 16)>), dim3((unsigned)grid),
+        hipLaunchKernelGGL((gemm_mfma_kernel<Eng, WGN, WGM, WN, WM, 1, (WN * WM >= 8)>), dim3((unsigned)grid),
                            dim3(WGN * WGM * 64), 0, st, a, tiles_n, tiles_m);
     return check_launch("gemm_mfma");
 }
@@ -391,7 +395,6 @@ static int launch_eng(const GemmArgs& a_in, hipStream_t st)
     switch (cfg.id) {
     case 0: return launch_cfg<Eng, 2, 2, 4, 4>(a, st);    // 256 x 256
     case 4: return launch_cfg<Eng, 2, 2, 4, 2>(a, st);    // 256 x 128, two blocks per CU
-    case 5: return launch_cfg<Eng, 2, 2, 2, 4>(a, st);    // 128 x 256, two blocks per CU
     case 6: return launch_cfg<Eng, 2, 2, 1, 1>(a, st);    // 64 x 64
     case 7: return launch_cfg<Eng, 2, 2, 2, 1>(a, st);    // 128 x 64
     case 1: return launch_cfg<Eng, 2, 2, 2, 2>(a, st);    // 128 x 128
