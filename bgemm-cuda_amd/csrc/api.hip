@@ -37,8 +37,8 @@ static void ws_needs(int variant, int planes, int64_t batch, int64_t M, int64_t 
 {
     *part = *counters = 0;
     if (variant != BGEMM_VARIANT_VALU && gemm_skinny_shape(planes, batch, M, N, K)) return;      // split inside the block
-    if (variant == BGEMM_VARIANT_VALU) gemm_valu_ws(batch, M, N, splitK, planes, part, counters);
-    else gemm_mfma_ws(batch, M, N, splitK, planes, part, counters);
+    if (variant == BGEMM_VARIANT_VALU) gemm_valu_ws(batch, M, N, K, splitK, planes, part, counters);
+    else gemm_mfma_ws(batch, M, N, K, splitK, planes, part, counters);
 }
 
 // one thread per counter
@@ -148,16 +148,18 @@ static int packed_forward(int mode, const void* W_tiled, const void* X_tiled, co
     if (splitK > 1 && !skinny) {
         size_t part, cnt;
         ws_needs(v, a.mc.planes, batch, M, N, K, splitK, &part, &cnt);
-        if (!ws || !counters)
-            return fail(BGEMM_EWORKSPACE, "bgemm_packed_forward: splitK=%d needs %zu workspace and %zu counter bytes",
-                        splitK, round256(part), round256(cnt * 4));
-        if (ws_bytes < part) return fail(BGEMM_EWORKSPACE, "bgemm_packed_forward: workspace %zu < %zu bytes", ws_bytes, part);
-        if (counter_bytes < cnt * 4)
-            return fail(BGEMM_EWORKSPACE, "bgemm_packed_forward: counters %zu < %zu bytes", counter_bytes, cnt * 4);
-        if (((uintptr_t)ws & 15) || ((uintptr_t)counters & 3))
-            return fail(BGEMM_EALIGN, "bgemm_packed_forward: workspace must be 16-byte aligned");
-        a.ws_part = (int32_t*)ws;
-        a.ws_cnt = (uint32_t*)counters;
+        if (part) {       // this shape will really be split (splitK is an upper bound)
+            if (!ws || !counters)
+                return fail(BGEMM_EWORKSPACE, "bgemm_packed_forward: splitK=%d needs %zu workspace and %zu counter bytes",
+                            splitK, round256(part), round256(cnt * 4));
+            if (ws_bytes < part) return fail(BGEMM_EWORKSPACE, "bgemm_packed_forward: workspace %zu < %zu bytes", ws_bytes, part);
+            if (counter_bytes < cnt * 4)
+                return fail(BGEMM_EWORKSPACE, "bgemm_packed_forward: counters %zu < %zu bytes", counter_bytes, cnt * 4);
+            if (((uintptr_t)ws & 15) || ((uintptr_t)counters & 3))
+                return fail(BGEMM_EALIGN, "bgemm_packed_forward: workspace must be 16-byte aligned");
+            a.ws_part = (int32_t*)ws;
+            a.ws_cnt = (uint32_t*)counters;
+        }
     }
     if (v == BGEMM_VARIANT_VALU) return launch_gemm_valu(a, (hipStream_t)stream);
     if (skinny) return launch_gemm_skinny(a, (hipStream_t)stream, v == BGEMM_VARIANT_MFMA_F4);

@@ -357,13 +357,14 @@ static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int splitK, int pla
     return {3, 32, 128};
 }
 
-void gemm_mfma_ws(int64_t batch, int64_t M, int64_t N, int splitK, int planes, size_t* part_bytes,
+void gemm_mfma_ws(int64_t batch, int64_t M, int64_t N, int64_t K, int splitK, int planes, size_t* part_bytes,
                   size_t* counters)
 {
     const MfmaCfg c = pick_cfg(batch, M, N, splitK, planes);
     const int64_t tiles = batch * cdiv(N, c.bn) * cdiv(M, c.bm);
-    *part_bytes = splitK > 1 ? (size_t)tiles * splitK * c.bn * c.bm * 4 : 0;
-    *counters = splitK > 1 ? (size_t)tiles : 0;
+    const int s = effective_split(tiles, splitK, (int)k_tiles(K));       // as launch_eng will split
+    *part_bytes = s > 1 ? (size_t)tiles * s * c.bn * c.bm * 4 : 0;
+    *counters = s > 1 ? (size_t)tiles : 0;
 }
 
 template <typename Eng, int WGN, int WGM, int WN, int WM>

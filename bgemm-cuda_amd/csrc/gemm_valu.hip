@@ -146,12 +146,13 @@ __global__ __launch_bounds__(256) void gemm_valu_kernel(const GemmArgs a, const 
     }
 }
 
-void gemm_valu_ws(int64_t batch, int64_t M, int64_t N, int splitK, int planes, size_t* part_bytes, size_t* counters)
+void gemm_valu_ws(int64_t batch, int64_t M, int64_t N, int64_t K, int splitK, int planes, size_t* part_bytes, size_t* counters)
 {
     (void)planes;
     const int64_t tiles = batch * cdiv(N, 64) * cdiv(M, 64);
-    *part_bytes = splitK > 1 ? (size_t)tiles * splitK * 64 * 64 * 4 : 0;
-    *counters = splitK > 1 ? (size_t)tiles : 0;
+    const int s = effective_split(tiles, splitK, (int)k_tiles(K));       // as launch_gemm_valu will split
+    *part_bytes = s > 1 ? (size_t)tiles * s * 64 * 64 * 4 : 0;
+    *counters = s > 1 ? (size_t)tiles : 0;
 }
 
 int launch_gemm_valu(const GemmArgs& a_in, hipStream_t st)

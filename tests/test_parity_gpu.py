@@ -310,9 +310,36 @@ def test_dropin_argument_errors():
         lk.bgemm_linear_forward_cuda(x, x, 0, 1)
 
 
+@pytest.mark.parametrize("variant", VARIANTS)
+@pytest.mark.parametrize("M,N,K,splits", [(130, 170, 16384, (2,)), (100, 200, 40000, (3, 5, 8)), (300, 260, 24800, (2, 4))])
+def test_split_k_handover_long_k(oracle, variant, M, N, K, splits):
+    """Shapes with few output tiles and a long K, where the cross-block split-K really happens (K is only
+    split while every range keeps 24 K-tiles): partial tiles through the workspace, tickets, all output kinds."""
+    import _lib
+    rng = np.random.default_rng(M + N + K)
+    w, x = rand_f16(rng, M, K), rand_f16(rng, N, K)
+    Wp, Xp = oracle.c_pack_sign(w), oracle.c_pack_sign(x)
+    nz, sg = oracle.c_pack_ternary(x)
+    want = {MODE_XOR: oracle.c_bgemm_packed(1, Wp, Xp, K), MODE_ATTN: oracle.c_bgemm_packed(2, Wp, Xp, K),
+            MODE_BWTA: oracle.c_bwta_packed(Wp, nz, sg, K)}
+    wp, xp, xt = lk.pack_sign(to_dev(w)), lk.pack_sign(to_dev(x)), lk.pack_ternary(to_dev(x))
+    L = _lib.lib()
+    for sk in splits:
+        assert L.bgemm_packed_workspace_bytes(MODE_XOR, 1, M, N, K, sk, variant) > 0      # it does split
+        for mode in (MODE_XOR, MODE_ATTN, MODE_BWTA):
+            got = lk.bgemm_packed_forward(wp, xt if mode == MODE_BWTA else xp, mode, torch.int32, sk, variant)
+            assert (got[0].cpu().numpy() == want[mode]).all(), (mode, sk)
+        goth = lk.bgemm_packed_forward(wp, xp, MODE_XOR, torch.half, sk, variant)[0].cpu().numpy()
+        assert (goth.view(np.uint16) == f16_of(want[MODE_XOR]).view(np.uint16)).all()
+    sw = rng.uniform(1e-4, 3e-3, M).astype(np.float32)
+    gots = lk.bgemm_packed_forward(wp, xp, MODE_XOR, splitK=splits[-1], variant=variant,
+                                   scale=(to_dev(sw), torch.full((1,), 0.75, device=DEV), None))[0].cpu().numpy()
+    assert (_bits(gots) == _bits(oracle.np_scale_epilogue(want[MODE_XOR], sw, np.float32(0.75), None))).all()
+
+
 def test_split_k_workspace_left_clean():
     rng = np.random.default_rng(77)
-    w, x = rand_f16(rng, 96, 2048, zeros=False), rand_f16(rng, 40, 2048, zeros=False)
+    w, x = rand_f16(rng, 96, 16384, zeros=False), rand_f16(rng, 200, 16384, zeros=False)
     wp, xp = lk.pack_sign(to_dev(w)), lk.pack_sign(to_dev(x))
     first = lk.bgemm_packed_forward(wp, xp, MODE_XOR, torch.int32, 4, VARIANT_MFMA)
     for variant in VARIANTS:
