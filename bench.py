@@ -291,22 +291,24 @@ def bench_c2(steps, warmup):
             "bit_exact": same}
 
 
-def run_extra(which):
-    """The non-headline benchmark configurations: 'c4' decode BWTA, 'c3' attention, 'c2' MLP, 'sweep'."""
+def run_extra(which, quick=False, variant=0):
+    """The non-headline benchmark configurations: 'c4' decode BWTA, 'c3' attention, 'c2' MLP, 'sweep'.
+    quick: a tenth of the launches (for counter collection, where every dispatch is serialised)."""
     extra = []
+    div = 10 if quick else 1
     if which in ("c4", "all"):
         for N in (1, 4, 16):
             for sk in (1, 8):
-                extra.append(bench_c4(2000, 200, N, sk))
+                extra.append(bench_c4(2000 // div, 200 // div, N, sk, variant))
                 log(json.dumps(extra[-1]))
         for N in (1, 4, 16):
-            extra.append(bench_c4_batched(400, N))
+            extra.append(bench_c4_batched(400 // div, N))
             log(json.dumps(extra[-1]))
     if which in ("c3", "all"):
-        extra.append(bench_c3(200, 20))
+        extra.append(bench_c3(200 // div, 20 // div + 1, variant))
         log(json.dumps(extra[-1]))
     if which in ("c2", "all"):
-        extra.append(bench_c2(200, 20))
+        extra.append(bench_c2(200 // div, 20 // div + 1))
         log(json.dumps(extra[-1]))
     if which in ("sweep", "all"):
         for (K, N) in [(4096, 256), (4096, 2048), (16384, 256), (16384, 2048)]:
@@ -329,6 +331,7 @@ def main():
     ap.add_argument("--all", action="store_true", help="also time the other benchmark configurations")
     ap.add_argument("--only", choices=["c2", "c3", "c4", "sweep"], help="time just that configuration (for profiling)")
     ap.add_argument("--variant", type=int, default=0, help="0 auto, 1 VALU, 2 MFMA int8, 3 MFMA fp4")
+    ap.add_argument("--quick", action="store_true", help="with --only: a tenth of the launches (counter collection)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--floor", action="store_true",
                     help="print the hardware floors for the decode shape (empty launch, cold 5.6 MB read, sustained read)")
@@ -353,7 +356,7 @@ def main():
         print(json.dumps({"floor": bench_floor()}), flush=True)
         return
     if args.only:
-        print(json.dumps({"configs": run_extra(args.only)}), flush=True)
+        print(json.dumps({"configs": run_extra(args.only, args.quick, args.variant)}), flush=True)
         return
 
     c5, (w16, x16) = bench_c5(args.steps, args.warmup, variant=args.variant)
