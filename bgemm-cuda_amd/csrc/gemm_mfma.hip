@@ -116,8 +116,9 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
                     acc[0][i][j] = Eng::mma(Eng::make(cur[i]), Eng::make(cur[WN + j]), acc[0][i][j]);
 #pragma unroll
                     for (int d = q * DPG; d < (q + 1) * DPG; d++)
-                        nxt[d / 4][d % 4] = s + 1 < STEPS ? Eng::expand1(A[d / 4][d % 4], s + 1)
-                                                          : Eng::expand1(B[d / 4][d % 4], 0);
+                        nxt[d / 4][d % 4] = d / 4 < WN      // fragments 0 .. WN-1 are the activation side
+                            ? (s + 1 < STEPS ? Eng::expand1_x(A[d / 4][d % 4], s + 1) : Eng::expand1_x(B[d / 4][d % 4], 0))
+                            : (s + 1 < STEPS ? Eng::expand1_w(A[d / 4][d % 4], s + 1) : Eng::expand1_w(B[d / 4][d % 4], 0));
                     if (s == 0 && q < NF) pop[q] += __popc(A[q][0]) + __popc(A[q][1]) + __popc(A[q][2]) + __popc(A[q][3]);
                     if (s == STEPS - 1 && q < NF) load_frag(A[q], q, kt + 2);   // A is dead after step STEPS-2
                     __builtin_amdgcn_sched_barrier(0);
@@ -130,7 +131,7 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
 #pragma unroll
             for (int f = 0; f < NF; f++)
 #pragma unroll
-                for (int c = 0; c < 4; c++) buf[0][f][c] = Eng::expand1(rawA[f][c], 0);
+                for (int c = 0; c < 4; c++) buf[0][f][c] = f < WN ? Eng::expand1_x(rawA[f][c], 0) : Eng::expand1_w(rawA[f][c], 0);
             for (int kt = kt0; kt < kt1; kt += 2) {
                 k_tile(rawA, rawB, kt);
                 k_tile(rawB, rawA, kt + 1);
@@ -176,12 +177,12 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
         for (int s = 0; s < Eng::STEPS; s++) {
             typename Eng::Frag bw[WM];
 #pragma unroll
-            for (int j = 0; j < WM; j++) bw[j] = Eng::expand(wf[j], s);
+            for (int j = 0; j < WM; j++) bw[j] = Eng::expand_w(wf[j], s);
 #pragma unroll
             for (int p = 0; p < PL; p++)
 #pragma unroll
                 for (int i = 0; i < WN; i++) {
-                    const typename Eng::Frag ax = Eng::expand(xf[p][i], s);
+                    const typename Eng::Frag ax = Eng::expand_x(xf[p][i], s);
 #pragma unroll
                     for (int j = 0; j < WM; j++) acc[p][i][j] = Eng::mma(ax, bw[j], acc[p][i][j]);
                 }

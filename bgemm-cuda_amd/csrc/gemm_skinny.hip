@@ -98,9 +98,9 @@ __global__ __launch_bounds__(256) void gemm_skinny_stream_kernel(const GemmArgs 
             for (int t = 0; t < RT; t++) pa[t] += popc4(wq[q][t]);
 #pragma unroll
             for (int s = 0; s < Eng::STEPS; s++) {
-                const typename Eng::Frag ax = Eng::expand(xq[q], s);
+                const typename Eng::Frag ax = Eng::expand_x(xq[q], s);
 #pragma unroll
-                for (int t = 0; t < RT; t++) acc[t] = Eng::mma(ax, Eng::expand(wq[q][t], s), acc[t]);
+                for (int t = 0; t < RT; t++) acc[t] = Eng::mma(ax, Eng::expand_w(wq[q][t], s), acc[t]);
             }
         }
     };
@@ -206,9 +206,9 @@ __global__ __launch_bounds__(KW * 64) void gemm_skinny_splitk_kernel(const GemmA
                 for (int i = 0; i < NTL; i++) pb[i] += popc4(xq[q][i]);
 #pragma unroll
                 for (int s = 0; s < Eng::STEPS; s++) {
-                    const typename Eng::Frag bw = Eng::expand(wq[q], s);
+                    const typename Eng::Frag bw = Eng::expand_w(wq[q], s);
 #pragma unroll
-                    for (int i = 0; i < NTL; i++) acc[i] = Eng::mma(Eng::expand(xq[q][i], s), bw, acc[i]);
+                    for (int i = 0; i < NTL; i++) acc[i] = Eng::mma(Eng::expand_x(xq[q][i], s), bw, acc[i]);
                 }
             }
         }

@@ -23,6 +23,11 @@ struct EngI8 {
         return r;
     }
     __device__ static __forceinline__ unsigned expand1(const unsigned w, const int s) { return (w >> s) & 0x01010101u; }
+    // both operands expand alike
+    __device__ static __forceinline__ Frag expand_w(const uint4 w, const int s) { return expand(w, s); }
+    __device__ static __forceinline__ Frag expand_x(const uint4 w, const int s) { return expand(w, s); }
+    __device__ static __forceinline__ unsigned expand1_w(const unsigned w, const int s) { return expand1(w, s); }
+    __device__ static __forceinline__ unsigned expand1_x(const unsigned w, const int s) { return expand1(w, s); }
     __device__ static __forceinline__ Frag make(const unsigned (&f)[4])
     {
         Frag r = {(int)f[0], (int)f[1], (int)f[2], (int)f[3]};
@@ -36,28 +41,43 @@ struct EngI8 {
 };
 
 // fp4 engine: the same tile is four 64-deep steps of v_mfma_f32_32x32x64_f8f6f4 with E2M1
-// operands; nibble c of word q at step s is bit 4c+s, moved to nibble bit 1 (0b0010 = 1.0).
-// Products are 0 or 1 and the fp32 accumulator holds integers below 2^24, so it stays exact.
+// operands; nibble c of word q at step s is bit 4c+s.  E2M1 has three single-bit values,
+// 0b0001 = 0.5, 0b0010 = 1.0, 0b0100 = 2.0, so a bit can often stay where it is: the weight side
+// keeps bits 0..2 in place (0.5, 1, 2: one AND per step) and the activation side moves the same
+// bits to the reciprocal values (2, 1, 0.5), so every product of set bits is exactly 1; bit 3
+// (the sign position) is shifted to 1.0 on both sides.  Five VALU ops per weight word and six
+// per activation word instead of seven and seven.  Products are 0 or 1 and the fp32 accumulator
+// holds integers below 2^24, so it stays exact.
 struct EngF4 {
     typedef v16f Acc;
     typedef v8i Frag;
     static constexpr int STEPS = 4;
-    __device__ static __forceinline__ unsigned nib(const unsigned w, const int s)
+    __device__ static __forceinline__ unsigned expand1_w(const unsigned w, const int s)
     {
-        return (s == 0 ? (w << 1) : (w >> (s - 1))) & 0x22222222u;
+        return s == 3 ? (w >> 2) & 0x22222222u : w & (0x11111111u << s);
     }
-    __device__ static __forceinline__ Frag expand(const uint4 w, const int s)
+    __device__ static __forceinline__ unsigned expand1_x(const unsigned w, const int s)
+    {
+        return s == 0 ? (w << 2) & 0x44444444u : s == 1 ? w & 0x22222222u : (w >> 2) & (s == 2 ? 0x11111111u : 0x22222222u);
+    }
+    __device__ static __forceinline__ Frag expand_w(const uint4 w, const int s)
     {
         Frag r = {0, 0, 0, 0, 0, 0, 0, 0};
-        r[0] = nib(w.x, s); r[1] = nib(w.y, s); r[2] = nib(w.z, s); r[3] = nib(w.w, s);
+        r[0] = expand1_w(w.x, s); r[1] = expand1_w(w.y, s); r[2] = expand1_w(w.z, s); r[3] = expand1_w(w.w, s);
         return r;
     }
-    __device__ static __forceinline__ unsigned expand1(const unsigned w, const int s) { return nib(w, s); }
+    __device__ static __forceinline__ Frag expand_x(const uint4 w, const int s)
+    {
+        Frag r = {0, 0, 0, 0, 0, 0, 0, 0};
+        r[0] = expand1_x(w.x, s); r[1] = expand1_x(w.y, s); r[2] = expand1_x(w.z, s); r[3] = expand1_x(w.w, s);
+        return r;
+    }
     __device__ static __forceinline__ Frag make(const unsigned (&f)[4])
     {
         Frag r = {(int)f[0], (int)f[1], (int)f[2], (int)f[3], 0, 0, 0, 0};
         return r;
     }
+    // a = activation-side fragment, b = weight-side fragment
     __device__ static __forceinline__ Acc mma(const Frag a, const Frag b, const Acc c)
     {
         return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 4, 4, 0, 0, 0, 0);
