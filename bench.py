@@ -112,6 +112,27 @@ def bench_c5(steps, warmup, M=8192, N=8192, K=8192, splitK=1, variant=0):
             "bit_exact": ok, "act_pack_ms": pack_ms}, (w16, x16)
 
 
+def bench_c5_dropin(steps, warmup, M=8192, N=8192, K=8192):
+    """The same GEMM through the reference's own entry point, `bgemm_linear_forward_cuda(in_feats, weights)`:
+    fp16 operands in, both sign-packed on every call (one launch), fp16 out."""
+    import torch
+    import lowbit_kernel as lk
+    dev = torch.device("cuda:0")
+    w16, x16 = pm1_f16((M, K), 5001, dev), pm1_f16((N, K), 5002, dev)
+    out = [None]
+
+    def fn(i):
+        out[0] = lk.bgemm_linear_forward_cuda(x16, w16, 1, 1)
+    ms = time_gpu(fn, warmup, steps)
+    g = torch.Generator().manual_seed(7)
+    rs, cs = torch.randperm(M, generator=g)[:64].to(dev), torch.randperm(N, generator=g)[:64].to(dev)
+    want = (x16[cs].float() @ w16[rs].float().T).half()
+    ok = bool(torch.equal(out[0][cs][:, rs], want))
+    ops = 2.0 * M * N * K
+    return {"name": "C5 through the fp16 drop-in call %dx%dx%d (packs both operands per call, fp16 out)" % (M, N, K),
+            "ms": ms, "tops": ops / ms / 1e9, "ops": ops, "bit_exact": ok}
+
+
 def cpu_baseline_c5(w16, x16, budget_s=12.0):
     """Reference CPU path (torch matmul on +-1 fp32 tensors) on a bounded column slice."""
     import torch
@@ -311,6 +332,8 @@ def run_extra(which, quick=False, variant=0):
         extra.append(bench_c2(200 // div, 20 // div + 1))
         log(json.dumps(extra[-1]))
     if which in ("sweep", "all"):
+        extra.append(bench_c5_dropin(50 // div + 2, 5))
+        log(json.dumps(extra[-1]))
         for (K, N) in [(4096, 256), (4096, 2048), (16384, 256), (16384, 2048)]:
             for sk in (1, 2, 4):
                 r, _ = bench_c5(20, 3, 8192, N, K, sk)
