@@ -5,8 +5,8 @@
 // {0,1} matrices.  The operands stay bit-packed all the way into registers: one 16-byte
 // load per lane fetches a 32-row x 256-bit tile in exactly the order the 32x32 MFMA wants
 // its fragments (lane = half*32 + row), and the MFMA steps of the tile are produced by a
-// shift and a mask per register.  Both operands use the same rule, so the K permutation it
-// implies cancels.  Waves never exchange data: no LDS, no barriers in the main loop.  Row
+// mask (and for some steps a shift) per register.  Both operands map bits to steps by the same
+// rule, so the K permutation it implies cancels.  Waves never exchange data: no LDS, no barriers in the main loop.  Row
 // popcounts for the rank-one terms come from the same registers (4 v_bcnt per fragment).
 #include "common.h"
 #include "mfma_engines.h"

@@ -106,11 +106,14 @@ int bgemm_logical_from_tiled(const void* tiled, int64_t rows, int64_t K,
  *   X2_tiled : BWTA only, the sign&nonzero plane (X_tiled is the nonzero plane).
  *   batch    : number of independent GEMMs; strides in uint32 words / output elements
  *              (a stride of 0 shares that operand across the batch).
- *   splitK   : >= 1; K-tiles are divided into splitK contiguous ranges as in
- *              kernel_matmul.cuh:397-404 and reduced inside the same launch with integer
- *              adds, so the result does not depend on it.
- *   ws       : scratch for split-K partial tiles, bgemm_packed_workspace_bytes() bytes,
- *              no initialisation needed (NULL when that is 0).
+ *   splitK   : >= 1, an upper bound on the number of contiguous K ranges (partitioned as in
+ *              kernel_matmul.cuh:397-404) that are reduced inside the same launch with integer
+ *              adds, so the result does not depend on it.  K is only split where the output
+ *              tiles alone leave compute units idle and every range stays long enough to pay
+ *              for the hand-over; few activation rows are split inside the block.
+ *   ws       : scratch for split-K partial tiles, bgemm_packed_workspace_bytes() bytes for the
+ *              same arguments (0 when the shape will not be split), no initialisation needed
+ *              (NULL when that is 0).
  *   counters : split-K arrival counters, bgemm_packed_counter_bytes() bytes.  Must be
  *              zero-filled once before first use; every call leaves them zero again.
  *              Calls that share counters must not overlap in time.
