@@ -302,14 +302,23 @@ def bench_c2(steps, warmup):
         for Wp, sw in zip(Wps, sws):
             h = lk.bgemm_packed_forward(Wp, lk.pack_sign(h), lk.MODE_XOR, splitK=8, scale=(sw, sa, None))[0]
         return h
-    same = bool(torch.equal(fwd_ops(0), fwd_fused(0)))
+    N = x.shape[0]
+    hidden = [lk.zeros_packed(N, dims[1], 1, dev), lk.zeros_packed(N, dims[2], 1, dev)]
+
+    def fwd_bits(i):                            # hidden activations never stored: 4 launches
+        hp = lk.pack_sign(x)
+        for l in range(2):
+            hp = lk.bgemm_packed_forward(Wps[l], hp, lk.MODE_XOR, splitK=8, scale=(sws[l], sa, None), bits_out=hidden[l])
+        return lk.bgemm_packed_forward(Wps[2], hp, lk.MODE_XOR, splitK=8, scale=(sws[2], sa, None))[0]
+    same = bool(torch.equal(fwd_ops(0), fwd_fused(0))) and bool(torch.equal(fwd_ops(0), fwd_bits(0)))
     ms_ops = time_gpu(fwd_ops, warmup, steps)
     ms_fused = time_gpu(fwd_fused, warmup, steps)
     ms_graph = time_gpu_graph(fwd_fused, 4, 2, max(2, steps // 4))
+    ms_bits = time_gpu_graph(fwd_bits, 4, 2, max(2, steps // 4))
     ops = 2.0 * 128 * (784 * 4096 + 4096 * 4096 + 4096 * 10)
-    return {"name": "C2 MLP 784-4096-4096-10 batch 128, fp16 in/out, fused pack+GEMM+scale (6 launches, graph replay)",
-            "ms": ms_graph, "ms_eager_launch": ms_fused, "ms_op_by_op": ms_ops, "tops": ops / ms_graph / 1e9, "ops": ops,
-            "bit_exact": same}
+    return {"name": "C2 MLP 784-4096-4096-10 batch 128, fp16 in/out, bits between layers (4 launches, graph replay)",
+            "ms": ms_bits, "ms_fused_6_launches": ms_graph, "ms_eager_launch": ms_fused, "ms_op_by_op": ms_ops,
+            "tops": ops / ms_bits / 1e9, "ops": ops, "bit_exact": same}
 
 
 def run_extra(which, quick=False, variant=0):

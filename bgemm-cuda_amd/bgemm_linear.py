@@ -16,7 +16,7 @@ import torch.nn as nn
 
 import lowbit_kernel
 
-__all__ = ['BNNLinear', 'BGEMMLinear', 'BGEMMLinear_elastic_signed', 'bgemm_matmul', 'bgemm_attn_matmul',
+__all__ = ['BNNLinear', 'BGEMMLinear', 'BGEMMChain', 'BGEMMLinear_elastic_signed', 'bgemm_matmul', 'bgemm_attn_matmul',
            'BGEMMLinear_bireal', 'NNLinear_elastic_signed', 'bgemm_linear', 'bgemm_linear_bireal',
            'bgemm_linear_elastic_signed', 'nn_linear_elastic_signed', 'BinActive', 'ternary']
 
@@ -267,6 +267,40 @@ class BGEMMLinear(_ScaledBinaryLinear):
             return self._fused_forward(x)
         out = self._fn.apply(x - self.zpa, self.weight - self.zpw) * self.sw * self.sa
         return self._add_bias(out)
+
+
+class BGEMMChain(nn.Sequential):
+    """BGEMMLinear layers applied back to back (the binarisation is the only nonlinearity between them).
+    When no gradient is recorded the activations between layers exist only as bits: every GEMM but the last
+    writes the next layer's centred, sign-packed operand straight from its accumulators, so a chain of L
+    layers is L + 1 launches and never stores a hidden activation.  Same results as calling the layers one
+    after the other, bit for bit.  Not in the reference, which has no layer container."""
+
+    def _fusable(self, x):
+        layers = list(self)
+        return (len(layers) > 0 and all(isinstance(l, BGEMMLinear) and l.initialized and l._fn is not None for l in layers)
+                and all(l._fusable(x) for l in layers)
+                and all(a.weight.shape[0] == b.weight.shape[1] for a, b in zip(layers, layers[1:])))
+
+    def forward(self, x):
+        if not self._fusable(x):
+            return super().forward(x)          # also the first call, which initialises the layers' scales
+        layers = list(self)
+        lead = x.shape[:-1]
+        xp = lowbit_kernel.pack_sign(x.reshape(-1, x.shape[-1]), zero_point=layers[0].zpa)
+        if not hasattr(self, "_bits"):
+            self._bits = {}
+        for i, layer in enumerate(layers):
+            scale = (layer.sw.detach(), layer.sa.detach().reshape(1), None if layer.bias is None else layer.bias.detach())
+            if i + 1 == len(layers):
+                out = lowbit_kernel.bgemm_packed_forward(layer._packed_weight(), xp, lowbit_kernel.MODE_XOR, splitK=8, scale=scale)
+                return out.reshape(*lead, layer.weight.shape[0])
+            key = (i, xp.rows, x.device)
+            if key not in self._bits:      # zero-filled once: the GEMM writes real bits only, the padding stays zero
+                self._bits[key] = lowbit_kernel.zeros_packed(xp.rows, layer.weight.shape[0], 1, x.device)
+            xp = lowbit_kernel.bgemm_packed_forward(layer._packed_weight(), xp, lowbit_kernel.MODE_XOR, splitK=8, scale=scale,
+                                                    bits_out=self._bits[key],
+                                                    next_zero_point=layers[i + 1].zpa.detach().reshape(1))
 
 
 class BGEMMLinear_bireal(BGEMMLinear):

@@ -53,7 +53,7 @@ __global__ void clear_counters_kernel(uint32_t* c, int64_t n)
 using namespace bgemm;
 
 extern "C" const char* bgemm_last_error(void) { return g_err; }
-extern "C" int bgemm_abi_version(void) { return 3; }
+extern "C" int bgemm_abi_version(void) { return 4; }
 
 static bool ws_query(int mode, int64_t batch, int64_t M, int64_t N, int64_t K, int splitK, int variant,
                      size_t* part, size_t* counters)
@@ -93,20 +93,33 @@ __global__ void fill_empty_sum_kernel(const GemmArgs a)
     store_out(a, (int64_t)blockIdx.y * a.strideC + (i / a.M) * a.M, i % a.M, 0);
 }
 
+// K = 0 with a bits kind: one thread per output word, the 32 columns in turn.
+__global__ void fill_empty_bits_kernel(const GemmArgs a)
+{
+    const int64_t Mw = cdiv(a.M, 32), i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= a.N * Mw) return;
+    const int64_t n = i / Mw, jw = i % Mw;
+    unsigned w = 0;
+    for (int c = 0; c < 32; c++)
+        if (jw * 32 + c < a.M) w |= next_sign_bit(a, jw * 32 + c, 0) << (31 - c);
+    reinterpret_cast<uint32_t*>(a.out)[(int64_t)blockIdx.y * a.strideC + tiled_word_offset(n, jw, k_tiles(a.M))] = w;
+}
+
 static int packed_forward(int mode, const void* W_tiled, const void* X_tiled, const void* X2_tiled,
                           void* out, int out_dtype, int64_t batch, int64_t M, int64_t N, int64_t K,
                           int64_t strideW, int64_t strideX, int64_t strideC,
                           int splitK, int variant, void* ws, size_t ws_bytes,
                           void* counters, size_t counter_bytes,
-                          const void* sw, const void* sa, const void* bias, void* stream)
+                          const void* sw, const void* sa, const void* bias, const void* zp, void* stream)
 {
     g_err[0] = 0;
     GemmArgs a;
     memset(&a, 0, sizeof a);
     if (!mode_coef(mode, &a.mc)) return fail(BGEMM_EINVAL, "bgemm_packed_forward: unknown mode %d", mode);
-    if (out_dtype < BGEMM_OUT_I32 || out_dtype > BGEMM_OUT_F16_SCALED)
+    if (out_dtype < BGEMM_OUT_I32 || out_dtype > BGEMM_OUT_BITS_F16)
         return fail(BGEMM_EINVAL, "bgemm_packed_forward: unknown output dtype %d", out_dtype);
-    const bool scaled = out_dtype == BGEMM_OUT_F32_SCALED || out_dtype == BGEMM_OUT_F16_SCALED;
+    const bool bits = out_dtype == BGEMM_OUT_BITS_F32 || out_dtype == BGEMM_OUT_BITS_F16;
+    const bool scaled = bits || out_dtype == BGEMM_OUT_F32_SCALED || out_dtype == BGEMM_OUT_F16_SCALED;
     if (variant < BGEMM_VARIANT_AUTO || variant > BGEMM_VARIANT_MFMA_F4)
         return fail(BGEMM_EINVAL, "bgemm_packed_forward: unknown variant %d", variant);
     if (batch < 0 || M < 0 || N < 0 || K < 0 || splitK < 1 || splitK > 65535)
@@ -121,16 +134,21 @@ static int packed_forward(int mode, const void* W_tiled, const void* X_tiled, co
     if (batch == 0 || M == 0 || N == 0) return BGEMM_OK;
     if (!out) return fail(BGEMM_ENULL, "bgemm_packed_forward: out is NULL");
     if (scaled && (!sw || !sa)) return fail(BGEMM_ENULL, "bgemm_packed_forward_scaled: sw or sa is NULL");
-    if (batch > 1 && strideC < M * N)
-        return fail(BGEMM_EINVAL, "bgemm_packed_forward: strideC=%lld smaller than N*M", (long long)strideC);
+    if (batch > 1 && strideC < (bits ? bgemm_tiled_words(N, M) : M * N))
+        return fail(BGEMM_EINVAL, "bgemm_packed_forward: output stride %lld smaller than one output", (long long)strideC);
+    if (bits && ((uintptr_t)out & 3)) return fail(BGEMM_EALIGN, "bgemm_packed_forward_bits: output not 4-byte aligned");
     a.out = out; a.out_kind = out_dtype;
-    a.ep_sw = sw; a.ep_sa = sa; a.ep_bias = bias;
+    a.ep_sw = sw; a.ep_sa = sa; a.ep_bias = bias; a.ep_zp = zp;
     a.M = M; a.N = N; a.K = K;
     a.strideC = strideC;
     if (K == 0) {   // empty sum: every mode gives 0
         if (batch > 65535 || cdiv(N * M, 256) > 0x7fffffffLL) return fail(BGEMM_EINVAL, "bgemm_packed_forward: output too large");
-        hipLaunchKernelGGL(fill_empty_sum_kernel, dim3((unsigned)cdiv(N * M, 256), (unsigned)batch), dim3(256), 0,
-                           (hipStream_t)stream, a);
+        if (bits)
+            hipLaunchKernelGGL(fill_empty_bits_kernel, dim3((unsigned)cdiv(N * cdiv(M, 32), 256), (unsigned)batch), dim3(256), 0,
+                               (hipStream_t)stream, a);
+        else
+            hipLaunchKernelGGL(fill_empty_sum_kernel, dim3((unsigned)cdiv(N * M, 256), (unsigned)batch), dim3(256), 0,
+                               (hipStream_t)stream, a);
         return check_launch("bgemm_packed_forward: fill");
     }
     if (!W_tiled || !X_tiled || (a.mc.planes == 2 && !X2_tiled))
@@ -142,7 +160,7 @@ static int packed_forward(int mode, const void* W_tiled, const void* X_tiled, co
     a.MT = (int)row_tiles(M); a.NT = (int)row_tiles(N); a.KT = (int)k_tiles(K);
     a.strideW = strideW / 4; a.strideX = strideX / 4;
     a.batch = (int)batch; a.splitK = splitK;
-    a.vec_store = (M % 4 == 0) && (strideC % 4 == 0) && (((uintptr_t)out & 15) == 0);
+    a.vec_store = !bits && (M % 4 == 0) && (strideC % 4 == 0) && (((uintptr_t)out & 15) == 0);
     const int v = variant == BGEMM_VARIANT_AUTO ? pick_variant(mode, batch, M, N, K) : variant;
     const bool skinny = v != BGEMM_VARIANT_VALU && gemm_skinny_shape(a.mc.planes, batch, M, N, K);
     if (splitK > 1 && !skinny) {
@@ -175,7 +193,7 @@ extern "C" int bgemm_packed_forward(int mode, const void* W_tiled, const void* X
     if (out_dtype != BGEMM_OUT_I32 && out_dtype != BGEMM_OUT_F16)
         return fail(BGEMM_EINVAL, "bgemm_packed_forward: unknown output dtype %d", out_dtype);
     return packed_forward(mode, W_tiled, X_tiled, X2_tiled, out, out_dtype, batch, M, N, K, strideW, strideX, strideC,
-                          splitK, variant, ws, ws_bytes, counters, counter_bytes, nullptr, nullptr, nullptr, stream);
+                          splitK, variant, ws, ws_bytes, counters, counter_bytes, nullptr, nullptr, nullptr, nullptr, stream);
 }
 
 extern "C" int bgemm_packed_forward_scaled(int mode, const void* W_tiled, const void* X_tiled, const void* X2_tiled,
@@ -189,7 +207,22 @@ extern "C" int bgemm_packed_forward_scaled(int mode, const void* W_tiled, const 
         return fail(BGEMM_EINVAL, "bgemm_packed_forward_scaled: output dtype must be BGEMM_OUT_F32_SCALED or "
                                   "BGEMM_OUT_F16_SCALED, got %d", out_dtype);
     return packed_forward(mode, W_tiled, X_tiled, X2_tiled, out, out_dtype, batch, M, N, K, strideW, strideX, strideC,
-                          splitK, variant, ws, ws_bytes, counters, counter_bytes, sw, sa, bias, stream);
+                          splitK, variant, ws, ws_bytes, counters, counter_bytes, sw, sa, bias, nullptr, stream);
+}
+
+extern "C" int bgemm_packed_forward_bits(int mode, const void* W_tiled, const void* X_tiled, const void* X2_tiled,
+                                         void* out_tiled, int out_dtype, int64_t batch, int64_t M, int64_t N, int64_t K,
+                                         int64_t strideW, int64_t strideX, int64_t strideOut,
+                                         int splitK, int variant, void* ws, size_t ws_bytes,
+                                         void* counters, size_t counter_bytes,
+                                         const void* sw, const void* sa, const void* bias, const void* zero_point,
+                                         void* stream)
+{
+    if (out_dtype != BGEMM_OUT_BITS_F32 && out_dtype != BGEMM_OUT_BITS_F16)
+        return fail(BGEMM_EINVAL, "bgemm_packed_forward_bits: output dtype must be BGEMM_OUT_BITS_F32 or "
+                                  "BGEMM_OUT_BITS_F16, got %d", out_dtype);
+    return packed_forward(mode, W_tiled, X_tiled, X2_tiled, out_tiled, out_dtype, batch, M, N, K, strideW, strideX,
+                          strideOut, splitK, variant, ws, ws_bytes, counters, counter_bytes, sw, sa, bias, zero_point, stream);
 }
 
 // ---- fp16-operand call: pack both operands into the workspace, then the packed GEMM ----

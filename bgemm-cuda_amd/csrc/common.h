@@ -16,9 +16,16 @@ constexpr int TILE_KBITS = 256;
 constexpr int TILE_U4 = 64;      // uint4 slots per tile
 constexpr int TILE_WORDS = 256;  // uint32 words per tile
 
-static inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+__host__ __device__ static inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 static inline int64_t row_tiles(int64_t rows) { return cdiv(rows, TILE_ROWS); }
-static inline int64_t k_tiles(int64_t K) { return cdiv(K, TILE_KBITS); }
+__host__ __device__ static inline int64_t k_tiles(int64_t K) { return cdiv(K, TILE_KBITS); }
+
+// Word offset of logical word jw of `row` inside a tiled operand with KT k-tiles.
+__host__ __device__ static inline int64_t tiled_word_offset(int64_t row, int64_t jw, int64_t KT)
+{
+    const int64_t rt = row >> 5, r = row & 31, kt = jw >> 3, h = (jw >> 2) & 1, q = jw & 3;
+    return ((rt * KT + kt) * TILE_U4 + h * 32 + r) * 4 + q;
+}
 
 // Records a message for bgemm_last_error() and returns `code`.
 int fail(int code, const char* fmt, ...);
@@ -46,6 +53,7 @@ struct GemmArgs {
     const uint4* W; const uint4* X; const uint4* X2;
     void* out; int out_kind;       // BGEMM_OUT_*
     const void* ep_sw; const void* ep_sa; const void* ep_bias;   // scaled output kinds: per-column scale, scalar, bias
+    const void* ep_zp;    // bits kinds: the next layer's zero point (null = 0)
     int vec_store;        // rows of `out` are 16-byte aligned: the epilogue may store four elements per lane
     int64_t M, N, K;
     int MT, NT, KT;
@@ -151,6 +159,33 @@ __device__ __forceinline__ __half scaled_f16(const GemmArgs& a, const int64_t m,
     return r;
 }
 __device__ __forceinline__ int out_elem_shift(const int kind) { return (kind == BGEMM_OUT_F16 || kind == BGEMM_OUT_F16_SCALED) ? 1 : 2; }
+
+// Bits kinds: the scaled output is not stored; the next binary layer's operand is, i.e. the sign bit
+// of half_rn(y - zp) with y evaluated as above.  The subtraction is exact enough for its sign to
+// survive the rounding to fp16, so the sign bit of the fp32 difference is taken.
+__device__ __forceinline__ bool bits_kind(const int kind) { return kind >= BGEMM_OUT_BITS_F32; }
+__device__ __forceinline__ unsigned next_sign_bit(const GemmArgs& a, const int64_t m, const int v)
+{
+    float d;
+    if (a.out_kind == BGEMM_OUT_BITS_F32)
+        d = __fsub_rn(scaled_f32(a, m, v), a.ep_zp ? *reinterpret_cast<const float*>(a.ep_zp) : 0.f);
+    else
+        d = __fsub_rn(__half2float(scaled_f16(a, m, v)),
+                      a.ep_zp ? __half2float(*reinterpret_cast<const __half*>(a.ep_zp)) : 0.f);
+    return __float_as_uint(d) >> 31;
+}
+// One word of the tiled output: the 32 lanes of a half-wave hold the bits of columns m32 .. m32 + 31
+// (m32 a multiple of 32) of output row n, bit = 0 where the column does not exist.  Every lane of the
+// wave calls this; column i lands at bit 31 - i.
+__device__ __forceinline__ void store_bits_word(const GemmArgs& a, const int b, const int64_t n, const int64_t m32,
+                                                const unsigned bit)
+{
+    const int lane = threadIdx.x & 63;
+    const unsigned long long bal = __ballot(bit != 0);
+    const unsigned w = __brev((unsigned)(lane < 32 ? bal : bal >> 32));
+    if ((lane & 31) == 0 && n < a.N && m32 < a.M)
+        reinterpret_cast<uint32_t*>(a.out)[(int64_t)b * a.strideC + tiled_word_offset(n, m32 >> 5, k_tiles(a.M))] = w;
+}
 
 // Final store of one output element (column m of a row whose first element has index row0).
 template <int KIND>

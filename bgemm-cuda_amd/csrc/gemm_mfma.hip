@@ -329,7 +329,11 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
             for (int p = 0; p < 16 * WM; p++) {
                 const int idx = p * 64 + lane, row = idx / (32 * WM), c = idx % (32 * WM);
                 const int64_t n = nrow0 + row, m = mcol0 + c;
-                if (n < a.N && m < a.M) store_out(a, out_off + n * a.M, m, st[row * ROW_I + c]);
+                if (bits_kind(a.out_kind)) {        // half-waves hold 32 consecutive columns of one row
+                    const bool real = n < a.N && m < a.M;
+                    store_bits_word(a, b, n, mcol0 + (c & ~31), real ? next_sign_bit(a, m, st[row * ROW_I + c]) : 0u);
+                } else if (n < a.N && m < a.M)
+                    store_out(a, out_off + n * a.M, m, st[row * ROW_I + c]);
             }
         }
         __syncthreads();

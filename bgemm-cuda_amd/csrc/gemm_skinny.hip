@@ -129,7 +129,10 @@ __global__ __launch_bounds__(256) void gemm_skinny_stream_kernel(const GemmArgs 
             const int64_t m = ((int64_t)grp * RT + t) * 32 + r;
             const int val = skinny_value(mc, two, kbits, pa[t], pbn, pbn2, Eng::to_int(acc[t], v),
                                          Eng::to_int(acc[t], (v + 8) & 15));
-            if (m < a.M) store_out(a, out_row0 + (int64_t)n * a.M, m, val);
+            if (bits_kind(a.out_kind))          // a half-wave holds the 32 columns of this row tile for row n
+                store_bits_word(a, b, n, m - r, m < a.M ? next_sign_bit(a, m, val) : 0u);
+            else if (m < a.M)
+                store_out(a, out_row0 + (int64_t)n * a.M, m, val);
         }
     }
 }
@@ -245,7 +248,10 @@ __global__ __launch_bounds__(KW * 64) void gemm_skinny_splitk_kernel(const GemmA
         const int d2 = two ? sAcc[0][v + 8][hh * 32 + c] : 0;
         const int64_t m = (int64_t)rt * 32 + c;
         const int val = skinny_value(mc, two, kbits, sPa[c], sPb[i][nl], two ? sPb[0][nl + 16] : 0, d, d2);
-        if (m < a.M) store_out(a, (int64_t)b * a.strideC + (int64_t)n * a.M, m, val);
+        if (bits_kind(a.out_kind))
+            store_bits_word(a, b, n, (int64_t)rt * 32, m < a.M ? next_sign_bit(a, m, val) : 0u);
+        else if (m < a.M)
+            store_out(a, (int64_t)b * a.strideC + (int64_t)n * a.M, m, val);
     }
 }
 

@@ -135,6 +135,30 @@ __global__ __launch_bounds__(256) void gemm_valu_kernel(const GemmArgs a, const 
         }
     }
     const int64_t out_off = (int64_t)b * a.strideC;
+    if (bits_kind(a.out_kind)) {
+        // a wave holds rows ty = 4w .. 4w+3 (16 lanes each); columns tx + 16 j: two j make one 32-bit word
+        const int lane = tid & 63, g = lane >> 4;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int64_t n = (int64_t)tn * 64 + ty + 16 * i;
+#pragma unroll
+            for (int jj = 0; jj < 2; jj++) {
+                unsigned field[2];
+#pragma unroll
+                for (int q = 0; q < 2; q++) {
+                    const int64_t m = (int64_t)tm * 64 + tx + 16 * (2 * jj + q);
+                    const bool real = n < a.N && m < a.M;
+                    const unsigned long long bal = __ballot(real && next_sign_bit(a, m, val[i][2 * jj + q]) != 0);
+                    field[q] = (unsigned)(bal >> (16 * g)) & 0xffffu;
+                }
+                const int64_t m32 = (int64_t)tm * 64 + 32 * jj;
+                if (tx == 0 && n < a.N && m32 < a.M)
+                    reinterpret_cast<uint32_t*>(a.out)[out_off + tiled_word_offset(n, m32 >> 5, k_tiles(a.M))] =
+                        __brev(field[0] | (field[1] << 16));
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         const int64_t n = (int64_t)tn * 64 + ty + 16 * i;

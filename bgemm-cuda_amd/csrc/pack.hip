@@ -8,13 +8,6 @@
 
 namespace bgemm {
 
-// Word offset of logical word jw of `row` inside a tiled operand with KT k-tiles.
-__host__ __device__ static inline int64_t tiled_word_offset(int64_t row, int64_t jw, int64_t KT)
-{
-    const int64_t rt = row >> 5, r = row & 31, kt = jw >> 3, h = (jw >> 2) & 1, q = jw & 3;
-    return ((rt * KT + kt) * TILE_U4 + h * 32 + r) * 4 + q;
-}
-
 // One operand to pack.  mode bit3: tiled output written by the row-segment waves (small operands:
 // sixteen times as many, shorter waves).  mode bit0: also write the (sign & nonzero) plane and make plane 0 the
 // nonzero plane.  mode bit1: write the logical layout instead of the tiled one.  mode bit2: the

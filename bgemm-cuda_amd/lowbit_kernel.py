@@ -16,12 +16,12 @@ import torch
 
 import _lib as _b
 from _lib import (MODE_AND, MODE_XOR, MODE_ATTN, MODE_BWTA, MODE_ATTN_X, OUT_I32, OUT_F16, OUT_F32_SCALED,
-                  OUT_F16_SCALED, SRC_F16, SRC_F32, VARIANT_AUTO, VARIANT_VALU, VARIANT_MFMA, VARIANT_MFMA_F4)
+                  OUT_F16_SCALED, OUT_BITS_F32, OUT_BITS_F16, SRC_F16, SRC_F32, VARIANT_AUTO, VARIANT_VALU, VARIANT_MFMA, VARIANT_MFMA_F4)
 
 AND_POP, XOR_POP, ATTN_MM = 0, 1, 2   # lowbit_kernel/csrc/include/configs.h:70-72
 
 __all__ = ["bgemm_linear_forward_cuda", "binary_weight_prepacking", "pack_sign", "pack_ternary",
-           "bgemm_packed_forward", "PackedBits", "save_packed", "load_packed", "AND_POP", "XOR_POP", "ATTN_MM"]
+           "bgemm_packed_forward", "PackedBits", "zeros_packed", "save_packed", "load_packed", "AND_POP", "XOR_POP", "ATTN_MM"]
 
 
 _NULL_CTX = contextlib.nullcontext()
@@ -97,6 +97,13 @@ class PackedBits:
 
     def nbytes(self):
         return self.data.numel() * 4 * (2 if self.ternary else 1)
+
+
+def zeros_packed(rows, K, batch=1, device="cuda"):
+    """An all-zero binary operand of `rows` x `K` bits: the buffer a GEMM with ``bits_out=`` writes the next
+    layer's operand into (its padding must be zero, which later calls of the same shape preserve)."""
+    words = _b.lib().bgemm_tiled_words(rows, K)
+    return PackedBits(torch.zeros((batch, words), dtype=torch.int32, device=device), None, batch, rows, K)
 
 
 def _pack(x, ternary, zero_point=None):
@@ -191,13 +198,18 @@ def logical_from_tiled(packed, plane=0):
 
 
 def bgemm_packed_forward(w, x, mode=MODE_XOR, out_dtype=torch.int32, splitK=1, variant=VARIANT_AUTO, out=None,
-                         scale=None):
+                         scale=None, bits_out=None, next_zero_point=None):
     """GEMM on packed operands: ``out[b,n,m]`` for weight-side ``w`` (M rows) and activation-side
     ``x`` (N rows).  A batch of 1 on either side is shared across the other side's batch.
 
     ``scale=(sw, sa, bias)`` fuses the binary Linear's ``half(acc) * sw * sa (+ bias)``
     (bgemm_linear.py:482-484) into the store: ``sw`` [M], ``sa`` one element, ``bias`` [M] or None,
-    all fp32 (fp32 output) or all fp16 (fp16 output), rounded step by step as torch does."""
+    all fp32 (fp32 output) or all fp16 (fp16 output), rounded step by step as torch does.
+
+    ``bits_out=`` (a PackedBits of N rows x M bits from ``zeros_packed``, with ``scale``) stores no
+    activations at all: the scaled output is centred by ``next_zero_point`` (a one-element tensor of the
+    parameters' type, or None for 0), cast to fp16 and sign-packed as the next binary layer would do it, and
+    those bits are written into ``bits_out``, which is returned."""
     if w.K != x.K:
         raise ValueError("K mismatch: %d vs %d" % (w.K, x.K))
     if (mode == MODE_BWTA) != x.ternary:
@@ -221,11 +233,21 @@ def bgemm_packed_forward(w, x, mode=MODE_XOR, out_dtype=torch.int32, splitK=1, v
             if t.dtype != out_dtype or t.numel() != n or not t.is_contiguous():
                 raise ValueError("%s must be a contiguous %s tensor of %d elements" % (name, out_dtype, n))
         kind = OUT_F32_SCALED if out_dtype == torch.float32 else OUT_F16_SCALED
+        if bits_out is not None:
+            if bits_out.ternary or bits_out.rows != N or bits_out.K != M or bits_out.batch != batch:
+                raise ValueError("bits_out must be a binary PackedBits of %d x %d rows x bits, batch %d" % (N, M, batch))
+            if next_zero_point is not None:
+                _need_cuda(next_zero_point, "next_zero_point")
+                if next_zero_point.dtype != out_dtype or next_zero_point.numel() != 1:
+                    raise ValueError("next_zero_point must be a one-element %s tensor" % out_dtype)
+            kind = OUT_BITS_F32 if out_dtype == torch.float32 else OUT_BITS_F16
+    elif bits_out is not None:
+        raise ValueError("bits_out needs scale=(sw, sa, bias)")
     elif out_dtype not in (torch.int32, torch.half):
         raise ValueError("out_dtype must be torch.int32 or torch.half")
     else:
         kind = OUT_F16 if out_dtype == torch.half else OUT_I32
-    if out is None:
+    if out is None and bits_out is None:
         out = torch.empty((batch, N, M), dtype=out_dtype, device=dev)
     L = _b.lib()
     with _on(dev):
@@ -235,12 +257,19 @@ def bgemm_packed_forward(w, x, mode=MODE_XOR, out_dtype=torch.int32, splitK=1, v
             if part_bytes:
                 ws, cnt = _split_k_buffers(part_bytes, counter_bytes, dev)
         args = (mode, w.data.data_ptr(), x.data.data_ptr(), x.data2.data_ptr() if x.ternary else None,
-                out.data_ptr(), kind, batch, M, N, K,
-                w.words if w.batch > 1 else 0, x.words if x.batch > 1 else 0, N * M, splitK, variant,
+                out.data_ptr() if bits_out is None else bits_out.data.data_ptr(), kind, batch, M, N, K,
+                w.words if w.batch > 1 else 0, x.words if x.batch > 1 else 0,
+                N * M if bits_out is None else bits_out.words, splitK, variant,
                 ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0,
                 cnt.data_ptr() if cnt is not None else None, cnt.numel() if cnt is not None else 0)
         if scale is None:
             _b.check(L.bgemm_packed_forward(*args, _stream()))
+        elif bits_out is not None:
+            _b.check(L.bgemm_packed_forward_bits(*args, sw.data_ptr(), sa.data_ptr(),
+                                                 bias.data_ptr() if bias is not None else None,
+                                                 next_zero_point.data_ptr() if next_zero_point is not None else None,
+                                                 _stream()))
+            return bits_out
         else:
             _b.check(L.bgemm_packed_forward_scaled(*args, sw.data_ptr(), sa.data_ptr(),
                                                    bias.data_ptr() if bias is not None else None, _stream()))

@@ -38,7 +38,10 @@ enum { BGEMM_MODE_AND = 0, BGEMM_MODE_XOR = 1, BGEMM_MODE_ATTN = 2, BGEMM_MODE_B
 /* Output kinds.  I32 = the accumulator; F16 = the integer rounded to nearest even.
  * F32_SCALED / F16_SCALED = the binary Linear's scaling fused into the store (see
  * bgemm_packed_forward_scaled): fp32 resp. fp16 output, parameters of the same type. */
-enum { BGEMM_OUT_I32 = 0, BGEMM_OUT_F16 = 1, BGEMM_OUT_F32_SCALED = 2, BGEMM_OUT_F16_SCALED = 3 };
+enum { BGEMM_OUT_I32 = 0, BGEMM_OUT_F16 = 1, BGEMM_OUT_F32_SCALED = 2, BGEMM_OUT_F16_SCALED = 3,
+       /* the scaled value's sign bit after the next layer's centring, written as a tiled operand
+        * (see bgemm_packed_forward_bits); parameters fp32 resp. fp16 */
+       BGEMM_OUT_BITS_F32 = 4, BGEMM_OUT_BITS_F16 = 5 };
 /* Element type of a floating-point source operand. */
 enum { BGEMM_SRC_F16 = 0, BGEMM_SRC_F32 = 1 };
 /* Kernel family: AUTO picks per shape; VALU = and + popcount on the vector ALU;
@@ -142,6 +145,24 @@ int bgemm_packed_forward_scaled(int mode, const void* W_tiled, const void* X_til
                                 int splitK, int variant, void* ws, size_t ws_bytes,
                                 void* counters, size_t counter_bytes,
                                 const void* sw, const void* sa, const void* bias, void* stream);
+
+/* A binary Linear whose output feeds another binary Linear, with nothing but bits in between: the
+ * scaled output y = half(acc) * sw * sa (+ bias) is evaluated as in bgemm_packed_forward_scaled,
+ * then centred and sign-packed as the next layer would do it (tests/python/bgemm_linear.py:479-482
+ * followed by :140-141 and the pack of ptx_mma.cuh:341-380): bit = sign bit of half_rn(y - *zero_point).
+ * out_tiled receives the tiled operand of N rows x M bits (bgemm_tiled_words(N, M) words per batch
+ * entry, strideOut words apart).  Only real bits are written: the padding of the last row tile and
+ * K-tile must already be zero (zero-fill the buffer once; calls of the same shape keep it valid).
+ * out_dtype: BGEMM_OUT_BITS_F32 (fp32 sw, sa, bias, zero_point) or BGEMM_OUT_BITS_F16 (fp16); all
+ * are DEVICE pointers, bias may be NULL, zero_point NULL means 0.  No counterpart in the reference,
+ * which materialises the fp16 activations between layers. */
+int bgemm_packed_forward_bits(int mode, const void* W_tiled, const void* X_tiled, const void* X2_tiled,
+                              void* out_tiled, int out_dtype, int64_t batch, int64_t M, int64_t N, int64_t K,
+                              int64_t strideW, int64_t strideX, int64_t strideOut,
+                              int splitK, int variant, void* ws, size_t ws_bytes,
+                              void* counters, size_t counter_bytes,
+                              const void* sw, const void* sa, const void* bias, const void* zero_point,
+                              void* stream);
 
 /* ---- fp16-operand call, the drop-in for the reference launcher -----------------------
  * Same argument meaning as bin_pack_linear_kernel (fp6_linear.cu:275-286):

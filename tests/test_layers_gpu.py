@@ -128,6 +128,31 @@ def test_fused_inference_forward_equals_composed_ops(dtype, bias):
         assert torch.equal(lin(x), want)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.half])
+def test_chain_keeps_only_bits_between_layers(dtype):
+    """784 -> 4096 -> 4096 -> 10 with the hidden activations never stored: same output as layer by layer."""
+    torch.manual_seed(11)
+    chain = bl.BGEMMChain(bl.BGEMMLinear(784, 4096, bias=True), bl.BGEMMLinear(4096, 4096, bias=False),
+                          bl.BGEMMLinear(4096, 10, bias=True)).to(DEV).to(dtype)
+    x = torch.randn(128, 784, device=DEV).to(dtype)
+    with torch.no_grad():
+        first = chain(x)                       # initialises the scales layer by layer
+        assert chain._fusable(x)
+        fused = chain(x)
+        h = x
+        for layer in chain:
+            h = layer(h)
+    assert fused.dtype == dtype and tuple(fused.shape) == (128, 10)
+    assert torch.equal(fused, h) and torch.equal(fused, first)
+    x2 = torch.randn(3, 7, 784, device=DEV).to(dtype)      # another batch shape, leading dimensions
+    with torch.no_grad():
+        h = x2
+        for layer in chain:
+            h = layer(h)
+        assert torch.equal(chain(x2), h)
+    assert chain(x).requires_grad                          # with gradients: the ordinary path
+
+
 def test_elastic_module_matches_cpu_twin():
     torch.manual_seed(4)
     x = torch.randn(64, 256, device=DEV)

@@ -447,3 +447,69 @@ def test_packed_file_round_trip_on_device(tmp_path):
     a = lk.bgemm_packed_forward(wp, xt, MODE_BWTA, torch.int32)
     b = lk.bgemm_packed_forward(wp2, xt2, MODE_BWTA, torch.int32)
     assert torch.equal(a, b) and (a[0].cpu().numpy() == dense_ref(MODE_BWTA, w, x)).all()
+
+
+# ------------------------------------------------------------------ binary layer feeding a binary layer: bits out
+@pytest.mark.parametrize("variant", VARIANTS)
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("M,N,K,splitK,batch", [(96, 40, 784, 1, 1),        # general kernel, ragged everything
+                                                 (300, 128, 4096, 1, 1),     # skinny split-K, four tile rows
+                                                 (4100, 5, 300, 1, 3),       # skinny split-K, one tile row, batched
+                                                 (260, 70, 24800, 4, 1),     # cross-block split-K
+                                                 (512, 256, 512, 1, 2),      # whole tiles, batched
+                                                 (10, 128, 4096, 1, 1)])     # a single weight row tile
+def test_bits_output_is_next_layers_operand(oracle, variant, dtype, M, N, K, splitK, batch):
+    """The GEMM writes the next binary layer's packed operand directly: the bits must be those of
+    pack_sign((half(acc) * sw * sa + bias - zp).half()) evaluated op by op."""
+    rng = np.random.default_rng(M * 3 + N * 5 + K)
+    w = rng.standard_normal((batch, M, K)).astype(np.float16)
+    x = rng.standard_normal((batch, N, K)).astype(np.float16)
+    sw = rng.uniform(1e-4, 3e-3, M).astype(dtype)
+    sa = np.asarray(1.7371, dtype=dtype)
+    bias = (0.05 * rng.standard_normal(M)).astype(dtype)
+    wp, xp = lk.pack_sign(to_dev(w)), lk.pack_sign(to_dev(x))
+    for zp_val in (None, 0.013):
+        zp = None if zp_val is None else np.asarray(zp_val, dtype=dtype)
+        out = lk.zeros_packed(N, M, batch, DEV)
+        got = lk.bgemm_packed_forward(wp, xp, MODE_XOR, splitK=splitK, variant=variant, bits_out=out,
+                                      scale=(to_dev(sw), to_dev(sa.reshape(1)), to_dev(bias)),
+                                      next_zero_point=None if zp is None else to_dev(zp.reshape(1)))
+        assert got is out
+        for b in range(batch):
+            acc = oracle.c_bgemm_packed(1, oracle.c_pack_sign(w[b]), oracle.c_pack_sign(x[b]), K)
+            y = oracle.np_scale_epilogue(acc, sw, sa, bias)
+            want = oracle.c_pack_sign(oracle.np_center_to_f16(y, dtype(0) if zp is None else zp))
+            one = lk.PackedBits(out.data[b:b + 1], None, 1, N, M)
+            assert (lk.logical_from_tiled(one).cpu().numpy().view(np.uint32) == want).all(), (zp_val, b)
+        # the padding of the tiled buffer is left as it was: zero
+        words = out.data.cpu().numpy().view(np.uint32)
+        logical_bits = sum(int(np.unpackbits(lk.logical_from_tiled(lk.PackedBits(out.data[b:b + 1], None, 1, N, M))
+                                             .cpu().numpy().view(np.uint8)).sum()) for b in range(batch))
+        assert int(np.unpackbits(words.view(np.uint8)).sum()) == logical_bits
+
+
+def test_bits_output_chains_two_layers_and_empty_k(oracle):
+    """Two binary layers with nothing but bits in between equal the op-by-op chain; K = 0 gives the bits of the bias."""
+    rng = np.random.default_rng(99)
+    N, K, H, M = 128, 784, 512, 96
+    x = to_dev(rng.standard_normal((N, K)).astype(np.float16))
+    w1, w2 = to_dev(rng.standard_normal((H, K)).astype(np.float16)), to_dev(rng.standard_normal((M, H)).astype(np.float16))
+    sw1 = (w1.float().norm(1, 1) / w1.numel()).half()
+    sa, zp = torch.full((1,), 1.25, device=DEV).half(), torch.full((1,), 0.001, device=DEV).half()
+    w1p, w2p = lk.pack_sign(w1), lk.pack_sign(w2)
+    # op by op: fp16 activations materialised, then centred and packed
+    h = lk.bgemm_packed_forward(w1p, lk.pack_sign(x), MODE_XOR, scale=(sw1, sa, None))[0]
+    want = lk.bgemm_packed_forward(w2p, lk.pack_sign(h, zero_point=zp), MODE_XOR, torch.int32)
+    # fused: layer 1 writes layer 2's operand
+    hb = lk.bgemm_packed_forward(w1p, lk.pack_sign(x), MODE_XOR, scale=(sw1, sa, None), bits_out=lk.zeros_packed(N, H, 1, DEV),
+                                 next_zero_point=zp)
+    got = lk.bgemm_packed_forward(w2p, hb, MODE_XOR, torch.int32)
+    assert torch.equal(got, want)
+    # K = 0: acc = 0, so the bits are those of (bias - zp)
+    bias = to_dev(rng.standard_normal(70).astype(np.float32))
+    e = lambda r: lk.PackedBits(torch.empty((1, 0), dtype=torch.int32, device=DEV), None, 1, r, 0)
+    ob = lk.bgemm_packed_forward(e(70), e(9), MODE_XOR, bits_out=lk.zeros_packed(9, 70, 1, DEV),
+                                 scale=(torch.ones(70, device=DEV), torch.ones(1, device=DEV), bias),
+                                 next_zero_point=torch.full((1,), 0.25, device=DEV))
+    wantb = oracle.c_pack_sign(np.tile((bias.cpu().numpy() - np.float32(0.25)).astype(np.float16), (9, 1)))
+    assert (lk.logical_from_tiled(ob).cpu().numpy().view(np.uint32) == wantb).all()
