@@ -251,6 +251,13 @@ class BGEMMLinear(_ScaledBinaryLinear):
             self._wp_key = key
         return self._wp
 
+    def use_packed_weight(self, packed):
+        """Install an already packed, centred weight (for instance one read from a file) as the operand of the
+        inference path; it is used until the float weight changes."""
+        if (packed.rows, packed.K) != tuple(self.weight.shape):
+            raise ValueError(f"packed weight is {packed.rows}x{packed.K} bits, the layer is {tuple(self.weight.shape)}")
+        self._wp, self._wp_key = packed, (self.weight._version, self.weight.data_ptr(), self.weight.dtype)
+
     def _fused_forward(self, x):
         lead = x.shape[:-1]
         xp = lowbit_kernel.pack_sign(x.reshape(-1, x.shape[-1]), zero_point=self.zpa)
