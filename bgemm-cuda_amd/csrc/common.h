@@ -54,7 +54,8 @@ struct GemmArgs {
     void* out; int out_kind;       // BGEMM_OUT_*
     const void* ep_sw; const void* ep_sa; const void* ep_bias;   // scaled output kinds: per-column scale, scalar, bias
     const void* ep_zp;    // bits kinds: the next layer's zero point (null = 0)
-    int vec_store;        // rows of `out` are 16-byte aligned: the epilogue may store four elements per lane
+    int vec_store;        // 0, or the elements per lane the epilogue may store at once: 4 (rows of `out` 16-byte aligned
+                          // for int32, 8-byte for fp16) or 8 (fp16 kinds with rows of a multiple of 8)
     int64_t M, N, K;
     int MT, NT, KT;
     int64_t strideW, strideX, strideC;   // uint4 units for W/X, elements for C
@@ -158,7 +159,7 @@ __device__ __forceinline__ __half scaled_f16(const GemmArgs& a, const int64_t m,
     if (a.ep_bias) r = __float2half_rn(__fadd_rn(__half2float(r), __half2float(reinterpret_cast<const __half*>(a.ep_bias)[m])));
     return r;
 }
-__device__ __forceinline__ int out_elem_shift(const int kind) { return (kind == BGEMM_OUT_F16 || kind == BGEMM_OUT_F16_SCALED) ? 1 : 2; }
+__host__ __device__ __forceinline__ int out_elem_shift(const int kind) { return (kind == BGEMM_OUT_F16 || kind == BGEMM_OUT_F16_SCALED) ? 1 : 2; }
 
 // Bits kinds: the scaled output is not stored; the next binary layer's operand is, i.e. the sign bit
 // of half_rn(y - zp) with y evaluated as above.  The subtraction is exact enough for its sign to

@@ -288,24 +288,77 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
         constexpr int C4 = WM * 8;               // int4 per staged row
         constexpr int NP = 32 * C4 / 64;
         if (a.vec_store && a.out_kind == BGEMM_OUT_I32) {
-            // 16-byte stores: one instruction covers 64 * 4 consecutive elements of the strip
+            // 16-byte stores: one instruction covers 64 * 4 consecutive elements of the strip.  Eight
+            // LDS reads are issued together, then their stores; the address advances by whole rows.
+            constexpr int RSTEP = 64 / C4, CHUNK = NP < 8 ? NP : 8;
+            const int c4 = lane % C4, row0 = lane / C4;
+            const int* sp = st + row0 * ROW_I + c4 * 4;
+            const int64_t m = mcol0 + c4 * 4, dstep = RSTEP * row_bytes;
+            char* dst = out_base + (nrow0 + row0) * row_bytes + (m << 2);
+            if (m < a.M) {
+                if (nrow0 + 32 <= a.N) {             // uniform: the whole strip exists, nothing to mask
 #pragma unroll
-            for (int p = 0; p < NP; p++) {
-                const int idx = p * 64 + lane, row = idx / C4, c4 = idx % C4;
-                const int4 q = *reinterpret_cast<const int4*>(st + row * ROW_I + c4 * 4);
-                const int64_t n = nrow0 + row, m = mcol0 + c4 * 4;
-                if (n < a.N && m < a.M) *reinterpret_cast<int4*>(out_base + n * row_bytes + (m << 2)) = q;
+                    for (int p0 = 0; p0 < NP; p0 += CHUNK) {
+                        int4 q[CHUNK];
+#pragma unroll
+                        for (int p = 0; p < CHUNK; p++) q[p] = *reinterpret_cast<const int4*>(sp + (p0 + p) * RSTEP * ROW_I);
+#pragma unroll
+                        for (int p = 0; p < CHUNK; p++, dst += dstep) *reinterpret_cast<int4*>(dst) = q[p];
+                    }
+                } else {
+                    for (int row = row0; nrow0 + row < a.N; row += RSTEP, sp += RSTEP * ROW_I, dst += dstep)
+                        *reinterpret_cast<int4*>(dst) = *reinterpret_cast<const int4*>(sp);
+                }
+            }
+        } else if (a.vec_store == 8) {
+            // fp16 kinds, rows a multiple of eight long: eight elements and one 16-byte store per lane
+            constexpr int C8 = WM * 4, RSTEP = 64 / C8;          // lanes per staged row, rows per step
+            const int c8 = lane % C8, row0 = lane / C8;
+            const int64_t m = mcol0 + c8 * 8;
+            const int* sp = st + row0 * ROW_I + c8 * 8;
+            char* dst = out_base + (nrow0 + row0) * row_bytes + (m << 1);
+            const int64_t dstep = RSTEP * row_bytes;
+            const bool scaled = a.out_kind == BGEMM_OUT_F16_SCALED;
+            auto put8 = [&](const int4 q0, const int4 q1, char* const to, const bool sc) {
+                const int q[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+                union { __half h[8]; uint4 u; } pk;
+#pragma unroll
+                for (int e = 0; e < 8; e++) pk.h[e] = sc ? scaled_f16(a, m + e, q[e]) : __float2half_rn((float)q[e]);
+                *reinterpret_cast<uint4*>(to) = pk.u;
+            };
+            if (m < a.M) {
+                if (nrow0 + 32 <= a.N && !scaled) {  // uniform: whole strip, plain conversion: reads issued in pairs of rows
+#pragma unroll
+                    for (int r = 0; r < 32 / RSTEP; r += 2, dst += 2 * dstep) {
+                        const int* s0 = sp + r * RSTEP * ROW_I, * s1 = s0 + RSTEP * ROW_I;
+                        const int4 a0 = *reinterpret_cast<const int4*>(s0), a1 = *reinterpret_cast<const int4*>(s0 + 4);
+                        const int4 b0 = *reinterpret_cast<const int4*>(s1), b1 = *reinterpret_cast<const int4*>(s1 + 4);
+                        put8(a0, a1, dst, false);
+                        put8(b0, b1, dst + dstep, false);
+                    }
+                } else {
+#pragma unroll 2
+                    for (int row = row0; row < 32 && nrow0 + row < a.N; row += RSTEP, sp += RSTEP * ROW_I, dst += dstep)
+                        put8(*reinterpret_cast<const int4*>(sp), *reinterpret_cast<const int4*>(sp + 4), dst, scaled);
+                }
             }
         } else if (a.vec_store) {
-#pragma unroll 4
-            for (int p = 0; p < NP; p++) {
-                const int idx = p * 64 + lane, row = idx / C4, c4 = idx % C4;
-                const int4 q = *reinterpret_cast<const int4*>(st + row * ROW_I + c4 * 4);
-                const int64_t n = nrow0 + row, m = mcol0 + c4 * 4;
-                if (n < a.N && m < a.M) {
-                    char* const dst = out_base + n * row_bytes + (m << esz_shift);
+            // four elements per lane; the address advances by whole rows from step to step
+            constexpr int RSTEP = 64 / C4;
+            const int c4 = lane % C4, row0 = lane / C4;
+            const int64_t m = mcol0 + c4 * 4;
+            const int* sp = st + row0 * ROW_I + c4 * 4;
+            char* dst = out_base + (nrow0 + row0) * row_bytes + (m << esz_shift);
+            const int64_t dstep = RSTEP * row_bytes;
+            if (m < a.M) {
+#pragma unroll 2
+                for (int row = row0; row < 32 && nrow0 + row < a.N; row += RSTEP, sp += RSTEP * ROW_I, dst += dstep) {
+                    const int4 q = *reinterpret_cast<const int4*>(sp);
                     union { __half h[4]; uint2 u; } pk;
                     switch (a.out_kind) {
+                    case BGEMM_OUT_I32:
+                        *reinterpret_cast<int4*>(dst) = q;
+                        break;
                     case BGEMM_OUT_F16:
                         pk.h[0] = __float2half_rn((float)q.x); pk.h[1] = __float2half_rn((float)q.y);
                         pk.h[2] = __float2half_rn((float)q.z); pk.h[3] = __float2half_rn((float)q.w);
@@ -344,19 +397,21 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
 struct MfmaCfg { int id, bn, bm; };
 
 // Tile choice, from timings of each configuration over a sweep of shapes: the 256 x 256 tile (one
-// block per CU, hand-pipelined loop) needs at least two rounds of blocks to pay for its long
-// epilogue; 256 x 128 (two resident blocks per CU, so one block's stores overlap the other's main
-// loop) wins from one block per CU upwards; below that the smaller tiles, down to 32 x 128, are
-// chosen so that every CU gets a block.
-static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int splitK, int planes)
+// block per CU, hand-pipelined loop) needs at least two rounds of blocks and a long K (from 32
+// K-tiles) to pay for its long epilogue, during which its CU computes nothing; 256 x 128 (two
+// resident blocks per CU, so one block's stores overlap the other's main loop) wins from one block
+// per CU upwards, except on very short K (under 4 K-tiles), where 128 x 128 keeps more waves in
+// flight for what is then all prologue and epilogue; below that the smaller tiles, down to
+// 32 x 128, are chosen so that every CU gets a block.
+static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int splitK, int planes)
 {
-    // The tile is chosen for the output alone: K ranges are only added (effective_split) where
+    // The tile is chosen for the output and the length of K, not for splitK: K ranges are only added (effective_split) where
     // the tiles of the smallest efficient size still leave compute units idle.
     (void)splitK;
     auto blocks = [&](int bn, int bm) { return batch * cdiv(N, bn) * cdiv(M, bm); };
     if (M <= 64) return blocks(128, 64) >= 512 ? MfmaCfg{7, 128, 64} : MfmaCfg{6, 64, 64};   // narrow outputs
-    if (planes == 1 && blocks(256, 256) >= 512) return {0, 256, 256};
-    if (planes == 1 && blocks(256, 128) >= 256) return {4, 256, 128};
+    if (planes == 1 && blocks(256, 256) >= 512 && KT >= 32) return {0, 256, 256};
+    if (planes == 1 && blocks(256, 128) >= 256 && (KT >= 4 || blocks(128, 128) < 512)) return {4, 256, 128};
     if (blocks(128, 128) >= 512) return {1, 128, 128};
     if (blocks(64, 128) >= 256) return {2, 64, 128};
     return {3, 32, 128};
@@ -365,7 +420,7 @@ static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int splitK, int pla
 void gemm_mfma_ws(int64_t batch, int64_t M, int64_t N, int64_t K, int splitK, int planes, size_t* part_bytes,
                   size_t* counters)
 {
-    const MfmaCfg c = pick_cfg(batch, M, N, splitK, planes);
+    const MfmaCfg c = pick_cfg(batch, M, N, k_tiles(K), splitK, planes);
     const int64_t tiles = batch * cdiv(N, c.bn) * cdiv(M, c.bm);
     const int s = effective_split(tiles, splitK, (int)k_tiles(K));       // as launch_eng will split
     *part_bytes = s > 1 ? (size_t)tiles * s * c.bn * c.bm * 4 : 0;
@@ -396,7 +451,7 @@ template <typename Eng>
 static int launch_eng(const GemmArgs& a_in, hipStream_t st)
 {
     GemmArgs a = a_in;
-    const MfmaCfg cfg = pick_cfg(a.batch, a.M, a.N, a.splitK, a.mc.planes);   // as the workspace was sized
+    const MfmaCfg cfg = pick_cfg(a.batch, a.M, a.N, a.KT, a.splitK, a.mc.planes);   // as the workspace was sized
     a.splitK = effective_split((int64_t)a.batch * cdiv(a.N, cfg.bn) * cdiv(a.M, cfg.bm), a.splitK, a.KT);
     switch (cfg.id) {
     case 0: return launch_cfg<Eng, 2, 2, 4, 4>(a, st);    // 256 x 256
