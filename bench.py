@@ -363,6 +363,8 @@ def main():
     ap.add_argument("--all", action="store_true", help="also time the other benchmark configurations")
     ap.add_argument("--only", choices=["c2", "c3", "c4", "sweep"], help="time just that configuration (for profiling)")
     ap.add_argument("--variant", type=int, default=0, help="0 auto, 1 VALU, 2 MFMA int8, 3 MFMA fp4")
+    ap.add_argument("--split-k", type=int, default=1,
+                    help="splitK of the headline launch: the most K ranges a tile may be computed in (same bits for any value)")
     ap.add_argument("--quick", action="store_true", help="with --only: a tenth of the launches (counter collection)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--floor", action="store_true",
@@ -391,7 +393,7 @@ def main():
         print(json.dumps({"configs": run_extra(args.only, args.quick, args.variant)}), flush=True)
         return
 
-    c5, (w16, x16) = bench_c5(args.steps, args.warmup, variant=args.variant)
+    c5, (w16, x16) = bench_c5(args.steps, args.warmup, splitK=args.split_k, variant=args.variant)
     log("C5:", json.dumps(c5))
     cpu = None if args.no_cpu else cpu_baseline_c5(w16, x16)
     del w16, x16
@@ -409,7 +411,7 @@ def main():
         "dtype": "fp4" if fp4 else "int8",
         "data": "synthetic",
         "config": {"workload": "BASELINE.json config 5: BGEMM M=N=K=8192, {-1,+1}x{-1,+1}, weights and activations "
-                               "prepacked (tiled bit layout), int32 output, splitK=1",
+                               "prepacked (tiled bit layout), int32 output, splitK=%d" % args.split_k,
                    "arithmetic": ("1-bit operands expanded in registers to E2M1 (fp4) MFMA operands, fp32 accumulation "
                                   "of exact integers" if fp4 else
                                   "1-bit operands expanded in registers to int8 MFMA operands, int32 accumulation"),

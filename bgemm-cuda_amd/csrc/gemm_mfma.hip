@@ -210,13 +210,36 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
     int capa[WM];
 #pragma unroll
     for (int j = 0; j < WM; j++) capa[j] = __mul24(mc.c0, bits) + __mul24(mc.ca, pa[j]);
+    // Row terms go through a small LDS table of the wave's own, so that a strip fetches its 16 with four
+    // vector reads issued together (sixteen dependent lane permutes cost a strip two thousand cycles).
+    // All LDS traffic of the epilogue is private to the wave: LDS executes one wave's accesses in
+    // order, so compiler-level wave fences are all the synchronisation it needs, and the waves of a
+    // block drift apart freely (one computes a strip while another's stores drain).
+    __shared__ __align__(16) int rowp[WGN * WGM * WN * 32];
+    int* const rp = rowp + wave * (WN * 32);
+    auto wave_sync = [] {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
+    if (half == 0) {
+#pragma unroll
+        for (int i = 0; i < WN; i++) {
+            int rowterm = __mul24(mc.cb, pb[0][i]);
+            if (PL == 2) rowterm += __mul24(mc.cb2, pb[PL - 1][i]);
+            rp[i * 32 + col] = rowterm;
+        }
+    }
+    wave_sync();
     // this split's share of C for tile row i (recomputed rather than kept: registers are tight)
     auto tile_row_vals = [&](const int i, int (&val)[WM][16]) {
+        int4 r4[4];
+#pragma unroll
+        for (int g = 0; g < 4; g++) r4[g] = *reinterpret_cast<const int4*>(rp + i * 32 + 8 * g + 4 * half);
 #pragma unroll
         for (int v = 0; v < 16; v++) {
-            const int nrow = 8 * (v >> 2) + 4 * half + (v & 3);
-            int rowterm = __mul24(mc.cb, __shfl(pb[0][i], nrow));
-            if (PL == 2) rowterm += __mul24(mc.cb2, __shfl(pb[PL - 1][i], nrow));
+            const int4 q = r4[v >> 2];
+            const int rowterm = (v & 3) == 0 ? q.x : (v & 3) == 1 ? q.y : (v & 3) == 2 ? q.z : q.w;
 #pragma unroll
             for (int j = 0; j < WM; j++) {
                 int t = capa[j] + rowterm + __mul24(mc.cd, Eng::to_int(acc[0][i][j], v));
@@ -249,10 +272,10 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
     }
 
     // ---- store ------------------------------------------------------------------------------
-    // Every 32-row strip of the wave's tile is transposed through LDS, so that lanes own consecutive
-    // outputs of one row.  Only the plain int32 case with 16-byte-aligned rows is unrolled; the
-    // conversions of the other output kinds sit in rolled loops after the staging, which keeps them
-    // out of the fully unrolled part of the kernel.
+    // Every 32-row strip of the wave's tile is transposed through the wave's own LDS area, so that
+    // lanes own consecutive outputs of one row.  Only the plain int32 case with 16-byte-aligned rows
+    // is unrolled; the conversions of the other output kinds sit in rolled loops after the staging,
+    // which keeps them out of the fully unrolled part of the kernel.
     constexpr int ROW_I = WM * 32 + 8;       // staged row stride in ints (+8 keeps the two lane halves on
                                              // different LDS banks)
     __shared__ __align__(16) int stage[WGN * WGM * 32 * ROW_I];
@@ -283,7 +306,7 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
         for (int v = 0; v < 16; v++)
 #pragma unroll
             for (int j = 0; j < WM; j++) st[(8 * (v >> 2) + 4 * half + (v & 3)) * ROW_I + j * 32 + col] = val[j][v];
-        __syncthreads();
+        wave_sync();
         const int64_t nrow0 = (int64_t)(nt0 + i) * 32, mcol0 = (int64_t)mt0 * 32;
         constexpr int C4 = WM * 8;               // int4 per staged row
         constexpr int NP = 32 * C4 / 64;
@@ -389,7 +412,7 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
                     store_out(a, out_off + n * a.M, m, st[row * ROW_I + c]);
             }
         }
-        __syncthreads();
+        wave_sync();                                 // the next strip overwrites the staging area
     }
 }
 
