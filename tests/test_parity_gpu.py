@@ -407,6 +407,37 @@ def test_scaled_epilogue_empty_k_and_errors():
         lk.bgemm_packed_forward(w, x, MODE_XOR, scale=(sw, sa, b.half()))
 
 
+# ------------------------------------------------------------------ random shapes through every path
+@pytest.mark.parametrize("seed", range(96))
+def test_random_shapes_modes_kinds(seed):
+    """Seeded random shapes (ragged in every dimension, batches, K from one bit to twenty K-tiles), every
+    mode, every kernel design, int32 and fp16 stores, any splitK: bit-exact against the +-1 / {0,1} matmul."""
+    rng = np.random.default_rng(7000 + seed)
+    B = int(rng.choice([1, 1, 2, 5]))
+    M = int(rng.choice([rng.integers(1, 64), rng.integers(64, 1500), rng.integers(1500, 6000)]))
+    N = int(rng.choice([rng.integers(1, 17), rng.integers(17, 200), rng.integers(200, 900)]))
+    K = int(rng.choice([rng.integers(1, 256), rng.integers(256, 2048), rng.integers(2048, 5200)]))
+    mode = int(rng.choice([MODE_AND, MODE_XOR, MODE_ATTN, MODE_ATTN_X, MODE_BWTA]))
+    variant = int(rng.choice([VARIANT_AUTO, VARIANT_VALU, VARIANT_MFMA, VARIANT_MFMA_F4]))
+    splitK = int(rng.choice([1, 2, 3, 8]))
+    dt = torch.half if rng.integers(0, 2) else torch.int32
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    w = torch.randn((B, M, K), generator=g, device=DEV, dtype=torch.half)
+    x = torch.randn((B, N, K), generator=g, device=DEV, dtype=torch.half)
+    x[:, :, ::3] = 0
+    ws, xs = torch.where(torch.signbit(w), -1.0, 1.0), torch.where(torch.signbit(x), -1.0, 1.0)
+    want = {MODE_XOR: lambda: xs @ ws.transpose(1, 2),
+            MODE_AND: lambda: (xs < 0).float() @ (ws < 0).float().transpose(1, 2),
+            MODE_ATTN: lambda: xs @ (ws > 0).float().transpose(1, 2),
+            MODE_ATTN_X: lambda: (xs > 0).float() @ ws.transpose(1, 2),
+            MODE_BWTA: lambda: torch.sign(x.float()) @ ws.transpose(1, 2)}[mode]()
+    xin = lk.pack_ternary(x) if mode == MODE_BWTA else lk.pack_sign(x)
+    got = lk.bgemm_packed_forward(lk.pack_sign(w), xin, mode, dt, splitK, variant)
+    case = (B, M, N, K, mode, variant, splitK, dt)
+    assert tuple(got.shape) == (B, N, M), case
+    assert torch.equal(got, want.to(torch.int32) if dt == torch.int32 else want.half()), case
+
+
 # ------------------------------------------------------------------ skinny shapes with many row tiles
 @pytest.mark.parametrize("B,M,N,K", [(40, 4100, 5, 300),      # 5160 row tiles: one per wave, ragged M and K
                                      (70, 4000, 16, 2304),    # 8750 row tiles: two per wave, nine K-tiles
