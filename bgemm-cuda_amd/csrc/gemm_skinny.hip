@@ -113,22 +113,71 @@ __global__ __launch_bounds__(256) void gemm_skinny_stream_kernel(const GemmArgs 
     }
 
     // ---- rank-one terms and store, straight from the accumulators ---------------------------------
+    // The vector ALU is shared by the waves of a SIMD, so what a wave spends here is not hidden behind
+    // the others' loads: row terms and addresses are formed once, and the plain kinds get loops of
+    // their own with nothing but a multiply-add, a conversion and the store per output.
     pb += __shfl_xor(pb, 32);                    // lane r (either half) now holds the popcount of operand row r
 #pragma unroll
     for (int t = 0; t < RT; t++) pa[t] += __shfl_xor(pa[t], 32);
     const ModeCoef mc = a.mc;
-    const int kbits = (int)a.K;
+    const int NV = two ? 8 : 16;                 // rows 16..31 of a two-plane operand are the second plane
+    int colterm[RT];
+    bool col_ok[RT];
+#pragma unroll
+    for (int t = 0; t < RT; t++) {
+        colterm[t] = __mul24(mc.c0, (int)a.K) + __mul24(mc.ca, pa[t]);
+        col_ok[t] = ((int64_t)grp * RT + t) * 32 + r < a.M;
+    }
+    const int64_t m0 = (int64_t)grp * RT * 32 + r;                        // column of tile 0
     const int64_t out_row0 = (int64_t)b * a.strideC;
+    auto row_of = [&](const int v) { return 8 * (v >> 2) + 4 * h + (v & 3); };
+    auto value = [&](const int v, const int t, const int rowterm) {
+        int val = colterm[t] + rowterm + __mul24(mc.cd, Eng::to_int(acc[t], v));
+        if (two) val += __mul24(mc.cd2, Eng::to_int(acc[t], (v + 8) & 15));
+        return val;
+    };
+    // row terms: the popcounts sit in lanes 0..31; both candidates (lane half 0 / 1) are read as
+    // scalars and selected, which costs no LDS round trip
+    auto row_term = [&](const int v) {
+        const int n0 = 8 * (v >> 2) + (v & 3), n1 = n0 + 4;
+        int t0 = __mul24(mc.cb, __builtin_amdgcn_readlane(pb, n0)), t1 = __mul24(mc.cb, __builtin_amdgcn_readlane(pb, n1));
+        if (two) {
+            t0 += __mul24(mc.cb2, __builtin_amdgcn_readlane(pb, (n0 + 16) & 31));
+            t1 += __mul24(mc.cb2, __builtin_amdgcn_readlane(pb, (n1 + 16) & 31));
+        }
+        return h ? t1 : t0;
+    };
+    if (a.out_kind == BGEMM_OUT_I32 || a.out_kind == BGEMM_OUT_F16) {
+        const bool wide = a.out_kind == BGEMM_OUT_I32;
+        const int sh = wide ? 2 : 1;
+        const int64_t row_bytes = a.M << sh;
+        char* const base = reinterpret_cast<char*>(a.out) + ((out_row0 + m0) << sh) + 4 * h * row_bytes;
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            if (v >= NV) break;
+            const int rowterm = row_term(v);
+            if (row_of(v) >= a.N) continue;
+            char* const rowp = base + (8 * (v >> 2) + (v & 3)) * row_bytes;       // uniform offset from the lane's base
+#pragma unroll
+            for (int t = 0; t < RT; t++) {
+                if (!col_ok[t]) continue;
+                const int val = value(v, t, rowterm);
+                if (wide) *reinterpret_cast<int*>(rowp + t * 128) = val;
+                else *reinterpret_cast<__half*>(rowp + t * 64) = __float2half_rn((float)val);
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int v = 0; v < 16; v++) {
-        const int n = 8 * (v >> 2) + 4 * h + (v & 3);
-        const int pbn = __shfl(pb, n), pbn2 = __shfl(pb, (n + 16) & 31);
-        if (n >= a.N || (two && v >= 8)) continue;      // rows 16..31 of a two-plane operand are the second plane
+        if (v >= NV) break;
+        const int n = row_of(v);
+        const int rowterm = row_term(v);
+        if (n >= a.N) continue;
 #pragma unroll
         for (int t = 0; t < RT; t++) {
-            const int64_t m = ((int64_t)grp * RT + t) * 32 + r;
-            const int val = skinny_value(mc, two, kbits, pa[t], pbn, pbn2, Eng::to_int(acc[t], v),
-                                         Eng::to_int(acc[t], (v + 8) & 15));
+            const int64_t m = m0 + t * 32;
+            const int val = value(v, t, rowterm);
             if (bits_kind(a.out_kind))          // a half-wave holds the 32 columns of this row tile for row n
                 store_bits_word(a, b, n, m - r, m < a.M ? next_sign_bit(a, m, val) : 0u);
             else if (m < a.M)
