@@ -137,6 +137,8 @@ static int packed_forward(int mode, const void* W_tiled, const void* X_tiled, co
     if (batch > 1 && strideC < (bits ? bgemm_tiled_words(N, M) : M * N))
         return fail(BGEMM_EINVAL, "bgemm_packed_forward: output stride %lld smaller than one output", (long long)strideC);
     if (bits && ((uintptr_t)out & 3)) return fail(BGEMM_EALIGN, "bgemm_packed_forward_bits: output not 4-byte aligned");
+    if (!bits && ((uintptr_t)out & ((1u << out_elem_shift(out_dtype)) - 1)))
+        return fail(BGEMM_EALIGN, "bgemm_packed_forward: output not aligned to its element size");
     a.out = out; a.out_kind = out_dtype;
     a.ep_sw = sw; a.ep_sa = sa; a.ep_bias = bias; a.ep_zp = zp;
     a.M = M; a.N = N; a.K = K;

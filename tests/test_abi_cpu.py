@@ -62,6 +62,8 @@ def test_layout_sizes():
     (dict(W=None), _lib.ENULL),
     (dict(mode=3), _lib.ENULL),                       # BWTA without the second plane
     (dict(W=0x1008), _lib.EALIGN),
+    (dict(out=0x3002), _lib.EALIGN),                  # int32 output on a 2-byte boundary
+    (dict(out=0x3001, out_dtype=1), _lib.EALIGN),     # fp16 output on an odd address
     (dict(splitK=2), _lib.EWORKSPACE),                # no workspace given
     (dict(splitK=2, ws=0x10000, ws_bytes=1 << 20), _lib.EWORKSPACE),            # no counters given
     (dict(splitK=2, ws=0x10000, ws_bytes=16, cnt=0x20000, cnt_bytes=4096), _lib.EWORKSPACE),
