@@ -37,6 +37,7 @@ SIGNATURES = {
                                            _int, _int, _p, _sz, _p, _sz, _p, _p, _p, _p]),
     "bgemm_packed_forward_bits": (_int, [_int, _p, _p, _p, _p, _int, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
                                          _int, _int, _p, _sz, _p, _sz, _p, _p, _p, _p, _p]),
+    "bgemm_pack_sign_f16_transposed": (_int, [_p, _i64, _i64, _i64, _i64, _i64, _p, _p]),
     "bgemm_f16_workspace_bytes": (_sz, [_i64, _i64, _i64, _int]),
     "bgemm_f16_forward": (_int, [_p, _p, _p, _i64, _i64, _i64, _p, _sz, _int, _int, _p]),
 }

@@ -40,16 +40,25 @@ def _linear_grads(grad_out, x_sign, w_sign):
     return grad_x, grad_w
 
 
-def _batched_packed(x_rows, w_rows, mode):
-    """x_rows [..., N, K], w_rows [..., M, K] with equal leading dimensions -> fp16 [..., N, M]: one launch
-    over all leading dimensions on the batched packed entry point (no per-matrix Python loop)."""
+def _pack_right(mat):
+    """The right-hand operand of ``a @ mat`` (``mat`` is [..., K, M]) as a packed operand of M rows.  A transposed
+    view of a row-major [..., M, K] tensor (``k.transpose(-1, -2)``) is packed from those rows; anything else is
+    packed as it lies by the transposing pack.  No copy either way (bgemm_linear.py:25, :60 copy)."""
+    rows = mat.transpose(-1, -2)
+    if rows.is_contiguous():
+        return lowbit_kernel.pack_sign(rows.reshape(-1, *rows.shape[-2:]))
+    return lowbit_kernel.pack_sign_transposed(mat.reshape(-1, *mat.shape[-2:]))
+
+
+def _batched_packed(x_rows, right, mode):
+    """x_rows [..., N, K] @ right [..., K, M] with equal leading dimensions -> fp16 [..., N, M]: one launch over
+    all leading dimensions on the batched packed entry point (no per-matrix Python loop)."""
     lead = x_rows.shape[:-2]
-    if w_rows.shape[:-2] != lead:
-        raise ValueError("leading dimensions differ: %s vs %s" % (tuple(x_rows.shape), tuple(w_rows.shape)))
+    if right.shape[:-2] != lead:
+        raise ValueError("leading dimensions differ: %s vs %s" % (tuple(x_rows.shape), tuple(right.shape)))
     xp = lowbit_kernel.pack_sign(x_rows.reshape(-1, *x_rows.shape[-2:]))
-    wp = lowbit_kernel.pack_sign(w_rows.reshape(-1, *w_rows.shape[-2:]))
-    out = lowbit_kernel.bgemm_packed_forward(wp, xp, mode, torch.half)
-    return out.reshape(*lead, x_rows.shape[-2], w_rows.shape[-2])
+    out = lowbit_kernel.bgemm_packed_forward(_pack_right(right), xp, mode, torch.half)
+    return out.reshape(*lead, x_rows.shape[-2], right.shape[-1])
 
 
 class bgemm_matmul(torch.autograd.Function):
@@ -60,11 +69,13 @@ class bgemm_matmul(torch.autograd.Function):
     def forward(ctx, matA, matB, instruction='xor'):
         matA, matB = matA.to(torch.half), matB.to(torch.half)
         ctx.save_for_backward(matA, matB)
-        bt = matB.transpose(-1, -2).contiguous()
+        mode = lowbit_kernel.MODE_AND if instruction == 'and' else lowbit_kernel.MODE_XOR
         if matB.dim() > 2:
-            mode = lowbit_kernel.MODE_AND if instruction == 'and' else lowbit_kernel.MODE_XOR
-            return _batched_packed(matA, bt, mode)
-        return _kernel_2d(matA, bt, _instr(instruction))
+            return _batched_packed(matA, matB, mode)
+        lead = matA.shape[:-1]
+        out = lowbit_kernel.bgemm_packed_forward(_pack_right(matB), lowbit_kernel.pack_sign(matA.reshape(-1, matA.shape[-1])),
+                                                 mode, torch.half, splitK=8)[0]
+        return out.reshape(*lead, matB.shape[-1])
 
     @staticmethod
     def backward(ctx, grad_output):
@@ -84,12 +95,13 @@ class bgemm_attn_matmul(torch.autograd.Function):
     def forward(ctx, input1, input2, instruction="attn_mm"):
         input1, input2 = input1.to(torch.half), input2.to(torch.half)
         ctx.save_for_backward(input1, input2)
-        vt = input2.transpose(-1, -2).contiguous()
+        # attn stays as it lies (activation side, {0,1}), the value operand is packed as it lies by the
+        # transposing pack, and the result comes out as [..., S_q, d] directly: none of the reference's
+        # three transposes (bgemm_linear.py:58-61)
         if input1.dim() > 2:
-            # [B, H, S_q, S_k] x [B, H, S_k, d]: attn stays as it lies (activation side, {0,1}), only the
-            # small value operand is transposed; the result comes out as [B, H, S_q, d] directly
-            return _batched_packed(input1, vt, lowbit_kernel.MODE_ATTN_X)
-        return lowbit_kernel.bgemm_linear_forward_cuda(vt, input1, 1, lowbit_kernel.ATTN_MM).T
+            return _batched_packed(input1, input2, lowbit_kernel.MODE_ATTN_X)
+        return lowbit_kernel.bgemm_packed_forward(_pack_right(input2), lowbit_kernel.pack_sign(input1),
+                                                  lowbit_kernel.MODE_ATTN_X, torch.half, splitK=8)[0]
 
     @staticmethod
     def backward(ctx, grad_output):

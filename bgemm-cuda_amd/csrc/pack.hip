@@ -4,6 +4,7 @@
 // bytes are put in tile order through LDS, and the tile leaves as one 16-byte store per lane.
 // Logical output (the reference's row-major words): a wave packs 512 elements of one row.
 #include "common.h"
+#include <type_traits>
 #include <string.h>
 
 namespace bgemm {
@@ -127,20 +128,44 @@ __device__ __forceinline__ void pack_tile(const PackJob& j, const int64_t gw, co
     };
     // the whole tile lies inside the source and every row is 16-byte aligned: plain vector loads, all in flight
     const int64_t esz = f32 ? 4 : 2;
-    const bool interior = rt * TILE_ROWS + TILE_ROWS <= j.rows && kt * TILE_KBITS + TILE_KBITS <= j.K &&
-                          ((((uintptr_t)j.src) | (uintptr_t)(j.ld * esz)) & 15) == 0;
-    if (interior && !f32) {
-        const uint16_t* p = reinterpret_cast<const uint16_t*>(j.src) + row0 * j.ld + k0;
-        uint4 raw[16];
+    const bool rows_in = rt * TILE_ROWS + TILE_ROWS <= j.rows && ((((uintptr_t)j.src) | (uintptr_t)(j.ld * esz)) & 15) == 0;
+    const bool interior = rows_in && kt * TILE_KBITS + TILE_KBITS <= j.K;
+    if (!f32 && rows_in && (interior || (j.K & 7) == 0)) {
+        // also the last K-tile of a K that is a multiple of eight (head size 64: the only tile).  The lanes are
+        // spread over as many 8-element chunks as the tile's rows have here (8, 16 or 32), so a short row
+        // does not leave most of the wave idle: CW lanes per row, 64 / CW rows per step.
+        const int64_t left = j.K - kt * TILE_KBITS;
+        auto rows_by = [&](auto cw_tag) {
+            constexpr int CW = decltype(cw_tag)::value, RI = 64 / CW, STEPS = TILE_ROWS / RI;
+            const int cc = lane & (CW - 1), rs = lane / CW;
+            const int b0 = (((cc >> 4) * 32) * 4 + ((cc >> 2) & 3)) * 4 + (3 - (cc & 3));
+            const uint16_t* p = reinterpret_cast<const uint16_t*>(j.src) + (rt * TILE_ROWS + rs) * j.ld + kt * TILE_KBITS + 8 * cc;
+            const bool live = 8 * cc < left;
+            uint4 raw[STEPS];
 #pragma unroll
-        for (int jj = 0; jj < 16; jj++) raw[jj] = *reinterpret_cast<const uint4*>(p + (int64_t)(2 * jj) * j.ld);
+            for (int jj = 0; jj < STEPS; jj++)
+                raw[jj] = live ? *reinterpret_cast<const uint4*>(p + (int64_t)(RI * jj) * j.ld) : make_uint4(0u, 0u, 0u, 0u);
+            if (CW < 32)                           // the bytes of the chunks this tile does not have
+                for (int i = lane; i < (ternary ? 512 : 256); i += 64) reinterpret_cast<uint32_t*>(lds)[i] = 0u;
 #pragma unroll
-        for (int jj = 0; jj < 16; jj++) {
-            const uint4 v = raw[jj];
-            uint16_t h[8] = {(uint16_t)(v.x & 0xffff), (uint16_t)(v.x >> 16), (uint16_t)(v.y & 0xffff), (uint16_t)(v.y >> 16),
-                             (uint16_t)(v.z & 0xffff), (uint16_t)(v.z >> 16), (uint16_t)(v.w & 0xffff), (uint16_t)(v.w >> 16)};
-            emit(2 * jj + rsub, h, 8);
-        }
+            for (int jj = 0; jj < STEPS; jj++) {
+                const uint4 v = raw[jj];
+                uint16_t h[8] = {(uint16_t)(v.x & 0xffff), (uint16_t)(v.x >> 16), (uint16_t)(v.y & 0xffff), (uint16_t)(v.y >> 16),
+                                 (uint16_t)(v.z & 0xffff), (uint16_t)(v.z >> 16), (uint16_t)(v.w & 0xffff), (uint16_t)(v.w >> 16)};
+                const int r = RI * jj + rs;
+                if (j.zp && live) {
+#pragma unroll
+                    for (int e = 0; e < 8; e++) h[e] = half_bits(__fsub_rn(__half2float(__ushort_as_half(h[e])), zf));
+                }
+                uint32_t sg, nz;
+                bits8(h, sg, nz);
+                lds[b0 + r * 16] = (unsigned char)(ternary ? nz : sg);
+                if (ternary) lds[1024 + b0 + r * 16] = (unsigned char)(sg & nz);
+            }
+        };
+        if (left <= 64) rows_by(std::integral_constant<int, 8>{});
+        else if (left <= 128) rows_by(std::integral_constant<int, 16>{});
+        else rows_by(std::integral_constant<int, 32>{});
     } else if (interior) {
         const float* p = reinterpret_cast<const float*>(j.src) + row0 * j.ld + k0;
 #pragma unroll
@@ -234,7 +259,8 @@ static int make_job(PackJob* j, const void* src, int64_t rows, int64_t K, int64_
     j->rows_out = (mode & 2) ? rows : row_tiles(rows) * TILE_ROWS;
     j->nseg = cdiv(j->KT * TILE_KBITS, 512);
     // a wave per tile streams best, but an operand of a few hundred tiles would leave most SIMDs without one
-    if (!(mode & 2) && row_tiles(rows) * j->KT < 2048) j->mode |= 8;
+    // (measured crossover: 500 to 700 tiles)
+    if (!(mode & 2) && row_tiles(rows) * j->KT < 640) j->mode |= 8;
     j->waves = (j->mode & (2 | 8)) ? j->rows_out * j->nseg : row_tiles(rows) * j->KT;
     return BGEMM_OK;
 }
@@ -302,6 +328,90 @@ extern "C" int bgemm_pack_sign_centered(const void* src, int src_dtype, int64_t 
         return fail(BGEMM_EINVAL, "bgemm_pack_sign_centered: unknown source type %d", src_dtype);
     return pack_common(src, rows, K, ld, dst_tiled, nullptr, src_dtype == BGEMM_SRC_F32 ? 4 : 0, zero_point,
                        (hipStream_t)stream, "bgemm_pack_sign_centered");
+}
+
+// Transposed source ([K][rows] in memory): a wave builds one 32-row x 256-bit tile.  For each of its
+// four words, lane (h, k') reads the 32 consecutive fp16 of source row k = 256 kt + 128 h + 32 q + k'
+// (four 16-byte loads when the source allows, all sixteen in flight), gathers their sign bits into a
+// word (bit r = row r), and the 32 x 32 bit matrix held by the 32 lanes of a wave half is transposed
+// in registers with five masked exchanges: lane r then holds the word of row r, bit k' = column k'.
+__device__ __forceinline__ unsigned transpose32(unsigned w, const int lane)
+{
+#pragma unroll
+    for (int j = 16; j >= 1; j >>= 1) {
+        const unsigned m = j == 16 ? 0x0000ffffu : j == 8 ? 0x00ff00ffu : j == 4 ? 0x0f0f0f0fu : j == 2 ? 0x33333333u : 0x55555555u;
+        const unsigned other = __shfl_xor(w, j);
+        w = (lane & j) ? (w & (m << j)) | ((other >> j) & m) : (w & m) | ((other & m) << j);
+    }
+    return w;
+}
+
+__global__ __launch_bounds__(256) void pack_transposed_kernel(const uint16_t* __restrict__ src, const int64_t rows,
+                                                              const int64_t K, const int64_t ld, const int64_t bstride,
+                                                              uint4* __restrict__ dst, const int64_t tiles_per_matrix,
+                                                              const int64_t KT, const int64_t total_tiles)
+{
+    const int lane = threadIdx.x & 63, h = lane >> 5, kk = lane & 31;
+    const int64_t tile = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (tile >= total_tiles) return;             // whole wave leaves together
+    const int64_t b = tile / tiles_per_matrix, t = tile - b * tiles_per_matrix, rt = t / KT, kt = t - rt * KT;
+    const int64_t r0 = rt * 32, k0 = kt * TILE_KBITS + h * 128 + kk;
+    const uint16_t* p = src + b * bstride + k0 * ld + r0;
+    const bool vec = r0 + 32 <= rows && (((uintptr_t)src | (uintptr_t)(ld * 2) | (uintptr_t)(bstride * 2)) & 15) == 0;
+    unsigned w[4];
+    if (vec) {
+        uint4 raw[4][4];
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+#pragma unroll
+            for (int c = 0; c < 4; c++)
+                raw[q][c] = k0 + q * 32 < K ? reinterpret_cast<const uint4*>(p + (int64_t)q * 32 * ld)[c] : make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            unsigned x = 0;
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                const unsigned d[4] = {raw[q][c].x, raw[q][c].y, raw[q][c].z, raw[q][c].w};
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const unsigned sb = d[e] & 0x80008000u;          // sign bits of two halves
+                    x |= (((sb >> 15) | (sb >> 30)) & 3u) << (8 * c + 2 * e);
+                }
+            }
+            w[q] = x;
+        }
+    } else {
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            unsigned x = 0;
+            if (k0 + q * 32 < K)
+                for (int r = 0; r < 32; r++)
+                    if (r0 + r < rows) x |= (unsigned)(p[(int64_t)q * 32 * ld + r] >> 15) << r;
+            w[q] = x;
+        }
+    }
+    // lane r of each half now takes row r; element k' of a word goes to bit 31 - k'
+#pragma unroll
+    for (int q = 0; q < 4; q++) w[q] = __brev(transpose32(w[q], lane));
+    dst[tile * TILE_U4 + lane] = make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+extern "C" int bgemm_pack_sign_f16_transposed(const void* src, int64_t batch, int64_t rows, int64_t K, int64_t ld,
+                                              int64_t src_batch_stride, void* dst_tiled, void* stream)
+{
+    if (batch < 0 || rows < 0 || K < 0 || ld < rows || src_batch_stride < 0)
+        return fail(BGEMM_EINVAL, "bgemm_pack_sign_f16_transposed: bad shape batch=%lld rows=%lld K=%lld ld=%lld",
+                    (long long)batch, (long long)rows, (long long)K, (long long)ld);
+    if (batch == 0 || rows == 0 || K == 0) return BGEMM_OK;
+    if (!src || !dst_tiled) return fail(BGEMM_ENULL, "bgemm_pack_sign_f16_transposed: null pointer");
+    if (((uintptr_t)src & 1) || ((uintptr_t)dst_tiled & 15))
+        return fail(BGEMM_EALIGN, "bgemm_pack_sign_f16_transposed: source must be 2-byte, destination 16-byte aligned");
+    const int64_t KT = k_tiles(K), per = row_tiles(rows) * KT, total = batch * per, blocks = cdiv(total, 4);
+    if (blocks > 0x7fffffffLL) return fail(BGEMM_EINVAL, "bgemm_pack_sign_f16_transposed: operand too large");
+    hipLaunchKernelGGL(pack_transposed_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       reinterpret_cast<const uint16_t*>(src), rows, K, ld, src_batch_stride,
+                       reinterpret_cast<uint4*>(dst_tiled), per, KT, total);
+    return check_launch("bgemm_pack_sign_f16_transposed");
 }
 
 static int relayout(const void* src, void* dst, int64_t rows, int64_t K, int dir, void* stream, const char* who)

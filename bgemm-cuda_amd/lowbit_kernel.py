@@ -156,6 +156,26 @@ def pack_sign(x, zero_point=None):
     return _pack(x, False, zero_point)
 
 
+def pack_sign_transposed(x):
+    """fp16 ``[K,R]`` / ``[B,K,R]`` -> tiled sign bits of the transposes (``R`` rows of ``K`` bits each), read as
+    they lie: what ``pack_sign(x.transpose(-1, -2).contiguous())`` gives, without the copy.  The right-hand
+    operand of a matmul ``a @ b`` (``b`` is ``[K, M]``) and the value operand of attention are of this kind."""
+    _need_cuda(x, "input")
+    if x.dim() not in (2, 3):
+        raise ValueError("expected a 2-D or 3-D tensor, got %d-D" % x.dim())
+    x = x.to(torch.half)
+    if x.stride(-1) != 1 or x.stride(-2) < x.shape[-1] or (x.dim() == 3 and x.stride(0) < 0):
+        x = x.contiguous()
+    batch = 1 if x.dim() == 2 else x.shape[0]
+    K, rows = x.shape[-2], x.shape[-1]
+    L = _b.lib()
+    d0 = torch.empty((batch, L.bgemm_tiled_words(rows, K)), dtype=torch.int32, device=x.device)
+    with _on(x.device):
+        _b.check(L.bgemm_pack_sign_f16_transposed(x.data_ptr(), batch, rows, K, x.stride(-2),
+                                                  x.stride(0) if x.dim() == 3 else 0, d0.data_ptr(), _stream()))
+    return PackedBits(d0, None, batch, rows, K)
+
+
 def pack_ternary(x):
     """``[R,K]`` / ``[B,R,K]`` -> tiled (nonzero, sign&nonzero) planes of sign(x) in {-1,0,+1}."""
     return _pack(x, True)

@@ -96,6 +96,14 @@ int bgemm_pack_ternary_f16(const void* src, int64_t rows, int64_t K, int64_t ld,
  * was computed on the GPU needs no host read-back), or NULL for 0. */
 int bgemm_pack_sign_centered(const void* src, int src_dtype, int64_t rows, int64_t K, int64_t ld,
                              const void* zero_point, void* dst_tiled, void* stream);
+/* Sign pack of the TRANSPOSE of a batch of fp16 matrices: src holds `batch` matrices of
+ * [K][rows] (element (k, r) at src[b*src_batch_stride + k*ld + r]); matrix b of the result
+ * is the tiled operand of `rows` x K bits at dst_tiled + b*bgemm_tiled_words(rows, K) words.
+ * The right-hand operand of `matA @ matB` (tests/python/bgemm_linear.py:19-25) and the value
+ * operand of `attn @ value` (:55-60), which the reference brings into [rows][K] order with
+ * `.transpose(0, 1).contiguous()` before its kernel can read it, are packed as they lie. */
+int bgemm_pack_sign_f16_transposed(const void* src, int64_t batch, int64_t rows, int64_t K, int64_t ld,
+                                   int64_t src_batch_stride, void* dst_tiled, void* stream);
 /* logical <-> tiled re-layout of already packed bits (device buffers). */
 int bgemm_tile_from_logical(const uint32_t* logical, int64_t rows, int64_t K,
                             void* dst_tiled, void* stream);

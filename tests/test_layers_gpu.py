@@ -27,9 +27,11 @@ def test_bgemm_matmul_and_attn_matmul():
     q, k = torch.randn(32, 768, device=DEV), torch.randn(32, 768, device=DEV)
     attn = bl.bgemm_matmul.apply(q, k.transpose(-1, -2))
     assert torch.equal(attn.float(), torch.matmul(q.sign(), k.sign().T).half().float())
-    # a genuinely contiguous [K, M] right operand also works (the reference mis-reads it)
+    # a genuinely contiguous [K, M] right operand also works (the reference mis-reads it); it is packed as it lies
     kt = k.T.contiguous()
     assert torch.equal(bl.bgemm_matmul.apply(q, kt), attn)
+    assert torch.equal(bl.bgemm_matmul.apply(q.reshape(4, 8, 768), kt), attn.reshape(4, 8, 32))     # leading dimensions
+    assert torch.equal(bl.bgemm_matmul.apply(q, kt, 'and').float(), ((q < 0).float() @ (k < 0).float().T).half().float())
     a = torch.randn(128, 256, device=DEV)
     v = torch.randn(256, 64, device=DEV)
     out = bl.bgemm_attn_matmul.apply(a, v)

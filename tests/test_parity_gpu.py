@@ -109,6 +109,23 @@ def test_pack_strided_and_unaligned(oracle):
         assert (logical.cpu().numpy().view(np.uint32) == want).all()
 
 
+@pytest.mark.parametrize("B,K,R,pad", [(1, 1, 1, 0), (1, 300, 70, 0), (3, 512, 64, 0), (2, 1000, 33, 7), (5, 40, 200, 0)])
+def test_pack_transposed_equals_pack_of_the_transpose(B, K, R, pad):
+    """[B, K, R] sources packed as they lie = the ordinary pack of their transposes (ragged K and R, a row stride
+    larger than R, a batch, -0.0 and NaN sign bits)."""
+    g = torch.Generator(device=DEV).manual_seed(K * 7 + R)
+    big = torch.randn((B, K, R + pad), generator=g, device=DEV, dtype=torch.half)
+    big[:, ::3, ::5] = -0.0
+    big[:, 1::7, 2::3] = float("nan")
+    x = big[:, :, :R]                                         # row stride R + pad
+    want = lk.pack_sign(x.transpose(1, 2).contiguous())
+    got = lk.pack_sign_transposed(x)
+    assert (got.batch, got.rows, got.K) == (B, R, K) and torch.equal(got.data, want.data)
+    assert torch.equal(lk.pack_sign_transposed(x[0]).data, lk.pack_sign(x[0].T.contiguous()).data)
+    # a source whose last dimension is strided is copied first, same bits
+    assert torch.equal(lk.pack_sign_transposed(want_src := x.transpose(1, 2).contiguous().transpose(1, 2)).data, want.data)
+
+
 # ------------------------------------------------------------------ packed GEMM, small and ragged
 SMALL = [(1, 1, 1), (8, 5, 32), (33, 7, 40), (32, 32, 128), (10, 3, 784), (64, 1, 256), (65, 17, 300),
          (130, 70, 1000), (256, 256, 512), (40, 200, 2304),
