@@ -10,7 +10,9 @@ All work is enqueued on the current torch stream through the C ABI in
 include/bgemm_mi355x.h; torch supplies device memory and streams only.
 """
 import contextlib
+import collections
 import struct
+import weakref
 
 import torch
 
@@ -21,7 +23,8 @@ from _lib import (MODE_AND, MODE_XOR, MODE_ATTN, MODE_BWTA, MODE_ATTN_X, OUT_I32
 AND_POP, XOR_POP, ATTN_MM = 0, 1, 2   # lowbit_kernel/csrc/include/configs.h:70-72
 
 __all__ = ["bgemm_linear_forward_cuda", "binary_weight_prepacking", "pack_sign", "pack_ternary",
-           "bgemm_packed_forward", "PackedBits", "zeros_packed", "save_packed", "load_packed", "AND_POP", "XOR_POP", "ATTN_MM"]
+           "pack_sign_transposed", "bgemm_packed_forward", "PackedBits", "zeros_packed", "save_packed", "load_packed",
+           "set_weight_cache", "AND_POP", "XOR_POP", "ATTN_MM"]
 
 
 _NULL_CTX = contextlib.nullcontext()
@@ -296,6 +299,39 @@ def bgemm_packed_forward(w, x, mode=MODE_XOR, out_dtype=torch.int32, splitK=1, v
     return out
 
 
+# Opt-in cache of packed weights for the drop-in call.  The reference's interface takes fp16 weights
+# on every call, so every call packs them again: at decode shapes that is most of the time (reading
+# 90 MB of fp16 to produce 5.6 MB of bits).  With the cache on, a weight tensor that is the same object,
+# at the same version counter, as on an earlier call is not packed again.  Off by default because the
+# version counter only sees writes made through torch: memory changed behind torch's back (another
+# library writing through the raw pointer) would go unnoticed.
+_weight_cache = collections.OrderedDict()
+_weight_cache_entries = 0
+
+
+def set_weight_cache(entries):
+    """Keep the packed form of up to `entries` weight tensors seen by bgemm_linear_forward_cuda (0 = off, the
+    default).  An entry is used again only for the very same tensor object with an unchanged version counter."""
+    global _weight_cache_entries
+    _weight_cache_entries = max(0, int(entries))
+    while len(_weight_cache) > _weight_cache_entries:
+        _weight_cache.popitem(last=False)
+
+
+def _cached_packed_weight(w):
+    key = id(w)
+    hit = _weight_cache.get(key)
+    if hit is not None and hit[0]() is w and hit[1] == w._version and hit[2] == w.data_ptr():
+        _weight_cache.move_to_end(key)
+        return hit[3]
+    packed = pack_sign(w)
+    _weight_cache[key] = (weakref.ref(w), w._version, w.data_ptr(), packed)
+    _weight_cache.move_to_end(key)
+    while len(_weight_cache) > _weight_cache_entries:
+        _weight_cache.popitem(last=False)
+    return packed
+
+
 def bgemm_linear_forward_cuda(in_feats, weights, splitK=1, INSTR=1):
     """Computes BGEMM: half ``in_feats [N,K]``, half ``weights [M,K]`` -> half ``[N,M]``.
 
@@ -310,6 +346,15 @@ def bgemm_linear_forward_cuda(in_feats, weights, splitK=1, INSTR=1):
         raise TypeError("in_feats and weights must be torch.half")   # data_ptr<at::Half> in the reference
     if in_feats.shape[1] != weights.shape[1]:
         raise ValueError("K mismatch: in_feats %s vs weights %s" % (tuple(in_feats.shape), tuple(weights.shape)))
+    if INSTR not in (AND_POP, XOR_POP, ATTN_MM):
+        raise ValueError("INSTR must be 0 (and), 1 (xor) or 2 (attn), got %r" % (INSTR,))
+    if int(splitK) < 1:
+        raise ValueError("splitK must be at least 1, got %r" % (splitK,))
+    if _weight_cache_entries and weights.is_contiguous() and weights.numel() and in_feats.numel():
+        # the same arithmetic on packed operands: the weights' bits come from the cache
+        out = bgemm_packed_forward(_cached_packed_weight(weights), pack_sign(in_feats), int(INSTR), torch.half,
+                                   int(splitK))
+        return out[0]
     x, w = in_feats.contiguous(), weights.contiguous()
     N, K = x.shape
     M = w.shape[0]

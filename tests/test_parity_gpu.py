@@ -315,6 +315,34 @@ def test_dropin_rounds_to_nearest_even(oracle):
     assert (got.view(np.uint16) == want_h.view(np.uint16)).all()
 
 
+def test_dropin_weight_cache_is_opt_in_and_follows_the_tensor():
+    """With the cache on, the drop-in call packs a weight tensor once; a write through torch (version counter)
+    or another tensor object gets a fresh pack; results never differ from the uncached call."""
+    torch.manual_seed(9)
+    x = torch.randn(5, 300, device=DEV, dtype=torch.half)
+    w = torch.randn(70, 300, device=DEV, dtype=torch.half)
+    plain = lk.bgemm_linear_forward_cuda(x, w, 1, 1)
+    assert len(lk._weight_cache) == 0                                  # off by default
+    lk.set_weight_cache(2)
+    try:
+        for instr in (0, 1, 2):
+            assert torch.equal(lk.bgemm_linear_forward_cuda(x, w, 1, instr), lk.bgemm_linear_forward_cuda(x, w.clone(), 1, instr))
+        assert torch.equal(lk.bgemm_linear_forward_cuda(x, w, 4, 1), plain)
+        packed = lk._weight_cache[id(w)][3]
+        assert lk.bgemm_linear_forward_cuda(x, w, 1, 1) is not None and lk._weight_cache[id(w)][3] is packed   # reused
+        w.neg_()                                                        # in-place write: must be packed again
+        assert torch.equal(lk.bgemm_linear_forward_cuda(x, w, 1, 1), -plain)
+        assert lk._weight_cache[id(w)][3] is not packed
+        for _ in range(4):                                              # other tensors push old entries out
+            lk.bgemm_linear_forward_cuda(x, torch.randn_like(w), 1, 1)
+        assert len(lk._weight_cache) <= 2
+        with pytest.raises(ValueError):
+            lk.bgemm_linear_forward_cuda(x, w, 1, 3)
+    finally:
+        lk.set_weight_cache(0)
+    assert len(lk._weight_cache) == 0
+
+
 def test_dropin_argument_errors():
     x = torch.zeros(32, 128, dtype=torch.half, device=DEV)
     with pytest.raises(TypeError):
