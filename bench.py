@@ -217,6 +217,32 @@ def bench_c4_batched(steps, N, B=64):
             "gbs": bytes_alg / ms / 1e6, "ops": ops, "bytes": bytes_alg, "bit_exact": ok}
 
 
+def bench_c4_from_fp16(steps, N, copies=64):
+    """A decode step as a model runs it: fp16 activations in, prepacked W[11008,4096], int32 out.  Timed as two
+    launches (ternary pack, then the packed GEMM) and as the one launch that packs its activations itself; weights
+    rotate over `copies` buffers as in bench_c4."""
+    import torch
+    import lowbit_kernel as lk
+    dev = torch.device("cuda:0")
+    M, K = 11008, 4096
+    g = torch.Generator(device=dev).manual_seed(4200 + N)
+    t = torch.randint(0, 4, (N, K), generator=g, device=dev)
+    x16 = torch.where(t == 0, -1.0, torch.where(t == 3, 1.0, 0.0)).to(torch.half)
+    base = lk.pack_sign(pm1_f16((M, K), 4001, dev))
+    wps = [lk.PackedBits(base.data.clone(), None, 1, M, K) for _ in range(copies)]
+    two = lambda i: lk.bgemm_packed_forward(wps[i % copies], lk.pack_ternary(x16), lk.MODE_BWTA, torch.int32)
+    one = lambda i: lk.bgemm_packed_weight_forward(wps[i % copies], x16, lk.MODE_BWTA, torch.int32)
+    ok = bool(torch.equal(two(0)[0], one(0)))
+    ms_two = time_gpu_graph(two, copies, 2, max(2, steps // copies))
+    ms_one = time_gpu_graph(one, copies, 2, max(2, steps // copies))
+    ms_one_eager, ms_two_eager = time_gpu(one, 20, steps), time_gpu(two, 20, steps)
+    ops = 2.0 * M * N * K
+    bytes_alg = M * K / 8 + 2.0 * N * K + 4.0 * M * N
+    return {"name": "C4 decode step from fp16 activations, W[11008,4096] N=%d (one launch: the kernel packs x itself)" % N,
+            "ms": ms_one, "ms_pack_then_gemm": ms_two, "ms_eager_launch": ms_one_eager, "ms_pack_then_gemm_eager": ms_two_eager,
+            "tops": ops / ms_one / 1e9, "gbs": bytes_alg / ms_one / 1e6, "ops": ops, "bytes": bytes_alg, "bit_exact": ok}
+
+
 def bench_floor():
     """What the hardware allows a kernel of the decode path's shape: the cost of launching an empty kernel,
     of reading one cold 5.6 MB buffer (the packed W[11008,4096]), and the bandwidth a plain read sustains."""
@@ -333,6 +359,9 @@ def run_extra(which, quick=False, variant=0):
                 log(json.dumps(extra[-1]))
         for N in (1, 4, 16):
             extra.append(bench_c4_batched(400 // div, N))
+            log(json.dumps(extra[-1]))
+        for N in (1, 4):
+            extra.append(bench_c4_from_fp16(2000 // div, N))
             log(json.dumps(extra[-1]))
     if which in ("c3", "all"):
         extra.append(bench_c3(200 // div, 20 // div + 1, variant))

@@ -272,11 +272,12 @@ class BGEMMLinear(_ScaledBinaryLinear):
 
     def _fused_forward(self, x):
         lead = x.shape[:-1]
-        xp = lowbit_kernel.pack_sign(x.reshape(-1, x.shape[-1]), zero_point=self.zpa)
         bias = None if self.bias is None else self.bias.detach()
-        # splitK is an upper bound: the library only splits K where the output tiles alone leave CUs idle
-        out = lowbit_kernel.bgemm_packed_forward(self._packed_weight(), xp, lowbit_kernel.MODE_XOR, splitK=8,
-                                                 scale=(self.sw.detach(), self.sa.detach().reshape(1), bias))
+        # a few rows (a decode step): one launch, the kernel centres and packs x itself; more rows: one pack
+        # launch, then the GEMM (the library only splits K where the output tiles alone leave CUs idle)
+        out = lowbit_kernel.bgemm_packed_weight_forward(self._packed_weight(), x.reshape(-1, x.shape[-1]), lowbit_kernel.MODE_XOR,
+                                                        scale=(self.sw.detach(), self.sa.detach().reshape(1), bias),
+                                                        x_zero_point=self.zpa)
         return out.reshape(*lead, self.weight.shape[0])
 
     def forward(self, x):

@@ -53,7 +53,7 @@ __global__ void clear_counters_kernel(uint32_t* c, int64_t n)
 using namespace bgemm;
 
 extern "C" const char* bgemm_last_error(void) { return g_err; }
-extern "C" int bgemm_abi_version(void) { return 4; }
+extern "C" int bgemm_abi_version(void) { return 5; }
 
 static bool ws_query(int mode, int64_t batch, int64_t M, int64_t N, int64_t K, int splitK, int variant,
                      size_t* part, size_t* counters)
@@ -105,12 +105,16 @@ __global__ void fill_empty_bits_kernel(const GemmArgs a)
     reinterpret_cast<uint32_t*>(a.out)[(int64_t)blockIdx.y * a.strideC + tiled_word_offset(n, jw, k_tiles(a.M))] = w;
 }
 
+// Unpacked activations for the decode kernel that packs them itself (null = X_tiled / X2_tiled are used).
+struct RawActivations { const void* src; int f32; int64_t ld; const void* zero_point; };
+
 static int packed_forward(int mode, const void* W_tiled, const void* X_tiled, const void* X2_tiled,
                           void* out, int out_dtype, int64_t batch, int64_t M, int64_t N, int64_t K,
                           int64_t strideW, int64_t strideX, int64_t strideC,
                           int splitK, int variant, void* ws, size_t ws_bytes,
                           void* counters, size_t counter_bytes,
-                          const void* sw, const void* sa, const void* bias, const void* zp, void* stream)
+                          const void* sw, const void* sa, const void* bias, const void* zp, void* stream,
+                          const RawActivations* raw = nullptr)
 {
     g_err[0] = 0;
     GemmArgs a;
@@ -153,7 +157,16 @@ static int packed_forward(int mode, const void* W_tiled, const void* X_tiled, co
                                (hipStream_t)stream, a);
         return check_launch("bgemm_packed_forward: fill");
     }
-    if (!W_tiled || !X_tiled || (a.mc.planes == 2 && !X2_tiled))
+    if (raw) {
+        if (!W_tiled || !raw->src) return fail(BGEMM_ENULL, "bgemm_packed_weight_forward: operand pointer is NULL");
+        if (raw->ld < K) return fail(BGEMM_EINVAL, "bgemm_packed_weight_forward: row stride %lld < K", (long long)raw->ld);
+        if (batch != 1 || !gemm_skinny_fusex_shape(a.mc.planes, M, N) || variant == BGEMM_VARIANT_VALU)
+            return fail(BGEMM_EINVAL, "bgemm_packed_weight_forward: shape M=%lld N=%lld not taken by the decode kernel "
+                                      "(see bgemm_packed_weight_forward_supported)", (long long)M, (long long)N);
+        if ((uintptr_t)raw->src & (raw->f32 ? 3 : 1))
+            return fail(BGEMM_EALIGN, "bgemm_packed_weight_forward: activations not aligned to their element size");
+        a.xsrc = raw->src; a.xsrc_f32 = raw->f32; a.xld = raw->ld; a.xzp = raw->zero_point;
+    } else if (!W_tiled || !X_tiled || (a.mc.planes == 2 && !X2_tiled))
         return fail(BGEMM_ENULL, "bgemm_packed_forward: operand pointer is NULL");
     if (((uintptr_t)W_tiled & 15) || ((uintptr_t)X_tiled & 15) || ((uintptr_t)X2_tiled & 15))
         return fail(BGEMM_EALIGN, "bgemm_packed_forward: operands must be 16-byte aligned");
@@ -165,6 +178,7 @@ static int packed_forward(int mode, const void* W_tiled, const void* X_tiled, co
     a.vec_store = !bits && (M % 4 == 0) && (strideC % 4 == 0) && (((uintptr_t)out & 15) == 0) ? 4 : 0;
     if (a.vec_store && out_elem_shift(a.out_kind) == 1 && M % 8 == 0 && strideC % 8 == 0) a.vec_store = 8;
     const int v = variant == BGEMM_VARIANT_AUTO ? pick_variant(mode, batch, M, N, K) : variant;
+    if (raw) return launch_gemm_skinny(a, (hipStream_t)stream, v == BGEMM_VARIANT_MFMA_F4);
     const bool skinny = v != BGEMM_VARIANT_VALU && gemm_skinny_shape(a.mc.planes, batch, M, N, K);
     if (splitK > 1 && !skinny) {
         size_t part, cnt;
@@ -226,6 +240,28 @@ extern "C" int bgemm_packed_forward_bits(int mode, const void* W_tiled, const vo
                                   "BGEMM_OUT_BITS_F16, got %d", out_dtype);
     return packed_forward(mode, W_tiled, X_tiled, X2_tiled, out_tiled, out_dtype, batch, M, N, K, strideW, strideX,
                           strideOut, splitK, variant, ws, ws_bytes, counters, counter_bytes, sw, sa, bias, zero_point, stream);
+}
+
+extern "C" int bgemm_packed_weight_forward_supported(int mode, int64_t M, int64_t N, int64_t K)
+{
+    ModeCoef mc;
+    return mode_coef(mode, &mc) && M >= 1 && K >= 1 && K < (1LL << 24) && gemm_skinny_fusex_shape(mc.planes, M, N);
+}
+
+extern "C" int bgemm_packed_weight_forward(int mode, const void* W_tiled, const void* x, int x_dtype, int64_t ldx,
+                                           const void* x_zero_point, void* out, int out_dtype,
+                                           int64_t M, int64_t N, int64_t K, int variant,
+                                           const void* sw, const void* sa, const void* bias,
+                                           const void* next_zero_point, void* stream)
+{
+    if (x_dtype != BGEMM_SRC_F16 && x_dtype != BGEMM_SRC_F32)
+        return fail(BGEMM_EINVAL, "bgemm_packed_weight_forward: unknown activation type %d", x_dtype);
+    if (K == 0 || M == 0 || N == 0)      // nothing to pack: the packed entry point's empty cases
+        return packed_forward(mode, W_tiled, nullptr, nullptr, out, out_dtype, 1, M, N, K, 0, 0, 0, 1, variant, nullptr, 0,
+                              nullptr, 0, sw, sa, bias, next_zero_point, stream);
+    const RawActivations raw = {x, x_dtype == BGEMM_SRC_F32, ldx, x_zero_point};
+    return packed_forward(mode, W_tiled, nullptr, nullptr, out, out_dtype, 1, M, N, K, 0, 0, 0, 1, variant, nullptr, 0,
+                          nullptr, 0, sw, sa, bias, next_zero_point, stream, &raw);
 }
 
 // ---- fp16-operand call: pack both operands into the workspace, then the packed GEMM ----

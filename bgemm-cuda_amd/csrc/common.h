@@ -61,6 +61,9 @@ struct GemmArgs {
     int64_t strideW, strideX, strideC;   // uint4 units for W/X, elements for C
     int batch, splitK;
     ModeCoef mc;
+    // activations not packed yet (the decode kernel packs them itself): X/X2 are null and these describe
+    // the [N][K] source; with two planes the ternary planes of sign(x) are formed
+    const void* xsrc; int64_t xld; int xsrc_f32; const void* xzp;
     int32_t* ws_part;     // split-K partial tiles, [batch][tile][split] in register order (scratch)
     uint32_t* ws_cnt;     // split-K arrival counters, one per output tile, zero between calls
 };
@@ -216,6 +219,7 @@ int launch_gemm_mfma(const GemmArgs& a, hipStream_t st, bool fp4);
 int launch_gemm_valu(const GemmArgs& a, hipStream_t st);
 // Skinny shapes (few activation rows): K is split inside the block, no workspace.
 bool gemm_skinny_shape(int planes, int64_t batch, int64_t M, int64_t N, int64_t K);
+bool gemm_skinny_fusex_shape(int planes, int64_t M, int64_t N);
 int launch_gemm_skinny(const GemmArgs& a, hipStream_t st, bool fp4);
 // Split-K needs of each family for a shape: bytes of partial-tile scratch, number of counters.
 // (for the split that will actually be used: zero when the shape is not split at all)

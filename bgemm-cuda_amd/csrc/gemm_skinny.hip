@@ -15,6 +15,7 @@
 //    per wave, for small batches (N <= 128) against a few thousand weight rows.
 #include "common.h"
 #include "mfma_engines.h"
+#include "pack_bits.h"
 
 namespace bgemm {
 
@@ -191,12 +192,18 @@ __global__ __launch_bounds__(256) void gemm_skinny_stream_kernel(const GemmArgs 
 // for shapes whose output has too few tiles to occupy the chip in the general kernel (a batch of
 // 128 rows against a few thousand weight rows): all KW * (weight row tiles) waves work, each on a
 // short K range, instead of a few waves walking all of K.
-template <typename Eng, int KW, int NTL>
-__global__ __launch_bounds__(KW * 64) void gemm_skinny_splitk_kernel(const GemmArgs a)
+// FUSEX: the activations arrive unpacked (fp16 or fp32 rows, optionally minus a zero point): every wave
+// builds the activation tiles of its own K range itself, in LDS, while its weight loads are in flight,
+// which saves the separate pack launch of a decode step (a third of its time).  NTL == 1, batch == 1.
+template <typename Eng, int KW, int NTL, bool FUSEX = false>
+__global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_kernel(const GemmArgs a)
 {
     constexpr int NT = KW * 64;
+    constexpr int MAXT = (NTL == 1 && !FUSEX) ? 4 : 2;
+    static_assert(!FUSEX || NTL == 1, "in-kernel activation packing is built for one tile row");
     __shared__ int sAcc[NTL][16][64];            // accumulator layout of the MFMA: [v][lane]
     __shared__ int sPa[32], sPb[NTL][32];
+    __shared__ __align__(16) unsigned char sX[FUSEX ? KW : 1][FUSEX ? MAXT : 1][FUSEX ? 1024 : 16];
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int h = lane >> 5;
@@ -207,7 +214,8 @@ __global__ __launch_bounds__(KW * 64) void gemm_skinny_splitk_kernel(const GemmA
     split_range(a.KT, KW, wave, &kt0, &kt1);
 
     const uint4* xp[NTL];
-    if (NTL == 1) xp[0] = skinny_x_ptr(a, b, lane);
+    if (FUSEX) xp[0] = nullptr;
+    else if (NTL == 1) xp[0] = skinny_x_ptr(a, b, lane);
     else {
 #pragma unroll
         for (int i = 0; i < NTL; i++)            // tile rows past the end re-read the last one (never stored)
@@ -224,18 +232,92 @@ __global__ __launch_bounds__(KW * 64) void gemm_skinny_splitk_kernel(const GemmA
 #pragma unroll
     for (int i = 0; i < NTL; i++) pb[i] = 0;
 
+    // FUSEX: the activation tiles of this wave's K-tiles are built by the wave in its own LDS area: row n of
+    // the source goes to operand row n (sign bits) or, with two planes, its nonzero bits to row n and
+    // sign & nonzero to row n + 16; everything else in a tile is zero.  Lane (c = lane & 31, lane >> 5) takes
+    // elements 8c .. 8c + 7 of rows (lane >> 5) + 2j.  The loads of the first four rows go out BEFORE the
+    // weight loads (loads return in order: behind them they could only be used once the weights are in),
+    // and are turned into bits while the weights are in flight.
+    float xzf = 0.f;
+    if (FUSEX && a.xzp)
+        xzf = a.xsrc_f32 ? *reinterpret_cast<const float*>(a.xzp) : __half2float(*reinterpret_cast<const __half*>(a.xzp));
+    const int xc = lane & 31, xb0 = tile_byte_of_chunk(xc), xr = lane >> 5;
+    const bool xfast = FUSEX && !a.xsrc_f32 && (a.K & 7) == 0 && ((((uintptr_t)a.xsrc) | (uintptr_t)(a.xld * 2)) & 15) == 0;
+    auto x_put = [&](unsigned char* const t, const int n, uint16_t (&hb)[8]) {
+        uint32_t sg, nz;
+        bits8(hb, sg, nz);
+        if (two) {
+            t[xb0 + n * 16] = (unsigned char)nz;
+            t[xb0 + (n + 16) * 16] = (unsigned char)(sg & nz);
+        } else
+            t[xb0 + n * 16] = (unsigned char)sg;
+    };
+    auto x_rows_slow = [&](unsigned char* const t, const int kt, const int n_from) {
+        const int64_t esz = a.xsrc_f32 ? 4 : 2;
+        for (int n = n_from + xr; n < (int)a.N; n += 2) {
+            uint16_t hb[8];
+            load8_as_half(reinterpret_cast<const char*>(a.xsrc) + (int64_t)n * a.xld * esz, a.xsrc_f32 != 0,
+                          (int64_t)kt * TILE_KBITS + 8 * xc, a.K, a.xzp != nullptr, xzf, hb);
+            x_put(t, n, hb);
+        }
+    };
+
     // the wave's K range is short (K / KW) and requested MAXT K-tiles at a time: the kernel lives
     // on memory-level parallelism
-    constexpr int MAXT = NTL == 1 ? 4 : 2;
     for (int kb = kt0; kb < kt1 || kb == kt0; kb += MAXT) {
-        uint4 xq[MAXT][NTL], wq[MAXT];
+        uint4 xq[MAXT][NTL], wq[MAXT], xraw[FUSEX ? MAXT : 1][FUSEX ? 2 : 1];
         if (kb < kt1) {
+            if (FUSEX && xfast) {
+#pragma unroll
+                for (int q = 0; q < MAXT; q++)
+#pragma unroll
+                    for (int jr = 0; jr < 2; jr++) {
+                        const int n = xr + 2 * jr;
+                        const int64_t k0 = (int64_t)(kb + q) * TILE_KBITS + 8 * xc;
+                        xraw[q][jr] = (kb + q < kt1 && n < (int)a.N && k0 < a.K)
+                                          ? *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(a.xsrc) + (int64_t)n * a.xld + k0)
+                                          : make_uint4(0u, 0u, 0u, 0u);
+                    }
+            }
 #pragma unroll
             for (int q = 0; q < MAXT; q++) {
                 const int64_t off = (int64_t)min(kb + q, kt1 - 1) * TILE_U4;
+                if (!FUSEX) {
 #pragma unroll
-                for (int i = 0; i < NTL; i++) xq[q][i] = xp[i][off];
+                    for (int i = 0; i < NTL; i++) xq[q][i] = xp[i][off];
+                }
                 wq[q] = load_stream(wp + off);
+            }
+            if (FUSEX) {
+#pragma unroll
+                for (int q = 0; q < MAXT; q++) {
+                    if (kb + q >= kt1) break;
+                    unsigned char* const t = sX[wave][q];
+                    for (int i = lane; i < 256; i += 64) reinterpret_cast<uint32_t*>(t)[i] = 0u;
+                    if (xfast) {
+#pragma unroll
+                        for (int jr = 0; jr < 2; jr++) {
+                            const int n = xr + 2 * jr;
+                            const uint4 v = xraw[q][jr];
+                            uint16_t hb[8] = {(uint16_t)(v.x & 0xffff), (uint16_t)(v.x >> 16), (uint16_t)(v.y & 0xffff), (uint16_t)(v.y >> 16),
+                                              (uint16_t)(v.z & 0xffff), (uint16_t)(v.z >> 16), (uint16_t)(v.w & 0xffff), (uint16_t)(v.w >> 16)};
+                            if (a.xzp && (int64_t)(kb + q) * TILE_KBITS + 8 * xc < a.K) {
+#pragma unroll
+                                for (int e = 0; e < 8; e++) hb[e] = half_bits(__fsub_rn(__half2float(__ushort_as_half(hb[e])), xzf));
+                            }
+                            if (n < (int)a.N) x_put(t, n, hb);
+                        }
+                        x_rows_slow(t, kb + q, 4);               // rows from the fifth on, if any
+                    } else
+                        x_rows_slow(t, kb + q, 0);
+                }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+                for (int q = 0; q < MAXT; q++) xq[q][0] = reinterpret_cast<const uint4*>(sX[wave][min(q, kt1 - 1 - kb)])[lane];
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");      // the next chunk overwrites the area
+                __builtin_amdgcn_wave_barrier();
             }
         }
         if (kb == kt0) {
@@ -314,6 +396,20 @@ bool gemm_skinny_shape(int planes, int64_t batch, int64_t M, int64_t N, int64_t 
     return N <= 128 && K >= 2048 && batch * cdiv(N, 64) * cdiv(M, 128) < 256;
 }
 
+template <typename Eng>
+static int launch_splitk_fusex(const GemmArgs& a, hipStream_t st)
+{
+    const int64_t blocks = (int64_t)a.MT;
+    int kw = 1;
+    while (kw < 8 && (kw < a.splitK || blocks * kw < 4096) && kw * 2 <= a.KT) kw *= 2;
+    const dim3 g((unsigned)blocks);
+    if (kw == 1) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 1, 1, true>), g, dim3(64), 0, st, a);
+    else if (kw == 2) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 2, 1, true>), g, dim3(128), 0, st, a);
+    else if (kw == 4) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 4, 1, true>), g, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 8, 1, true>), g, dim3(512), 0, st, a);
+    return check_launch("gemm_skinny");
+}
+
 template <typename Eng, int NTL>
 static int launch_splitk(const GemmArgs& a, hipStream_t st)
 {
@@ -349,8 +445,19 @@ static int launch_stream(const GemmArgs& a, hipStream_t st)
     return check_launch("gemm_skinny");
 }
 
+// Shapes whose activations the decode kernel packs itself: one matrix, up to four activation rows (a
+// decode step; every wave packs the rows for its own K range, and all waves of a SIMD share its vector
+// ALU, so beyond four rows the separate pack launch is faster), few enough weight row tiles that K is
+// split inside the block.
+bool gemm_skinny_fusex_shape(int planes, int64_t M, int64_t N)
+{
+    (void)planes;
+    return N >= 1 && N <= 4 && row_tiles(M) < 4096;
+}
+
 int launch_gemm_skinny(const GemmArgs& a, hipStream_t st, bool fp4)
 {
+    if (a.xsrc) return fp4 ? launch_splitk_fusex<EngF4>(a, st) : launch_splitk_fusex<EngI8>(a, st);
     // Enough row tiles for about four waves on every SIMD: no K split needed (the result does not
     // depend on it).  Two row tiles per wave share one expansion of the activation tiles.
     const int64_t row_tiles = (int64_t)a.batch * a.MT;

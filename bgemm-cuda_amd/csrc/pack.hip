@@ -4,6 +4,7 @@
 // bytes are put in tile order through LDS, and the tile leaves as one 16-byte store per lane.
 // Logical output (the reference's row-major words): a wave packs 512 elements of one row.
 #include "common.h"
+#include "pack_bits.h"
 #include <type_traits>
 #include <string.h>
 
@@ -20,11 +21,6 @@ struct PackJob {
     const void* zp;
     int64_t rows_out, nseg, KT, Kw, waves;
 };
-
-__device__ __forceinline__ uint16_t half_bits(const float f)
-{
-    return __half_as_ushort(__float2half_rn(f));
-}
 
 // Logical output: one wave packs 512 consecutive K elements of one row (16 words).
 __device__ __forceinline__ void pack_wave(const PackJob& j, const int64_t gw, const int lane)
@@ -87,17 +83,6 @@ __device__ __forceinline__ void pack_wave(const PackJob& j, const int64_t gw, co
         const int64_t o = tiled_word_offset(row, jw, j.KT);
         j.dst0[o] = p0;
         if (ternary) j.dst1[o] = p1;
-    }
-}
-
-// Sign (and nonzero) bits of eight fp16 bit patterns, element e at bit 7 - e.
-__device__ __forceinline__ void bits8(const uint16_t (&h)[8], uint32_t& sg, uint32_t& nz)
-{
-    sg = 0; nz = 0;
-#pragma unroll
-    for (int e = 0; e < 8; e++) {
-        sg |= (uint32_t)(h[e] >> 15) << (7 - e);
-        nz |= (uint32_t)((h[e] & 0x7fff) != 0) << (7 - e);
     }
 }
 

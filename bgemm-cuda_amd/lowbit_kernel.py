@@ -23,7 +23,7 @@ from _lib import (MODE_AND, MODE_XOR, MODE_ATTN, MODE_BWTA, MODE_ATTN_X, OUT_I32
 AND_POP, XOR_POP, ATTN_MM = 0, 1, 2   # lowbit_kernel/csrc/include/configs.h:70-72
 
 __all__ = ["bgemm_linear_forward_cuda", "binary_weight_prepacking", "pack_sign", "pack_ternary",
-           "pack_sign_transposed", "bgemm_packed_forward", "PackedBits", "zeros_packed", "save_packed", "load_packed",
+           "pack_sign_transposed", "bgemm_packed_forward", "bgemm_packed_weight_forward", "PackedBits", "zeros_packed", "save_packed", "load_packed",
            "set_weight_cache", "AND_POP", "XOR_POP", "ATTN_MM"]
 
 
@@ -330,6 +330,63 @@ def _cached_packed_weight(w):
     while len(_weight_cache) > _weight_cache_entries:
         _weight_cache.popitem(last=False)
     return packed
+
+
+def bgemm_packed_weight_forward(w, x, mode=MODE_XOR, out_dtype=torch.int32, scale=None, x_zero_point=None,
+                                variant=VARIANT_AUTO):
+    """Prepacked weights ``w`` (M rows) x activations ``x`` as they are, fp16 or fp32 ``[N,K]`` -> ``[N,M]``.
+
+    For the few rows of a decode step (N <= 4) this is ONE launch: the kernel forms the
+    activation bits itself (``MODE_BWTA``: the ternary planes of sign(x); the other modes: sign bits of ``x``
+    or, with ``x_zero_point``, of ``(x - x_zero_point).to(torch.half)``).  Larger batches go through the pack
+    kernel and the packed entry point: same results either way.  ``scale`` as in bgemm_packed_forward."""
+    _need_cuda(x, "x")
+    if x.dim() != 2 or x.shape[1] != w.K:
+        raise ValueError("x must be [N, %d], got %s" % (w.K, tuple(x.shape)))
+    if w.ternary or w.batch != 1:
+        raise ValueError("the weight side is one binary matrix")
+    if x.dtype not in (torch.half, torch.float32):
+        raise TypeError("activations must be fp16 or fp32, got %s" % x.dtype)
+    ternary = mode == MODE_BWTA
+    if ternary and x_zero_point is not None:
+        raise ValueError("a zero point is only taken by the sign modes")
+    if x_zero_point is not None:
+        _need_cuda(x_zero_point, "x_zero_point")
+        if x_zero_point.numel() != 1:
+            raise TypeError("x_zero_point must be a one-element tensor")
+        x_zero_point = x_zero_point.detach().to(x.dtype)
+    N, K, M = x.shape[0], w.K, w.rows
+    L = _b.lib()
+    if not (N and M and K and L.bgemm_packed_weight_forward_supported(mode, M, N, K)) or variant == VARIANT_VALU:
+        xp = pack_ternary(x) if ternary else pack_sign(x, zero_point=x_zero_point)
+        return bgemm_packed_forward(w, xp, mode, out_dtype, 8, variant, scale=scale)[0]
+    if x.stride(1) != 1 or x.stride(0) < K:
+        x = x.contiguous()
+    sw = sa = bias = None
+    if scale is not None:
+        sw, sa, bias = scale
+        out_dtype = sw.dtype
+        if out_dtype not in (torch.float32, torch.half):
+            raise TypeError("scales must be fp32 or fp16")
+        for name, t, n in (("sw", sw, M), ("sa", sa, 1), ("bias", bias, M)):
+            if t is None and name == "bias":
+                continue
+            _need_cuda(t, name)
+            if t.dtype != out_dtype or t.numel() != n or not t.is_contiguous():
+                raise ValueError("%s must be a contiguous %s tensor of %d elements" % (name, out_dtype, n))
+        kind = OUT_F32_SCALED if out_dtype == torch.float32 else OUT_F16_SCALED
+    elif out_dtype not in (torch.int32, torch.half):
+        raise ValueError("out_dtype must be torch.int32 or torch.half")
+    else:
+        kind = OUT_F16 if out_dtype == torch.half else OUT_I32
+    out = torch.empty((N, M), dtype=out_dtype, device=x.device)
+    with _on(x.device):
+        _b.check(L.bgemm_packed_weight_forward(
+            mode, w.data.data_ptr(), x.data_ptr(), SRC_F32 if x.dtype == torch.float32 else SRC_F16, x.stride(0),
+            x_zero_point.data_ptr() if x_zero_point is not None else None, out.data_ptr(), kind, M, N, K, variant,
+            sw.data_ptr() if sw is not None else None, sa.data_ptr() if sa is not None else None,
+            bias.data_ptr() if bias is not None else None, None, _stream()))
+    return out
 
 
 def bgemm_linear_forward_cuda(in_feats, weights, splitK=1, INSTR=1):

@@ -172,6 +172,22 @@ int bgemm_packed_forward_bits(int mode, const void* W_tiled, const void* X_tiled
                               const void* sw, const void* sa, const void* bias, const void* zero_point,
                               void* stream);
 
+/* Decode step with the activations as they come out of the previous layer: prepacked weights x
+ * fp16 or fp32 activations [N][K] (row stride ldx elements), one launch.  The kernel forms the sign bits
+ * (with BGEMM_MODE_BWTA the ternary planes of sign(x)) itself, from `x - *x_zero_point` rounded to fp16
+ * when a zero point is given: bgemm_pack_sign_centered / bgemm_pack_ternary_f16 followed by the packed
+ * entry point (tests/python/bgemm_linear.py:479-484 for a batch of a few rows), without the pack launch.
+ * Any output kind: out_dtype BGEMM_OUT_I32 / F16 (sw, sa, bias, next_zero_point NULL), the scaled kinds
+ * (sw, sa; bias optional) or the bits kinds (also next_zero_point, optional).  Only shapes the decode
+ * kernel takes this way (N <= 4 rows, M < 131072): ask _supported() first; other shapes
+ * return BGEMM_EINVAL and go through the pack entry points and bgemm_packed_forward*. */
+int bgemm_packed_weight_forward_supported(int mode, int64_t M, int64_t N, int64_t K);
+int bgemm_packed_weight_forward(int mode, const void* W_tiled, const void* x, int x_dtype, int64_t ldx,
+                                const void* x_zero_point, void* out, int out_dtype,
+                                int64_t M, int64_t N, int64_t K, int variant,
+                                const void* sw, const void* sa, const void* bias,
+                                const void* next_zero_point, void* stream);
+
 /* ---- fp16-operand call, the drop-in for the reference launcher -----------------------
  * Same argument meaning as bin_pack_linear_kernel (fp6_linear.cu:275-286):
  * W = weights half [M][K], X = in_feats half [N][K], C = half [N][M], INSTR in {0,1,2}.

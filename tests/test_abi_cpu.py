@@ -29,7 +29,7 @@ def test_header_symbols_exported():
 
 def test_layout_sizes():
     L = _lib.lib()
-    assert L.bgemm_abi_version() == _lib.ABI_VERSION == 4
+    assert L.bgemm_abi_version() == _lib.ABI_VERSION == 5
     assert L.bgemm_tiled_words(1, 1) == 256
     assert L.bgemm_tiled_words(32, 256) == 256
     assert L.bgemm_tiled_words(33, 257) == 4 * 256
@@ -84,6 +84,29 @@ def test_packed_forward_rejects(kwargs, code):
     assert L.bgemm_last_error()            # a message was recorded
     with pytest.raises(ValueError):
         _lib.check(rc)
+
+
+def test_decode_entry_states_its_shapes_and_rejects_others():
+    L = _lib.lib()
+    assert L.bgemm_packed_weight_forward_supported(1, 11008, 1, 4096) == 1
+    assert L.bgemm_packed_weight_forward_supported(1, 11008, 4, 4096) == 1
+    assert L.bgemm_packed_weight_forward_supported(1, 11008, 5, 4096) == 0           # beyond a few rows: pack kernel first
+    assert L.bgemm_packed_weight_forward_supported(3, 11008, 4, 4096) == 1           # ternary planes
+    assert L.bgemm_packed_weight_forward_supported(3, 11008, 17, 4096) == 0
+    assert L.bgemm_packed_weight_forward_supported(1, 131072, 1, 4096) == 0          # streamed, not split in the block
+    assert L.bgemm_packed_weight_forward_supported(9, 64, 1, 64) == 0
+    names = ("mode", "W", "x", "dt", "ld", "zp", "out", "od", "M", "N", "K", "v", "sw", "sa", "b", "nz", "st")
+    base = dict(mode=1, W=0x1000, x=0x2000, dt=0, ld=4096, zp=None, out=0x3000, od=0, M=64, N=4, K=4096, v=0, sw=None,
+                sa=None, b=None, nz=None, st=None)
+    call = lambda **k: L.bgemm_packed_weight_forward(*[{**base, **k}[n] for n in names])
+    assert call(N=64) == _lib.EINVAL           # not a decode shape
+    assert call(dt=7) == _lib.EINVAL
+    assert call(ld=100) == _lib.EINVAL         # row stride shorter than K
+    assert call(x=None) == _lib.ENULL
+    assert call(x=0x2001) == _lib.EALIGN
+    assert call(od=2) == _lib.ENULL            # scaled kind without scales
+    assert call(v=1) == _lib.EINVAL            # the VALU design has no such kernel
+    assert call(N=0) == 0 and call(M=0) == 0   # nothing to do
 
 
 def test_empty_problems_are_ok_without_launch():

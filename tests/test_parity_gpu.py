@@ -452,6 +452,47 @@ def test_scaled_epilogue_empty_k_and_errors():
         lk.bgemm_packed_forward(w, x, MODE_XOR, scale=(sw, sa, b.half()))
 
 
+# ------------------------------------------------------------------ decode step on unpacked activations
+@pytest.mark.parametrize("variant", [VARIANT_AUTO, VARIANT_MFMA, VARIANT_MFMA_F4])
+@pytest.mark.parametrize("M,N,K", [(11008, 1, 4096), (4100, 4, 1000), (300, 2, 40), (64, 4, 2500), (1000, 3, 256), (33, 1, 8), (500, 16, 512)])
+def test_decode_step_packs_its_own_activations(variant, M, N, K):
+    """One launch on fp16 / fp32 activations = pack launch + packed GEMM, bit for bit: every mode, ternary planes,
+    zero point, strided rows, scaled output."""
+    g = torch.Generator(device=DEV).manual_seed(M + 7 * N + K)
+    w = torch.randn((M, K), generator=g, device=DEV, dtype=torch.half)
+    wide = torch.randn((N, K + 24), generator=g, device=DEV, dtype=torch.float32)
+    wide[:, ::4] = 0
+    wide[:, 1::9] = -0.0
+    wp = lk.pack_sign(w)
+    for dt in (torch.half, torch.float32):
+        x = wide.to(dt)[:, 8:8 + K]                       # row stride K + 24, rows not 16-byte aligned for odd K
+        for mode in (MODE_XOR, MODE_AND, MODE_ATTN, MODE_ATTN_X, MODE_BWTA):
+            if mode == MODE_BWTA and N > 16:
+                continue
+            xp = lk.pack_ternary(x) if mode == MODE_BWTA else lk.pack_sign(x)
+            want = lk.bgemm_packed_forward(wp, xp, mode, torch.int32, 1, variant)[0]
+            assert torch.equal(lk.bgemm_packed_weight_forward(wp, x, mode, torch.int32, variant=variant), want), (dt, mode)
+        zp = x.mean().reshape(1)
+        sw = (torch.rand(M, generator=g, device=DEV) + 0.5).to(dt)
+        sa, bias = torch.tensor([0.37], device=DEV, dtype=dt), torch.randn(M, generator=g, device=DEV).to(dt)
+        want = lk.bgemm_packed_forward(wp, lk.pack_sign(x, zero_point=zp), MODE_XOR, splitK=1, variant=variant, scale=(sw, sa, bias))[0]
+        got = lk.bgemm_packed_weight_forward(wp, x, MODE_XOR, scale=(sw, sa, bias), x_zero_point=zp, variant=variant)
+        assert got.dtype == dt and torch.equal(got, want), dt
+    assert torch.equal(lk.bgemm_packed_weight_forward(wp, x, MODE_XOR, torch.half), lk.bgemm_packed_forward(wp, lk.pack_sign(x), MODE_XOR, torch.half)[0])
+
+
+def test_decode_step_larger_batches_fall_back_to_two_launches():
+    g = torch.Generator(device=DEV).manual_seed(3)
+    w = torch.randn((500, 700), generator=g, device=DEV, dtype=torch.half)
+    x = torch.randn((77, 700), generator=g, device=DEV, dtype=torch.half)
+    wp = lk.pack_sign(w)
+    assert torch.equal(lk.bgemm_packed_weight_forward(wp, x, MODE_XOR), lk.bgemm_packed_forward(wp, lk.pack_sign(x), MODE_XOR)[0])
+    xt = torch.sign(x[:20])
+    assert torch.equal(lk.bgemm_packed_weight_forward(wp, xt, MODE_BWTA), lk.bgemm_packed_forward(wp, lk.pack_ternary(xt), MODE_BWTA)[0])
+    with pytest.raises(ValueError):
+        lk.bgemm_packed_weight_forward(wp, x[:, :100], MODE_XOR)
+
+
 # ------------------------------------------------------------------ random shapes through every path
 @pytest.mark.parametrize("seed", range(96))
 def test_random_shapes_modes_kinds(seed):
