@@ -332,6 +332,9 @@ def _cached_packed_weight(w):
     return packed
 
 
+_decode_shapes = {}       # (mode, M, N, K) -> does the decode kernel take unpacked activations of this shape
+
+
 def bgemm_packed_weight_forward(w, x, mode=MODE_XOR, out_dtype=torch.int32, scale=None, x_zero_point=None,
                                 variant=VARIANT_AUTO):
     """Prepacked weights ``w`` (M rows) x activations ``x`` as they are, fp16 or fp32 ``[N,K]`` -> ``[N,M]``.
@@ -357,7 +360,10 @@ def bgemm_packed_weight_forward(w, x, mode=MODE_XOR, out_dtype=torch.int32, scal
         x_zero_point = x_zero_point.detach().to(x.dtype)
     N, K, M = x.shape[0], w.K, w.rows
     L = _b.lib()
-    if not (N and M and K and L.bgemm_packed_weight_forward_supported(mode, M, N, K)) or variant == VARIANT_VALU:
+    one_launch = _decode_shapes.get((mode, M, N, K))
+    if one_launch is None:
+        one_launch = _decode_shapes[(mode, M, N, K)] = bool(N and M and K and L.bgemm_packed_weight_forward_supported(mode, M, N, K))
+    if not one_launch or variant == VARIANT_VALU:
         xp = pack_ternary(x) if ternary else pack_sign(x, zero_point=x_zero_point)
         return bgemm_packed_forward(w, xp, mode, out_dtype, 8, variant, scale=scale)[0]
     if x.stride(1) != 1 or x.stride(0) < K:
