@@ -243,6 +243,13 @@ __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_ker
         xzf = a.xsrc_f32 ? *reinterpret_cast<const float*>(a.xzp) : __half2float(*reinterpret_cast<const __half*>(a.xzp));
     const int xc = lane & 31, xb0 = tile_byte_of_chunk(xc), xr = lane >> 5;
     const bool xfast = FUSEX && !a.xsrc_f32 && (a.K & 7) == 0 && ((((uintptr_t)a.xsrc) | (uintptr_t)(a.xld * 2)) & 15) == 0;
+    auto x_put_bits = [&](unsigned char* const t, const int n, const uint32_t sg, const uint32_t nz) {
+        if (two) {
+            t[xb0 + n * 16] = (unsigned char)nz;
+            t[xb0 + (n + 16) * 16] = (unsigned char)(sg & nz);
+        } else
+            t[xb0 + n * 16] = (unsigned char)sg;
+    };
     auto x_put = [&](unsigned char* const t, const int n, uint16_t (&hb)[8]) {
         uint32_t sg, nz;
         bits8(hb, sg, nz);
@@ -299,13 +306,18 @@ __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_ker
                         for (int jr = 0; jr < 2; jr++) {
                             const int n = xr + 2 * jr;
                             const uint4 v = xraw[q][jr];
-                            uint16_t hb[8] = {(uint16_t)(v.x & 0xffff), (uint16_t)(v.x >> 16), (uint16_t)(v.y & 0xffff), (uint16_t)(v.y >> 16),
-                                              (uint16_t)(v.z & 0xffff), (uint16_t)(v.z >> 16), (uint16_t)(v.w & 0xffff), (uint16_t)(v.w >> 16)};
+                            if (n >= (int)a.N) continue;
                             if (a.xzp && (int64_t)(kb + q) * TILE_KBITS + 8 * xc < a.K) {
+                                uint16_t hb[8] = {(uint16_t)(v.x & 0xffff), (uint16_t)(v.x >> 16), (uint16_t)(v.y & 0xffff), (uint16_t)(v.y >> 16),
+                                                  (uint16_t)(v.z & 0xffff), (uint16_t)(v.z >> 16), (uint16_t)(v.w & 0xffff), (uint16_t)(v.w >> 16)};
 #pragma unroll
                                 for (int e = 0; e < 8; e++) hb[e] = half_bits(__fsub_rn(__half2float(__ushort_as_half(hb[e])), xzf));
+                                x_put(t, n, hb);
+                            } else {
+                                uint32_t sg, nz;
+                                bits8(v, sg, nz);
+                                x_put_bits(t, n, sg, nz);
                             }
-                            if (n < (int)a.N) x_put(t, n, hb);
                         }
                         x_rows_slow(t, kb + q, 4);               // rows from the fifth on, if any
                     } else

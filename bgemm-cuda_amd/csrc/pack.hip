@@ -138,12 +138,13 @@ __device__ __forceinline__ void pack_tile(const PackJob& j, const int64_t gw, co
                 uint16_t h[8] = {(uint16_t)(v.x & 0xffff), (uint16_t)(v.x >> 16), (uint16_t)(v.y & 0xffff), (uint16_t)(v.y >> 16),
                                  (uint16_t)(v.z & 0xffff), (uint16_t)(v.z >> 16), (uint16_t)(v.w & 0xffff), (uint16_t)(v.w >> 16)};
                 const int r = RI * jj + rs;
+                uint32_t sg, nz;
                 if (j.zp && live) {
 #pragma unroll
                     for (int e = 0; e < 8; e++) h[e] = half_bits(__fsub_rn(__half2float(__ushort_as_half(h[e])), zf));
-                }
-                uint32_t sg, nz;
-                bits8(h, sg, nz);
+                    bits8(h, sg, nz);
+                } else
+                    bits8(v, sg, nz);
                 lds[b0 + r * 16] = (unsigned char)(ternary ? nz : sg);
                 if (ternary) lds[1024 + b0 + r * 16] = (unsigned char)(sg & nz);
             }

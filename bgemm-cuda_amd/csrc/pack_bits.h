@@ -21,6 +21,23 @@ __device__ __forceinline__ void bits8(const uint16_t (&h)[8], uint32_t& sg, uint
     }
 }
 
+// The same for eight fp16 as they come out of one 16-byte load (element 2i in the low half of word i),
+// two halves at a time: a half is nonzero iff adding 0x7fff to its low 15 bits reaches bit 15.
+__device__ __forceinline__ void bits8(const uint4 v, uint32_t& sg, uint32_t& nz)
+{
+    const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+    sg = 0; nz = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t s = d[i] & 0x80008000u;
+        const uint32_t u = d[i] & 0x7fff7fffu;
+        const uint32_t z = ((u + 0x7fff7fffu) | u) & 0x80008000u;
+        sg |= (s >> (8 + 2 * i)) | (s >> (25 + 2 * i));          // low half -> bit 7 - 2i, high half -> bit 6 - 2i
+        nz |= (z >> (8 + 2 * i)) | (z >> (25 + 2 * i));
+    }
+    sg &= 0xffu; nz &= 0xffu;
+}
+
 // fp16 bit patterns of elements k0 .. k0 + 7 of one source row (fp16, or fp32 rounded to fp16 as
 // `.to(torch.half)` rounds), after subtracting the zero point if there is one; elements from K on
 // read as +0.0.  `row` points at the row's first element.
