@@ -270,14 +270,34 @@ class BGEMMLinear(_ScaledBinaryLinear):
             raise ValueError(f"packed weight is {packed.rows}x{packed.K} bits, the layer is {tuple(self.weight.shape)}")
         self._wp, self._wp_key = packed, (self.weight._version, self.weight.data_ptr(), self.weight.dtype)
 
+    def _inference_state(self):
+        """Detached views of the parameters for the inference path, rebuilt only when a parameter is replaced or
+        moved (new object or new storage); in-place updates show through the views."""
+        key = (id(self.sw), self.sw.data_ptr(), id(self.sa), self.sa.data_ptr(), id(self.bias),
+               None if self.bias is None else self.bias.data_ptr(), id(self.zpa), self.zpa.data_ptr(), self.weight.dtype)
+        st = self.__dict__.get("_inf")
+        if st is None or st[0] != key:
+            dt = self.weight.dtype
+            sw, sa = self.sw.detach().contiguous(), self.sa.detach().reshape(1)
+            bias = None if self.bias is None else self.bias.detach().contiguous()
+            zpa = self.zpa.detach().to(dt).reshape(1)
+            same = self.zpa.dtype == dt           # otherwise zpa above is a copy: refresh it on every call
+            st = self.__dict__["_inf"] = (key, sw, sa, bias, zpa if same else None)
+        return st
+
     def _fused_forward(self, x):
         lead = x.shape[:-1]
-        bias = None if self.bias is None else self.bias.detach()
+        _, sw, sa, bias, zpa = self._inference_state()
+        if zpa is None:
+            zpa = self.zpa.detach().to(x.dtype).reshape(1)
+        x2 = x.reshape(-1, x.shape[-1])
+        wp = self._packed_weight()
         # a few rows (a decode step): one launch, the kernel centres and packs x itself; more rows: one pack
         # launch, then the GEMM (the library only splits K where the output tiles alone leave CUs idle)
-        out = lowbit_kernel.bgemm_packed_weight_forward(self._packed_weight(), x.reshape(-1, x.shape[-1]), lowbit_kernel.MODE_XOR,
-                                                        scale=(self.sw.detach(), self.sa.detach().reshape(1), bias),
-                                                        x_zero_point=self.zpa)
+        if x2.shape[0] <= 4 and x2.is_contiguous() and lowbit_kernel.decode_shape_supported(lowbit_kernel.MODE_XOR, wp.rows, x2.shape[0], wp.K):
+            out = lowbit_kernel.decode_linear_launch(wp, x2, sw, sa, bias, zpa)
+        else:
+            out = lowbit_kernel.bgemm_packed_weight_forward(wp, x2, lowbit_kernel.MODE_XOR, scale=(sw, sa, bias), x_zero_point=zpa)
         return out.reshape(*lead, self.weight.shape[0])
 
     def forward(self, x):

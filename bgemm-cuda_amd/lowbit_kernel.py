@@ -343,6 +343,29 @@ def _cached_packed_weight(w):
 _decode_shapes = {}       # (mode, M, N, K) -> does the decode kernel take unpacked activations of this shape
 
 
+def decode_linear_launch(w, x, sw, sa, bias, zero_point):
+    """The one-launch binary Linear of a decode step with every check left to the caller (the layers validate
+    their parameters once, not on every token): ``x`` is a contiguous [N<=4, K] CUDA tensor of the parameters'
+    dtype (fp16 or fp32), ``sw``/``sa``/``bias``/``zero_point`` contiguous tensors of that dtype (bias may be
+    None), the shape one that ``bgemm_packed_weight_forward_supported`` accepts.  Returns [N, M]."""
+    dt = x.dtype
+    f32 = dt == torch.float32
+    out = torch.empty((x.shape[0], w.rows), dtype=dt, device=x.device)
+    with _on(x.device):
+        _b.check(_b.lib().bgemm_packed_weight_forward(
+            MODE_XOR, w.data.data_ptr(), x.data_ptr(), SRC_F32 if f32 else SRC_F16, x.shape[1], zero_point.data_ptr(),
+            out.data_ptr(), OUT_F32_SCALED if f32 else OUT_F16_SCALED, w.rows, x.shape[0], w.K, VARIANT_AUTO,
+            sw.data_ptr(), sa.data_ptr(), bias.data_ptr() if bias is not None else None, None, _stream()))
+    return out
+
+
+def decode_shape_supported(mode, M, N, K):
+    one_launch = _decode_shapes.get((mode, M, N, K))
+    if one_launch is None:
+        one_launch = _decode_shapes[(mode, M, N, K)] = bool(N and M and K and _b.lib().bgemm_packed_weight_forward_supported(mode, M, N, K))
+    return one_launch
+
+
 def bgemm_packed_weight_forward(w, x, mode=MODE_XOR, out_dtype=torch.int32, scale=None, x_zero_point=None,
                                 variant=VARIANT_AUTO):
     """Prepacked weights ``w`` (M rows) x activations ``x`` as they are, fp16 or fp32 ``[N,K]`` -> ``[N,M]``.
@@ -368,10 +391,7 @@ def bgemm_packed_weight_forward(w, x, mode=MODE_XOR, out_dtype=torch.int32, scal
         x_zero_point = x_zero_point.detach().to(x.dtype)
     N, K, M = x.shape[0], w.K, w.rows
     L = _b.lib()
-    one_launch = _decode_shapes.get((mode, M, N, K))
-    if one_launch is None:
-        one_launch = _decode_shapes[(mode, M, N, K)] = bool(N and M and K and L.bgemm_packed_weight_forward_supported(mode, M, N, K))
-    if not one_launch or variant == VARIANT_VALU:
+    if not decode_shape_supported(mode, M, N, K) or variant == VARIANT_VALU:
         xp = pack_ternary(x) if ternary else pack_sign(x, zero_point=x_zero_point)
         return bgemm_packed_forward(w, xp, mode, out_dtype, 8, variant, scale=scale)[0]
     if x.stride(1) != 1 or x.stride(0) < K:

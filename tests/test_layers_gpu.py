@@ -155,6 +155,42 @@ def test_chain_keeps_only_bits_between_layers(dtype):
     assert chain(x).requires_grad                          # with gradients: the ordinary path
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.half])
+def test_decode_rows_take_one_launch_and_follow_parameter_updates(dtype):
+    """Inputs of one to four rows go through the kernel that packs its own activations; the cached parameter
+    views must follow in-place updates, replaced parameters and dtype changes."""
+    torch.manual_seed(21)
+    lin = bl.BGEMMLinear(1000, 300, bias=True).to(DEV).to(dtype)
+    big = torch.randn(64, 1000, device=DEV).to(dtype)
+    with torch.no_grad():
+        lin(big)                                             # initialises the scales
+        lin.fuse_inference = False
+        want = lin(big)
+        lin.fuse_inference = True
+        for n in (1, 2, 4, 5):
+            assert torch.equal(lin(big[:n]), want[:n]), n
+        assert torch.equal(lin(big[:3].reshape(3, 1, 1000)), want[:3].reshape(3, 1, 300))
+        lin.sw.mul_(2.0); lin.bias.add_(1.0)                 # in place
+        lin.fuse_inference = False
+        want = lin(big[:2])
+        lin.fuse_inference = True
+        assert torch.equal(lin(big[:2]), want)
+        lin.sa = torch.nn.Parameter(lin.sa.detach() * 3)     # replaced
+        lin.fuse_inference = False
+        want = lin(big[:2])
+        lin.fuse_inference = True
+        assert torch.equal(lin(big[:2]), want)
+    other = torch.half if dtype == torch.float32 else torch.float32
+    lin = lin.to(other)
+    lin.zpa = lin.zpa.to(other)
+    with torch.no_grad():
+        x = big[:1].to(other)
+        lin.fuse_inference = False
+        want = lin(x)
+        lin.fuse_inference = True
+        assert lin(x).dtype == other and torch.equal(lin(x), want)
+
+
 def test_elastic_module_matches_cpu_twin():
     torch.manual_seed(4)
     x = torch.randn(64, 256, device=DEV)
