@@ -146,21 +146,73 @@ static inline int effective_split(int64_t tiles, int splitK, int KT)
 // through fp32 because |v| < 2^24); or the binary Linear's scaling fused in, op for op as torch
 // evaluates `half(acc) * sw * sa (+ bias)` (tests/python/bgemm_linear.py:482-484): with fp32
 // parameters every step is an fp32 op, with fp16 parameters every step rounds to fp16.  No step
-// may be contracted into an FMA.
+// may be contracted into an FMA: the functions switch contraction off and use plain operators (the
+// __fmul_rn / __fadd_rn wrappers are ordinary inline functions compiled with contraction allowed, so
+// a multiply and an add that come out of them can still be fused after inlining).
 __device__ __forceinline__ float scaled_f32(const GemmArgs& a, const int64_t m, const int v)
 {
-    float r = __fmul_rn(__half2float(__float2half_rn((float)v)), reinterpret_cast<const float*>(a.ep_sw)[m]);
-    r = __fmul_rn(r, *reinterpret_cast<const float*>(a.ep_sa));
-    if (a.ep_bias) r = __fadd_rn(r, reinterpret_cast<const float*>(a.ep_bias)[m]);
+#pragma clang fp contract(off)      // every step rounds by itself, as torch's separate kernels do
+    float r = (__half2float(__float2half_rn((float)v)) * reinterpret_cast<const float*>(a.ep_sw)[m]);
+    r = (r * *reinterpret_cast<const float*>(a.ep_sa));
+    if (a.ep_bias) r = (r + reinterpret_cast<const float*>(a.ep_bias)[m]);
     return r;
 }
 __device__ __forceinline__ __half scaled_f16(const GemmArgs& a, const int64_t m, const int v)
 {
+#pragma clang fp contract(off)      // every step rounds by itself, as torch's separate kernels do
     __half r = __float2half_rn((float)v);
-    r = __float2half_rn(__fmul_rn(__half2float(r), __half2float(reinterpret_cast<const __half*>(a.ep_sw)[m])));
-    r = __float2half_rn(__fmul_rn(__half2float(r), __half2float(*reinterpret_cast<const __half*>(a.ep_sa))));
-    if (a.ep_bias) r = __float2half_rn(__fadd_rn(__half2float(r), __half2float(reinterpret_cast<const __half*>(a.ep_bias)[m])));
+    r = __float2half_rn((__half2float(r) * __half2float(reinterpret_cast<const __half*>(a.ep_sw)[m])));
+    r = __float2half_rn((__half2float(r) * __half2float(*reinterpret_cast<const __half*>(a.ep_sa))));
+    if (a.ep_bias) r = __float2half_rn((__half2float(r) + __half2float(reinterpret_cast<const __half*>(a.ep_bias)[m])));
     return r;
+}
+// The same with the column's parameters already in registers (a store loop walks rows of fixed columns:
+// the parameters are fetched once per column, not once per element).  fp16 parameters widened to fp32
+// are the values the functions above compute with, so the results are identical.
+struct ColParams { float sw, bias; };
+__device__ __forceinline__ bool f32_params(const int kind) { return kind == BGEMM_OUT_F32_SCALED || kind == BGEMM_OUT_BITS_F32; }
+__device__ __forceinline__ float ep_scalar(const int kind, const void* p)
+{
+    return f32_params(kind) ? *reinterpret_cast<const float*>(p) : __half2float(*reinterpret_cast<const __half*>(p));
+}
+__device__ __forceinline__ ColParams col_params(const GemmArgs& a, const int64_t m)
+{
+    ColParams c = {0.f, 0.f};
+    if (m < a.M && a.ep_sw) {
+        if (f32_params(a.out_kind)) {
+            c.sw = reinterpret_cast<const float*>(a.ep_sw)[m];
+            if (a.ep_bias) c.bias = reinterpret_cast<const float*>(a.ep_bias)[m];
+        } else {
+            c.sw = __half2float(reinterpret_cast<const __half*>(a.ep_sw)[m]);
+            if (a.ep_bias) c.bias = __half2float(reinterpret_cast<const __half*>(a.ep_bias)[m]);
+        }
+    }
+    return c;
+}
+__device__ __forceinline__ float scaled_f32(const int v, const ColParams c, const float sa, const bool has_bias)
+{
+#pragma clang fp contract(off)      // every step rounds by itself, as torch's separate kernels do
+    float r = (__half2float(__float2half_rn((float)v)) * c.sw);
+    r = (r * sa);
+    if (has_bias) r = (r + c.bias);
+    return r;
+}
+__device__ __forceinline__ __half scaled_f16(const int v, const ColParams c, const float sa, const bool has_bias)
+{
+#pragma clang fp contract(off)      // every step rounds by itself, as torch's separate kernels do
+    __half r = __float2half_rn((float)v);
+    r = __float2half_rn((__half2float(r) * c.sw));
+    r = __float2half_rn((__half2float(r) * sa));
+    if (has_bias) r = __float2half_rn((__half2float(r) + c.bias));
+    return r;
+}
+// sign bit of half_rn(y - zp) for the bits kinds, y as above
+__device__ __forceinline__ unsigned next_sign_bit(const int kind, const int v, const ColParams c, const float sa,
+                                                  const bool has_bias, const float zp)
+{
+#pragma clang fp contract(off)      // every step rounds by itself, as torch's separate kernels do
+    const float y = kind == BGEMM_OUT_BITS_F32 ? scaled_f32(v, c, sa, has_bias) : __half2float(scaled_f16(v, c, sa, has_bias));
+    return __float_as_uint((y - zp)) >> 31;
 }
 __host__ __device__ __forceinline__ int out_elem_shift(const int kind) { return (kind == BGEMM_OUT_F16 || kind == BGEMM_OUT_F16_SCALED) ? 1 : 2; }
 
@@ -170,12 +222,12 @@ __host__ __device__ __forceinline__ int out_elem_shift(const int kind) { return 
 __device__ __forceinline__ bool bits_kind(const int kind) { return kind >= BGEMM_OUT_BITS_F32; }
 __device__ __forceinline__ unsigned next_sign_bit(const GemmArgs& a, const int64_t m, const int v)
 {
+#pragma clang fp contract(off)      // every step rounds by itself, as torch's separate kernels do
     float d;
     if (a.out_kind == BGEMM_OUT_BITS_F32)
-        d = __fsub_rn(scaled_f32(a, m, v), a.ep_zp ? *reinterpret_cast<const float*>(a.ep_zp) : 0.f);
+        d = scaled_f32(a, m, v) - (a.ep_zp ? *reinterpret_cast<const float*>(a.ep_zp) : 0.f);
     else
-        d = __fsub_rn(__half2float(scaled_f16(a, m, v)),
-                      a.ep_zp ? __half2float(*reinterpret_cast<const __half*>(a.ep_zp)) : 0.f);
+        d = __half2float(scaled_f16(a, m, v)) - (a.ep_zp ? __half2float(*reinterpret_cast<const __half*>(a.ep_zp)) : 0.f);
     return __float_as_uint(d) >> 31;
 }
 // One word of the tiled output: the 32 lanes of a half-wave hold the bits of columns m32 .. m32 + 31

@@ -342,11 +342,19 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
             char* dst = out_base + (nrow0 + row0) * row_bytes + (m << 1);
             const int64_t dstep = RSTEP * row_bytes;
             const bool scaled = a.out_kind == BGEMM_OUT_F16_SCALED;
+            ColParams cp[8];                     // this lane's eight columns, the same for every row of the strip
+            float saf = 0.f;
+            if (scaled) {
+                saf = ep_scalar(a.out_kind, a.ep_sa);
+#pragma unroll
+                for (int e = 0; e < 8; e++) cp[e] = col_params(a, m + e);
+            }
+            const bool has_bias = a.ep_bias != nullptr;
             auto put8 = [&](const int4 q0, const int4 q1, char* const to, const bool sc) {
                 const int q[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
                 union { __half h[8]; uint4 u; } pk;
 #pragma unroll
-                for (int e = 0; e < 8; e++) pk.h[e] = sc ? scaled_f16(a, m + e, q[e]) : __float2half_rn((float)q[e]);
+                for (int e = 0; e < 8; e++) pk.h[e] = sc ? scaled_f16(q[e], cp[e], saf, has_bias) : __float2half_rn((float)q[e]);
                 *reinterpret_cast<uint4*>(to) = pk.u;
             };
             if (m < a.M) {
@@ -373,6 +381,15 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
             const int* sp = st + row0 * ROW_I + c4 * 4;
             char* dst = out_base + (nrow0 + row0) * row_bytes + (m << esz_shift);
             const int64_t dstep = RSTEP * row_bytes;
+            const bool scaled = a.out_kind == BGEMM_OUT_F32_SCALED || a.out_kind == BGEMM_OUT_F16_SCALED;
+            const bool has_bias = a.ep_bias != nullptr;
+            ColParams cp[4];
+            float saf = 0.f;
+            if (scaled) {
+                saf = ep_scalar(a.out_kind, a.ep_sa);
+#pragma unroll
+                for (int e = 0; e < 4; e++) cp[e] = col_params(a, m + e);
+            }
             if (m < a.M) {
 #pragma unroll 2
                 for (int row = row0; row < 32 && nrow0 + row < a.N; row += RSTEP, sp += RSTEP * ROW_I, dst += dstep) {
@@ -388,26 +405,39 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
                         *reinterpret_cast<uint2*>(dst) = pk.u;
                         break;
                     case BGEMM_OUT_F32_SCALED:
-                        *reinterpret_cast<float4*>(dst) = make_float4(scaled_f32(a, m, q.x), scaled_f32(a, m + 1, q.y),
-                                                                      scaled_f32(a, m + 2, q.z), scaled_f32(a, m + 3, q.w));
+                        *reinterpret_cast<float4*>(dst) = make_float4(scaled_f32(q.x, cp[0], saf, has_bias), scaled_f32(q.y, cp[1], saf, has_bias),
+                                                                      scaled_f32(q.z, cp[2], saf, has_bias), scaled_f32(q.w, cp[3], saf, has_bias));
                         break;
                     default:
-                        pk.h[0] = scaled_f16(a, m, q.x); pk.h[1] = scaled_f16(a, m + 1, q.y);
-                        pk.h[2] = scaled_f16(a, m + 2, q.z); pk.h[3] = scaled_f16(a, m + 3, q.w);
+                        pk.h[0] = scaled_f16(q.x, cp[0], saf, has_bias); pk.h[1] = scaled_f16(q.y, cp[1], saf, has_bias);
+                        pk.h[2] = scaled_f16(q.z, cp[2], saf, has_bias); pk.h[3] = scaled_f16(q.w, cp[3], saf, has_bias);
                         *reinterpret_cast<uint2*>(dst) = pk.u;
                         break;
                     }
                 }
             }
         } else {
-            // ragged or unaligned rows: one element per lane and step
+            // ragged or unaligned rows, and the bits kinds: one element per lane and step.  A lane meets one
+            // column (two where the strip is 128 wide), whose parameters it fetches once.
+            constexpr int NC = WM == 4 ? 2 : 1;
+            const bool bits = bits_kind(a.out_kind);
+            const bool has_bias = a.ep_bias != nullptr;
+            ColParams cp[NC];
+            float saf = 0.f, zpf = 0.f;
+            if (bits) {
+                saf = ep_scalar(a.out_kind, a.ep_sa);
+                if (a.ep_zp) zpf = ep_scalar(a.out_kind, a.ep_zp);
+#pragma unroll
+                for (int k = 0; k < NC; k++) cp[k] = col_params(a, mcol0 + (lane + 64 * k) % (32 * WM));
+            }
 #pragma unroll 4
             for (int p = 0; p < 16 * WM; p++) {
                 const int idx = p * 64 + lane, row = idx / (32 * WM), c = idx % (32 * WM);
                 const int64_t n = nrow0 + row, m = mcol0 + c;
-                if (bits_kind(a.out_kind)) {        // half-waves hold 32 consecutive columns of one row
+                if (bits) {                         // half-waves hold 32 consecutive columns of one row
                     const bool real = n < a.N && m < a.M;
-                    store_bits_word(a, b, n, mcol0 + (c & ~31), real ? next_sign_bit(a, m, st[row * ROW_I + c]) : 0u);
+                    const unsigned bit = next_sign_bit(a.out_kind, st[row * ROW_I + c], cp[NC == 2 ? (p & 1) : 0], saf, has_bias, zpf);
+                    store_bits_word(a, b, n, mcol0 + (c & ~31), real ? bit : 0u);
                 } else if (n < a.N && m < a.M)
                     store_out(a, out_off + n * a.M, m, st[row * ROW_I + c]);
             }

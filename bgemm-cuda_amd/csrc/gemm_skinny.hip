@@ -398,14 +398,18 @@ __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_ker
     }
 }
 
-// Shapes the skinny kernels take: one activation tile row always; up to four when the general
-// kernel's 64 x 128 output tiles would number fewer than the compute units and K is long enough
-// for the split to pay for the meeting in LDS.
+// Shapes the skinny kernels take: one activation tile row always.  Two to four tile rows only where
+// splitting K inside the block buys more than the general kernel's 32 x 128 tiles do (timed over a
+// sweep of shapes): few of those tiles and at least 16 K-tiles for up to 64 rows, a handful of tiles,
+// or a long K (from 32 K-tiles) on less than one tile per compute unit.
 bool gemm_skinny_shape(int planes, int64_t batch, int64_t M, int64_t N, int64_t K)
 {
     if (planes == 2) return N <= 16;
     if (N <= 32) return true;
-    return N <= 128 && K >= 2048 && batch * cdiv(N, 64) * cdiv(M, 128) < 256;
+    const int64_t tiles = batch * cdiv(N, 32) * cdiv(M, 128), KT = k_tiles(K);
+    if (N <= 64 && KT >= 16 && tiles < 128) return true;
+    if (N <= 128 && KT >= 8 && tiles < 32) return true;          // a handful of tiles: nothing else to spread over the chip
+    return N <= 128 && KT >= 32 && tiles < 256;
 }
 
 template <typename Eng>
