@@ -430,16 +430,36 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
 #pragma unroll
                 for (int k = 0; k < NC; k++) cp[k] = col_params(a, mcol0 + (lane + 64 * k) % (32 * WM));
             }
+            if (bits) {
+                // half-waves hold 32 consecutive columns of one row: a ballot makes the output word.  The strip
+                // starts on a row tile of the output operand, so its words sit at fixed steps from one base.
+                uint32_t* const obase = reinterpret_cast<uint32_t*>(a.out) + (int64_t)b * a.strideC;
+                const int64_t okt = k_tiles(a.M);
+                int64_t wbase[NC];
+                bool col_ok[NC], word_ok[NC];
+#pragma unroll
+                for (int k = 0; k < NC; k++) {
+                    const int c = (lane + 64 * k) % (32 * WM);
+                    col_ok[k] = mcol0 + c < a.M;
+                    word_ok[k] = mcol0 + (c & ~31) < a.M;
+                    wbase[k] = tiled_word_offset(nrow0, (mcol0 + c) >> 5, okt);
+                }
 #pragma unroll 4
-            for (int p = 0; p < 16 * WM; p++) {
-                const int idx = p * 64 + lane, row = idx / (32 * WM), c = idx % (32 * WM);
-                const int64_t n = nrow0 + row, m = mcol0 + c;
-                if (bits) {                         // half-waves hold 32 consecutive columns of one row
-                    const bool real = n < a.N && m < a.M;
-                    const unsigned bit = next_sign_bit(a.out_kind, st[row * ROW_I + c], cp[NC == 2 ? (p & 1) : 0], saf, has_bias, zpf);
-                    store_bits_word(a, b, n, mcol0 + (c & ~31), real ? bit : 0u);
-                } else if (n < a.N && m < a.M)
-                    store_out(a, out_off + n * a.M, m, st[row * ROW_I + c]);
+                for (int p = 0; p < 16 * WM; p++) {
+                    const int idx = p * 64 + lane, row = idx / (32 * WM), c = idx % (32 * WM), k = NC == 2 ? (p & 1) : 0;
+                    const bool row_ok = nrow0 + row < a.N;
+                    const unsigned bit = next_sign_bit(a.out_kind, st[row * ROW_I + c], cp[k], saf, has_bias, zpf);
+                    const unsigned long long bal = __ballot(bit != 0 && row_ok && col_ok[k]);
+                    const unsigned w = __brev((unsigned)(lane < 32 ? bal : bal >> 32));
+                    if ((lane & 31) == 0 && row_ok && word_ok[k]) obase[wbase[k] + row * 4] = w;
+                }
+            } else {
+#pragma unroll 4
+                for (int p = 0; p < 16 * WM; p++) {
+                    const int idx = p * 64 + lane, row = idx / (32 * WM), c = idx % (32 * WM);
+                    const int64_t n = nrow0 + row, m = mcol0 + c;
+                    if (n < a.N && m < a.M) store_out(a, out_off + n * a.M, m, st[row * ROW_I + c]);
+                }
             }
         }
         wave_sync();                                 // the next strip overwrites the staging area
