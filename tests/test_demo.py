@@ -54,3 +54,29 @@ def test_kernel_and_torch_elastic_layers_train_alike():
     a = mlp_demo.run("bgemm_elastic", epochs=2, train_samples=4096, test_samples=512, device="cuda:0", log=lambda s: None)
     b = mlp_demo.run("nn_elastic", epochs=2, train_samples=4096, test_samples=512, device="cuda:0", log=lambda s: None)
     assert abs(a["history"][-1][0] - b["history"][-1][0]) < 0.05 and abs(a["accuracy"] - b["accuracy"]) < 0.05
+
+
+@pytest.mark.gpu
+def test_binary_self_attention_block_kernels_equal_dense_torch():
+    """The BERT self-attention block with both matmuls on the binary kernels gives, bit for bit, what dense torch
+    matmuls on the de-binarised tensors give; gradients reach every projection."""
+    import attention_demo
+    torch.manual_seed(12)
+    block = attention_demo.BinarySelfAttention(hidden_size=768, num_attention_heads=12).to("cuda:0")
+    x = torch.randn(2, 128, 768, device="cuda:0")
+    mask = torch.zeros(2, 1, 1, 128, device="cuda:0")
+    mask[1, :, :, 100:] = -10000.0                       # padded tail of the second sequence
+    with torch.no_grad():
+        block(x, mask)                                   # initialises the layers' scales
+        out_k, scores_k = block(x, mask)
+        block.kernels = False
+        out_t, scores_t = block(x, mask)
+        block.kernels = True
+    assert tuple(out_k.shape) == (2, 128, 768) and tuple(scores_k.shape) == (2, 12, 128, 128)
+    assert torch.equal(scores_k, scores_t) and torch.equal(out_k, out_t)
+    assert int((scores_k[0] * 8).round().abs().max()) <= 64      # scores are integers in [-64, 64] over sqrt(64)
+    out, _ = block(x, mask)
+    # a loss with gradients of order one: the Functions' backward runs in fp16, as the reference's does
+    (out.float() * torch.randn_like(out)).sum().backward()
+    for lin in (block.query, block.key, block.value, block.dense):
+        assert lin.weight.grad is not None and torch.isfinite(lin.weight.grad).all() and lin.weight.grad.abs().sum() > 0
