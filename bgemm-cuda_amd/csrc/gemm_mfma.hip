@@ -486,7 +486,7 @@ static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int spl
     if (planes == 1 && blocks(256, 256) >= 512 && KT >= 32) return {0, 256, 256};
     if (planes == 1 && blocks(256, 128) >= 256 && (KT >= 4 || blocks(128, 128) < 512)) return {4, 256, 128};
     if (blocks(128, 128) >= 512) return {1, 128, 128};
-    if (blocks(64, 128) >= 256) return {2, 64, 128};
+    if (blocks(64, 128) >= 512) return {2, 64, 128};      // below two blocks a unit, twice as many 32-row tiles are faster
     return {3, 32, 128};
 }
 
