@@ -13,7 +13,7 @@ OK, EINVAL, ENULL, EWORKSPACE, ELAUNCH, EALIGN = 0, -1, -2, -3, -4, -5
 MODE_AND, MODE_XOR, MODE_ATTN, MODE_BWTA, MODE_ATTN_X = 0, 1, 2, 3, 4
 OUT_I32, OUT_F16, OUT_F32_SCALED, OUT_F16_SCALED, OUT_BITS_F32, OUT_BITS_F16 = 0, 1, 2, 3, 4, 5
 SRC_F16, SRC_F32 = 0, 1
-ABI_VERSION = 5
+ABI_VERSION = 6
 VARIANT_AUTO, VARIANT_VALU, VARIANT_MFMA, VARIANT_MFMA_F4 = 0, 1, 2, 3
 
 _i64, _p, _int, _sz = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
@@ -38,6 +38,8 @@ SIGNATURES = {
     "bgemm_packed_forward_bits": (_int, [_int, _p, _p, _p, _p, _int, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
                                          _int, _int, _p, _sz, _p, _sz, _p, _p, _p, _p, _p]),
     "bgemm_pack_sign_f16_transposed": (_int, [_p, _i64, _i64, _i64, _i64, _i64, _p, _p]),
+    "bgemm_pack_batched": (_int, [_p, _int, _int, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _p, _p, _p]),
+    "bgemm_pack_transposed_batched": (_int, [_p, _int, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _p, _p]),
     "bgemm_packed_weight_forward_supported": (_int, [_int, _i64, _i64, _i64]),
     "bgemm_packed_weight_forward": (_int, [_int, _p, _p, _int, _i64, _p, _p, _int, _i64, _i64, _i64, _int, _p, _p, _p, _p, _p]),
     "bgemm_f16_workspace_bytes": (_sz, [_i64, _i64, _i64, _int]),

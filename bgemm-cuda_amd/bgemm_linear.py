@@ -40,14 +40,20 @@ def _linear_grads(grad_out, x_sign, w_sign):
     return grad_x, grad_w
 
 
+def _matrices(t):
+    """Up to two leading dimensions are handed to the pack as they are (strides and all); more are folded."""
+    return t if t.dim() <= 4 else t.reshape(-1, *t.shape[-2:])
+
+
 def _pack_right(mat):
     """The right-hand operand of ``a @ mat`` (``mat`` is [..., K, M]) as a packed operand of M rows.  A transposed
-    view of a row-major [..., M, K] tensor (``k.transpose(-1, -2)``) is packed from those rows; anything else is
-    packed as it lies by the transposing pack.  No copy either way (bgemm_linear.py:25, :60 copy)."""
+    view of row-major [..., M, K] matrices (``k.transpose(-1, -2)``) is packed from those rows; anything else is
+    packed as it lies by the transposing pack.  No copy either way (bgemm_linear.py:25, :60 copy), also for
+    the strided [B, H, S, d] views of attention."""
     rows = mat.transpose(-1, -2)
-    if rows.is_contiguous():
-        return lowbit_kernel.pack_sign(rows.reshape(-1, *rows.shape[-2:]))
-    return lowbit_kernel.pack_sign_transposed(mat.reshape(-1, *mat.shape[-2:]))
+    if rows.stride(-1) == 1 and rows.stride(-2) >= rows.shape[-1]:
+        return lowbit_kernel.pack_sign(_matrices(rows))
+    return lowbit_kernel.pack_sign_transposed(_matrices(mat))
 
 
 def _batched_packed(x_rows, right, mode):
@@ -56,7 +62,7 @@ def _batched_packed(x_rows, right, mode):
     lead = x_rows.shape[:-2]
     if right.shape[:-2] != lead:
         raise ValueError("leading dimensions differ: %s vs %s" % (tuple(x_rows.shape), tuple(right.shape)))
-    xp = lowbit_kernel.pack_sign(x_rows.reshape(-1, *x_rows.shape[-2:]))
+    xp = lowbit_kernel.pack_sign(_matrices(x_rows))
     out = lowbit_kernel.bgemm_packed_forward(_pack_right(right), xp, mode, torch.half)
     return out.reshape(*lead, x_rows.shape[-2], right.shape[-1])
 
@@ -67,8 +73,10 @@ class bgemm_matmul(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, matA, matB, instruction='xor'):
-        matA, matB = matA.to(torch.half), matB.to(torch.half)
-        ctx.save_for_backward(matA, matB)
+        if ctx.needs_input_grad[0] or ctx.needs_input_grad[1]:
+            matA, matB = matA.to(torch.half), matB.to(torch.half)
+            ctx.save_for_backward(matA, matB)
+        # otherwise the pack reads fp32 operands itself: rounding to fp16 keeps the sign bit
         mode = lowbit_kernel.MODE_AND if instruction == 'and' else lowbit_kernel.MODE_XOR
         if matB.dim() > 2:
             return _batched_packed(matA, matB, mode)
@@ -93,8 +101,9 @@ class bgemm_attn_matmul(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, input1, input2, instruction="attn_mm"):
-        input1, input2 = input1.to(torch.half), input2.to(torch.half)
-        ctx.save_for_backward(input1, input2)
+        if ctx.needs_input_grad[0] or ctx.needs_input_grad[1]:
+            input1, input2 = input1.to(torch.half), input2.to(torch.half)
+            ctx.save_for_backward(input1, input2)
         # attn stays as it lies (activation side, {0,1}), the value operand is packed as it lies by the
         # transposing pack, and the result comes out as [..., S_q, d] directly: none of the reference's
         # three transposes (bgemm_linear.py:58-61)

@@ -15,12 +15,25 @@ namespace bgemm {
 // nonzero plane.  mode bit1: write the logical layout instead of the tiled one.  mode bit2: the
 // source is fp32 (rounded to fp16 first, as the layers' `.to(torch.half)` does).
 // zp: device scalar of the source type subtracted before that rounding, or null.
+// A job may hold nmat = outer x inner matrices of `rows` rows each (tiled output only): matrix (o, i) starts
+// so * o + si * i elements into src and fills its own mtiles row tiles of the output, one matrix after the other.
 struct PackJob {
     const void* src; int64_t rows, K, ld;
     uint32_t* dst0; uint32_t* dst1; int mode;
     const void* zp;
     int64_t rows_out, nseg, KT, Kw, waves;
+    int64_t nmat, inner, so, si, mtiles;
 };
+
+// Element offset of output row `row` in the source, or -1 for a row of padding.
+__device__ __forceinline__ int64_t source_row(const PackJob& j, const int64_t row)
+{
+    if (j.nmat == 1) return row < j.rows ? row * j.ld : -1;
+    const int64_t mpad = j.mtiles * TILE_ROWS, b = row / mpad, rl = row - b * mpad;
+    if (rl >= j.rows) return -1;
+    const int64_t o = b / j.inner, i = b - o * j.inner;
+    return o * j.so + i * j.si + rl * j.ld;
+}
 
 // Logical output: one wave packs 512 consecutive K elements of one row (16 words).
 __device__ __forceinline__ void pack_wave(const PackJob& j, const int64_t gw, const int lane)
@@ -32,9 +45,10 @@ __device__ __forceinline__ void pack_wave(const PackJob& j, const int64_t gw, co
     uint16_t h[8];                        // fp16 bit patterns; elements past K stay +0.0
 #pragma unroll
     for (int e = 0; e < 8; e++) h[e] = 0;
-    if (row < j.rows && k0 < j.K) {
+    const int64_t soff = source_row(j, row);
+    if (soff >= 0 && k0 < j.K) {
         if (j.mode & 4) {
-            const float* p = reinterpret_cast<const float*>(j.src) + row * j.ld + k0;
+            const float* p = reinterpret_cast<const float*>(j.src) + soff + k0;
             const float z = j.zp ? *reinterpret_cast<const float*>(j.zp) : 0.f;
             if (k0 + 8 <= j.K && (((uintptr_t)p) & 15) == 0) {
                 const float4 u = *reinterpret_cast<const float4*>(p), v = *reinterpret_cast<const float4*>(p + 4);
@@ -46,7 +60,7 @@ __device__ __forceinline__ void pack_wave(const PackJob& j, const int64_t gw, co
                 for (int e = 0; e < 8; e++) if (k0 + e < j.K) h[e] = half_bits(j.zp ? __fsub_rn(p[e], z) : p[e]);
             }
         } else {
-            const uint16_t* p = reinterpret_cast<const uint16_t*>(j.src) + row * j.ld + k0;
+            const uint16_t* p = reinterpret_cast<const uint16_t*>(j.src) + soff + k0;
             if (k0 + 8 <= j.K && (((uintptr_t)p) & 15) == 0) {
                 const uint4 v = *reinterpret_cast<const uint4*>(p);
                 h[0] = v.x & 0xffff; h[1] = v.x >> 16; h[2] = v.y & 0xffff; h[3] = v.y >> 16;
@@ -93,7 +107,14 @@ __device__ __forceinline__ void pack_tile(const PackJob& j, const int64_t gw, co
     const int64_t rt = gw / j.KT, kt = gw - rt * j.KT;
     if (rt * TILE_ROWS >= j.rows_out) return;              // whole wave leaves together
     const int c = lane & 31, rsub = lane >> 5;
-    const int64_t row0 = rt * TILE_ROWS + rsub, k0 = kt * TILE_KBITS + 8 * c;
+    const int64_t k0 = kt * TILE_KBITS + 8 * c;
+    // where the tile's first row lies in the source, and how many source rows there are from it on
+    int64_t off0 = rt * TILE_ROWS * j.ld, rows_left = j.rows - rt * TILE_ROWS;
+    if (j.nmat > 1) {
+        const int64_t b = rt / j.mtiles, rtl = rt - b * j.mtiles, o = b / j.inner, i = b - o * j.inner;
+        off0 = o * j.so + i * j.si + rtl * TILE_ROWS * j.ld;
+        rows_left = j.rows - rtl * TILE_ROWS;
+    }
     const bool ternary = j.mode & 1, f32 = j.mode & 4;
     // byte of (row r, lane c) inside the tile: word c >> 2 of the row goes to slot h * 32 + r, position q;
     // the row's first element is the word's most significant bit, i.e. byte 3 of the little-endian word
@@ -113,7 +134,8 @@ __device__ __forceinline__ void pack_tile(const PackJob& j, const int64_t gw, co
     };
     // the whole tile lies inside the source and every row is 16-byte aligned: plain vector loads, all in flight
     const int64_t esz = f32 ? 4 : 2;
-    const bool rows_in = rt * TILE_ROWS + TILE_ROWS <= j.rows && ((((uintptr_t)j.src) | (uintptr_t)(j.ld * esz)) & 15) == 0;
+    const bool rows_in = rows_left >= TILE_ROWS &&
+                         ((((uintptr_t)j.src) | (uintptr_t)(j.ld * esz) | (uintptr_t)(j.so * esz) | (uintptr_t)(j.si * esz)) & 15) == 0;
     const bool interior = rows_in && kt * TILE_KBITS + TILE_KBITS <= j.K;
     if (!f32 && rows_in && (interior || (j.K & 7) == 0)) {
         // also the last K-tile of a K that is a multiple of eight (head size 64: the only tile).  The lanes are
@@ -124,7 +146,7 @@ __device__ __forceinline__ void pack_tile(const PackJob& j, const int64_t gw, co
             constexpr int CW = decltype(cw_tag)::value, RI = 64 / CW, STEPS = TILE_ROWS / RI;
             const int cc = lane & (CW - 1), rs = lane / CW;
             const int b0 = (((cc >> 4) * 32) * 4 + ((cc >> 2) & 3)) * 4 + (3 - (cc & 3));
-            const uint16_t* p = reinterpret_cast<const uint16_t*>(j.src) + (rt * TILE_ROWS + rs) * j.ld + kt * TILE_KBITS + 8 * cc;
+            const uint16_t* p = reinterpret_cast<const uint16_t*>(j.src) + off0 + rs * j.ld + kt * TILE_KBITS + 8 * cc;
             const bool live = 8 * cc < left;
             uint4 raw[STEPS];
 #pragma unroll
@@ -153,7 +175,7 @@ __device__ __forceinline__ void pack_tile(const PackJob& j, const int64_t gw, co
         else if (left <= 128) rows_by(std::integral_constant<int, 16>{});
         else rows_by(std::integral_constant<int, 32>{});
     } else if (interior) {
-        const float* p = reinterpret_cast<const float*>(j.src) + row0 * j.ld + k0;
+        const float* p = reinterpret_cast<const float*>(j.src) + off0 + rsub * j.ld + k0;
 #pragma unroll
         for (int g = 0; g < 2; g++) {
             float4 lo[8], hi[8];
@@ -175,19 +197,19 @@ __device__ __forceinline__ void pack_tile(const PackJob& j, const int64_t gw, co
     } else {
         // edge tiles and unaligned sources: element loads, rows and columns past the end read as +0.0
         for (int jj = 0; jj < 16; jj++) {
-            const int64_t row = row0 + 2 * jj;
+            const int row = 2 * jj + rsub;
             uint16_t h[8];
 #pragma unroll
             for (int e = 0; e < 8; e++) h[e] = 0;
             int valid = 0;
-            if (row < j.rows && k0 < j.K) {
+            if (row < rows_left && k0 < j.K) {
                 valid = (int)(j.K - k0 < 8 ? j.K - k0 : 8);
                 if (f32) {
-                    const float* q = reinterpret_cast<const float*>(j.src) + row * j.ld + k0;
+                    const float* q = reinterpret_cast<const float*>(j.src) + off0 + row * j.ld + k0;
 #pragma unroll
                     for (int e = 0; e < 8; e++) if (e < valid) h[e] = half_bits(j.zp ? __fsub_rn(q[e], zf) : q[e]);
                 } else {
-                    const uint16_t* q = reinterpret_cast<const uint16_t*>(j.src) + row * j.ld + k0;
+                    const uint16_t* q = reinterpret_cast<const uint16_t*>(j.src) + off0 + row * j.ld + k0;
 #pragma unroll
                     for (int e = 0; e < 8; e++) if (e < valid) h[e] = q[e];
                 }
@@ -231,23 +253,27 @@ __global__ __launch_bounds__(256) void relayout_kernel(
 }
 
 static int make_job(PackJob* j, const void* src, int64_t rows, int64_t K, int64_t ld, void* d0, void* d1, int mode,
-                    const void* zp, const char* who)
+                    const void* zp, const char* who, int64_t outer = 1, int64_t inner = 1, int64_t so = 0, int64_t si = 0)
 {
     if (rows < 0 || K < 0 || ld < K) return fail(BGEMM_EINVAL, "%s: bad shape rows=%lld K=%lld ld=%lld", who,
                                                  (long long)rows, (long long)K, (long long)ld);
+    if (outer < 0 || inner < 0 || so < 0 || si < 0 || ((mode & 2) && outer * inner != 1))
+        return fail(BGEMM_EINVAL, "%s: bad batch %lld x %lld, strides %lld, %lld", who, (long long)outer,
+                    (long long)inner, (long long)so, (long long)si);
     memset(j, 0, sizeof *j);
-    if (rows == 0 || K == 0) return BGEMM_OK;
+    if (rows == 0 || K == 0 || outer * inner == 0) return BGEMM_OK;
     if (!src || !d0 || ((mode & 1) && !d1)) return fail(BGEMM_ENULL, "%s: null pointer", who);
     if (((uintptr_t)d0 & 15) || ((uintptr_t)d1 & 15)) return fail(BGEMM_EALIGN, "%s: destination not 16-byte aligned", who);
     j->src = src; j->zp = zp; j->rows = rows; j->K = K; j->ld = ld;
     j->dst0 = (uint32_t*)d0; j->dst1 = (uint32_t*)d1; j->mode = mode;
     j->KT = k_tiles(K); j->Kw = cdiv(K, 32);
-    j->rows_out = (mode & 2) ? rows : row_tiles(rows) * TILE_ROWS;
+    j->nmat = outer * inner; j->inner = inner; j->so = so; j->si = si; j->mtiles = row_tiles(rows);
+    j->rows_out = (mode & 2) ? rows : j->nmat * j->mtiles * TILE_ROWS;
     j->nseg = cdiv(j->KT * TILE_KBITS, 512);
     // a wave per tile streams best, but an operand of a few hundred tiles would leave most SIMDs without one
     // (measured crossover: 500 to 700 tiles)
-    if (!(mode & 2) && row_tiles(rows) * j->KT < 640) j->mode |= 8;
-    j->waves = (j->mode & (2 | 8)) ? j->rows_out * j->nseg : row_tiles(rows) * j->KT;
+    if (!(mode & 2) && j->nmat * j->mtiles * j->KT < 640) j->mode |= 8;
+    j->waves = (j->mode & (2 | 8)) ? j->rows_out * j->nseg : j->nmat * j->mtiles * j->KT;
     return BGEMM_OK;
 }
 
@@ -261,11 +287,12 @@ static int launch_jobs(const PackJob& j0, const PackJob& j1, hipStream_t st, con
 }
 
 static int pack_common(const void* src, int64_t rows, int64_t K, int64_t ld, void* d0, void* d1,
-                       int mode, const void* zp, hipStream_t st, const char* who)
+                       int mode, const void* zp, hipStream_t st, const char* who,
+                       int64_t outer = 1, int64_t inner = 1, int64_t so = 0, int64_t si = 0)
 {
     PackJob j0, j1;
     memset(&j1, 0, sizeof j1);
-    const int rc = make_job(&j0, src, rows, K, ld, d0, d1, mode, zp, who);
+    const int rc = make_job(&j0, src, rows, K, ld, d0, d1, mode, zp, who, outer, inner, so, si);
     return rc ? rc : launch_jobs(j0, j1, st, who);
 }
 
@@ -316,6 +343,19 @@ extern "C" int bgemm_pack_sign_centered(const void* src, int src_dtype, int64_t 
                        (hipStream_t)stream, "bgemm_pack_sign_centered");
 }
 
+extern "C" int bgemm_pack_batched(const void* src, int src_dtype, int ternary, const void* zero_point,
+                                  int64_t batch_outer, int64_t batch_inner, int64_t rows, int64_t K, int64_t ld,
+                                  int64_t stride_outer, int64_t stride_inner, void* dst0_tiled, void* dst1_tiled,
+                                  void* stream)
+{
+    if (src_dtype != BGEMM_SRC_F16 && src_dtype != BGEMM_SRC_F32)
+        return fail(BGEMM_EINVAL, "bgemm_pack_batched: unknown source type %d", src_dtype);
+    if (ternary && zero_point) return fail(BGEMM_EINVAL, "bgemm_pack_batched: a zero point goes with the sign pack only");
+    return pack_common(src, rows, K, ld, dst0_tiled, ternary ? dst1_tiled : nullptr,
+                       (ternary ? 1 : 0) | (src_dtype == BGEMM_SRC_F32 ? 4 : 0), zero_point, (hipStream_t)stream,
+                       "bgemm_pack_batched", batch_outer, batch_inner, stride_outer, stride_inner);
+}
+
 // Transposed source ([K][rows] in memory): a wave builds one 32-row x 256-bit tile.  For each of its
 // four words, lane (h, k') reads the 32 consecutive fp16 of source row k = 256 kt + 128 h + 32 q + k'
 // (four 16-byte loads when the source allows, all sixteen in flight), gathers their sign bits into a
@@ -332,36 +372,46 @@ __device__ __forceinline__ unsigned transpose32(unsigned w, const int lane)
     return w;
 }
 
-__global__ __launch_bounds__(256) void pack_transposed_kernel(const uint16_t* __restrict__ src, const int64_t rows,
-                                                              const int64_t K, const int64_t ld, const int64_t bstride,
+template <bool F32>
+__global__ __launch_bounds__(256) void pack_transposed_kernel(const void* __restrict__ src_, const int64_t rows,
+                                                              const int64_t K, const int64_t ld, const int64_t inner,
+                                                              const int64_t so, const int64_t si,
                                                               uint4* __restrict__ dst, const int64_t tiles_per_matrix,
                                                               const int64_t KT, const int64_t total_tiles)
 {
+    typedef typename std::conditional<F32, uint32_t, uint16_t>::type E;
+    constexpr int EB = sizeof(E), NV = 32 * EB / 16;       // 16-byte loads per 32 elements
     const int lane = threadIdx.x & 63, h = lane >> 5, kk = lane & 31;
     const int64_t tile = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (tile >= total_tiles) return;             // whole wave leaves together
     const int64_t b = tile / tiles_per_matrix, t = tile - b * tiles_per_matrix, rt = t / KT, kt = t - rt * KT;
+    const int64_t o = b / inner, i = b - o * inner;
     const int64_t r0 = rt * 32, k0 = kt * TILE_KBITS + h * 128 + kk;
-    const uint16_t* p = src + b * bstride + k0 * ld + r0;
-    const bool vec = r0 + 32 <= rows && (((uintptr_t)src | (uintptr_t)(ld * 2) | (uintptr_t)(bstride * 2)) & 15) == 0;
+    const E* p = reinterpret_cast<const E*>(src_) + o * so + i * si + k0 * ld + r0;
+    const bool vec = r0 + 32 <= rows &&
+                     (((uintptr_t)src_ | (uintptr_t)(ld * EB) | (uintptr_t)(so * EB) | (uintptr_t)(si * EB)) & 15) == 0;
     unsigned w[4];
     if (vec) {
-        uint4 raw[4][4];
+        uint4 raw[4][NV];
 #pragma unroll
         for (int q = 0; q < 4; q++)
 #pragma unroll
-            for (int c = 0; c < 4; c++)
+            for (int c = 0; c < NV; c++)
                 raw[q][c] = k0 + q * 32 < K ? reinterpret_cast<const uint4*>(p + (int64_t)q * 32 * ld)[c] : make_uint4(0u, 0u, 0u, 0u);
 #pragma unroll
         for (int q = 0; q < 4; q++) {
             unsigned x = 0;
 #pragma unroll
-            for (int c = 0; c < 4; c++) {
+            for (int c = 0; c < NV; c++) {
                 const unsigned d[4] = {raw[q][c].x, raw[q][c].y, raw[q][c].z, raw[q][c].w};
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    const unsigned sb = d[e] & 0x80008000u;          // sign bits of two halves
-                    x |= (((sb >> 15) | (sb >> 30)) & 3u) << (8 * c + 2 * e);
+                    if (F32)
+                        x |= (d[e] >> 31) << (4 * c + e);
+                    else {
+                        const unsigned sb = d[e] & 0x80008000u;          // sign bits of two halves
+                        x |= (((sb >> 15) | (sb >> 30)) & 3u) << (8 * c + 2 * e);
+                    }
                 }
             }
             w[q] = x;
@@ -372,7 +422,7 @@ __global__ __launch_bounds__(256) void pack_transposed_kernel(const uint16_t* __
             unsigned x = 0;
             if (k0 + q * 32 < K)
                 for (int r = 0; r < 32; r++)
-                    if (r0 + r < rows) x |= (unsigned)(p[(int64_t)q * 32 * ld + r] >> 15) << r;
+                    if (r0 + r < rows) x |= (unsigned)(p[(int64_t)q * 32 * ld + r] >> (8 * EB - 1)) << r;
             w[q] = x;
         }
     }
@@ -382,22 +432,36 @@ __global__ __launch_bounds__(256) void pack_transposed_kernel(const uint16_t* __
     dst[tile * TILE_U4 + lane] = make_uint4(w[0], w[1], w[2], w[3]);
 }
 
+extern "C" int bgemm_pack_transposed_batched(const void* src, int src_dtype, int64_t batch_outer, int64_t batch_inner,
+                                             int64_t rows, int64_t K, int64_t ld, int64_t stride_outer,
+                                             int64_t stride_inner, void* dst_tiled, void* stream)
+{
+    const char* who = "bgemm_pack_transposed_batched";
+    if (src_dtype != BGEMM_SRC_F16 && src_dtype != BGEMM_SRC_F32) return fail(BGEMM_EINVAL, "%s: unknown source type %d", who, src_dtype);
+    if (batch_outer < 0 || batch_inner < 0 || rows < 0 || K < 0 || ld < rows || stride_outer < 0 || stride_inner < 0)
+        return fail(BGEMM_EINVAL, "%s: bad shape batch=%lld x %lld rows=%lld K=%lld ld=%lld", who, (long long)batch_outer,
+                    (long long)batch_inner, (long long)rows, (long long)K, (long long)ld);
+    const int64_t batch = batch_outer * batch_inner;
+    if (batch == 0 || rows == 0 || K == 0) return BGEMM_OK;
+    if (!src || !dst_tiled) return fail(BGEMM_ENULL, "%s: null pointer", who);
+    const bool f32 = src_dtype == BGEMM_SRC_F32;
+    if (((uintptr_t)src & (f32 ? 3 : 1)) || ((uintptr_t)dst_tiled & 15))
+        return fail(BGEMM_EALIGN, "%s: source must be aligned to its elements, destination to 16 bytes", who);
+    const int64_t KT = k_tiles(K), per = row_tiles(rows) * KT, total = batch * per, blocks = cdiv(total, 4);
+    if (blocks > 0x7fffffffLL) return fail(BGEMM_EINVAL, "%s: operand too large", who);
+    if (f32)
+        hipLaunchKernelGGL(pack_transposed_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, src, rows,
+                           K, ld, batch_inner, stride_outer, stride_inner, reinterpret_cast<uint4*>(dst_tiled), per, KT, total);
+    else
+        hipLaunchKernelGGL(pack_transposed_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, src, rows,
+                           K, ld, batch_inner, stride_outer, stride_inner, reinterpret_cast<uint4*>(dst_tiled), per, KT, total);
+    return check_launch(who);
+}
+
 extern "C" int bgemm_pack_sign_f16_transposed(const void* src, int64_t batch, int64_t rows, int64_t K, int64_t ld,
                                               int64_t src_batch_stride, void* dst_tiled, void* stream)
 {
-    if (batch < 0 || rows < 0 || K < 0 || ld < rows || src_batch_stride < 0)
-        return fail(BGEMM_EINVAL, "bgemm_pack_sign_f16_transposed: bad shape batch=%lld rows=%lld K=%lld ld=%lld",
-                    (long long)batch, (long long)rows, (long long)K, (long long)ld);
-    if (batch == 0 || rows == 0 || K == 0) return BGEMM_OK;
-    if (!src || !dst_tiled) return fail(BGEMM_ENULL, "bgemm_pack_sign_f16_transposed: null pointer");
-    if (((uintptr_t)src & 1) || ((uintptr_t)dst_tiled & 15))
-        return fail(BGEMM_EALIGN, "bgemm_pack_sign_f16_transposed: source must be 2-byte, destination 16-byte aligned");
-    const int64_t KT = k_tiles(K), per = row_tiles(rows) * KT, total = batch * per, blocks = cdiv(total, 4);
-    if (blocks > 0x7fffffffLL) return fail(BGEMM_EINVAL, "bgemm_pack_sign_f16_transposed: operand too large");
-    hipLaunchKernelGGL(pack_transposed_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
-                       reinterpret_cast<const uint16_t*>(src), rows, K, ld, src_batch_stride,
-                       reinterpret_cast<uint4*>(dst_tiled), per, KT, total);
-    return check_launch("bgemm_pack_sign_f16_transposed");
+    return bgemm_pack_transposed_batched(src, BGEMM_SRC_F16, 1, batch, rows, K, ld, 0, src_batch_stride, dst_tiled, stream);
 }
 
 static int relayout(const void* src, void* dst, int64_t rows, int64_t K, int dir, void* stream, const char* who)

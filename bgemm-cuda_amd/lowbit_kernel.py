@@ -117,74 +117,76 @@ def zeros_packed(rows, K, batch=1, device="cuda"):
     return PackedBits(torch.zeros((batch, words), dtype=torch.int32, device=device), None, batch, rows, K)
 
 
+def _batch_layout(x):
+    """(outer, inner, stride_outer, stride_inner) of the leading dimensions of a 2-D to 4-D tensor."""
+    if x.dim() == 2:
+        return 1, 1, 0, 0
+    if x.dim() == 3:
+        return 1, x.shape[0], 0, x.stride(0)
+    return x.shape[0], x.shape[1], x.stride(0), x.stride(1)
+
+
+def _pack_source(x, what):
+    """fp16 and fp32 tensors are read where they lie if their last dimension is dense and rows do not overlap;
+    anything else is brought to contiguous fp16 first."""
+    _need_cuda(x, what)
+    if x.dim() not in (2, 3, 4):
+        raise ValueError("expected a 2-D, 3-D or 4-D tensor, got %d-D" % x.dim())
+    if x.dtype not in (torch.half, torch.float32):
+        x = x.to(torch.half)
+    if x.numel() and (x.stride(-1) != 1 or x.stride(-2) < x.shape[-1]):
+        x = x.contiguous()
+    return x
+
+
 def _pack(x, ternary, zero_point=None):
-    _need_cuda(x, "input")
-    if x.dim() not in (2, 3):
-        raise ValueError("expected a 2-D or 3-D tensor, got %d-D" % x.dim())
+    if zero_point is not None and isinstance(x, torch.Tensor) and x.dtype not in (torch.half, torch.float32):
+        raise TypeError("centred packing reads fp16 or fp32 sources, got %s" % x.dtype)
+    x = _pack_source(x, "input")
     if zero_point is not None:
         if ternary:
             raise ValueError("a zero point is only taken by the sign pack")
-        if x.dtype not in (torch.half, torch.float32):
-            raise TypeError("centred packing reads fp16 or fp32 sources, got %s" % x.dtype)
         if not isinstance(zero_point, torch.Tensor) or zero_point.numel() != 1:
             raise TypeError("zero_point must be a one-element tensor")
         _need_cuda(zero_point, "zero_point")
         zero_point = zero_point.detach().to(x.dtype)
-        x = x.contiguous()
-    else:
-        x = x.to(torch.half).contiguous()
-    batch = 1 if x.dim() == 2 else x.shape[0]
+    outer, inner, so, si = _batch_layout(x)
+    batch = outer * inner
     rows, K = x.shape[-2], x.shape[-1]
     L = _b.lib()
-    words = L.bgemm_tiled_words(rows, K)
-    d0 = torch.empty((batch, words), dtype=torch.int32, device=x.device)
+    d0 = torch.empty((batch, L.bgemm_tiled_words(rows, K)), dtype=torch.int32, device=x.device)
     d1 = torch.empty_like(d0) if ternary else None
     with _on(x.device):
-        st = _stream()
-        if batch > 1 and rows % 32 == 0:
-            # whole tiles per matrix: the batch is one tall matrix in the tiled layout
-            groups = [(x.data_ptr(), batch * rows, d0.data_ptr(), d1.data_ptr() if ternary else None)]
-        else:
-            groups = [(x[i].data_ptr() if x.dim() == 3 else x.data_ptr(), rows, d0[i].data_ptr(),
-                       d1[i].data_ptr() if ternary else None) for i in range(batch)]
-        for src, r, p0, p1 in groups:
-            if ternary:
-                _b.check(L.bgemm_pack_ternary_f16(src, r, K, K, p0, p1, st))
-            elif zero_point is not None:
-                _b.check(L.bgemm_pack_sign_centered(src, SRC_F32 if x.dtype == torch.float32 else SRC_F16, r, K, K,
-                                                    zero_point.data_ptr(), p0, st))
-            else:
-                _b.check(L.bgemm_pack_sign_f16(src, r, K, K, p0, st))
+        _b.check(L.bgemm_pack_batched(x.data_ptr(), SRC_F32 if x.dtype == torch.float32 else SRC_F16, int(ternary),
+                                      None if zero_point is None else zero_point.data_ptr(), outer, inner, rows, K,
+                                      x.stride(-2), so, si, d0.data_ptr(), d1.data_ptr() if ternary else None, _stream()))
     return PackedBits(d0, d1, batch, rows, K)
 
 
 def pack_sign(x, zero_point=None):
-    """fp16 (or castable) ``[R,K]`` / ``[B,R,K]`` -> tiled sign bits (bit = 1 for negative, -0.0 included).
+    """fp16 or fp32 (or castable) ``[R,K]`` / ``[B,R,K]`` / ``[B,H,R,K]`` -> tiled sign bits (bit = 1 for negative,
+    -0.0 included), one launch for the whole batch.  Strided views whose last dimension is dense are read
+    where they lie (``permute(0, 2, 1, 3)`` of a ``[B, S, H*d]`` projection, a slice of rows or columns).
 
     With ``zero_point`` (a one-element device tensor) the bits are those of
-    ``(x - zero_point).to(torch.half)`` for an fp16 or fp32 ``x``, computed in the same pass: the
-    operand the binary Linear layers feed the kernel (bgemm_linear.py:479-482)."""
+    ``(x - zero_point).to(torch.half)``, computed in the same pass: the operand the binary Linear layers
+    feed the kernel (bgemm_linear.py:479-482)."""
     return _pack(x, False, zero_point)
 
 
 def pack_sign_transposed(x):
-    """fp16 ``[K,R]`` / ``[B,K,R]`` -> tiled sign bits of the transposes (``R`` rows of ``K`` bits each), read as
-    they lie: what ``pack_sign(x.transpose(-1, -2).contiguous())`` gives, without the copy.  The right-hand
+    """``[K,R]`` / ``[B,K,R]`` / ``[B,H,K,R]`` -> tiled sign bits of the transposes (``R`` rows of ``K`` bits each),
+    read as they lie: what ``pack_sign(x.transpose(-1, -2).contiguous())`` gives, without the copy.  The right-hand
     operand of a matmul ``a @ b`` (``b`` is ``[K, M]``) and the value operand of attention are of this kind."""
-    _need_cuda(x, "input")
-    if x.dim() not in (2, 3):
-        raise ValueError("expected a 2-D or 3-D tensor, got %d-D" % x.dim())
-    x = x.to(torch.half)
-    if x.stride(-1) != 1 or x.stride(-2) < x.shape[-1] or (x.dim() == 3 and x.stride(0) < 0):
-        x = x.contiguous()
-    batch = 1 if x.dim() == 2 else x.shape[0]
+    x = _pack_source(x, "input")
+    outer, inner, so, si = _batch_layout(x)
     K, rows = x.shape[-2], x.shape[-1]
     L = _b.lib()
-    d0 = torch.empty((batch, L.bgemm_tiled_words(rows, K)), dtype=torch.int32, device=x.device)
+    d0 = torch.empty((outer * inner, L.bgemm_tiled_words(rows, K)), dtype=torch.int32, device=x.device)
     with _on(x.device):
-        _b.check(L.bgemm_pack_sign_f16_transposed(x.data_ptr(), batch, rows, K, x.stride(-2),
-                                                  x.stride(0) if x.dim() == 3 else 0, d0.data_ptr(), _stream()))
-    return PackedBits(d0, None, batch, rows, K)
+        _b.check(L.bgemm_pack_transposed_batched(x.data_ptr(), SRC_F32 if x.dtype == torch.float32 else SRC_F16,
+                                                 outer, inner, rows, K, x.stride(-2), so, si, d0.data_ptr(), _stream()))
+    return PackedBits(d0, None, outer * inner, rows, K)
 
 
 def pack_ternary(x):

@@ -104,6 +104,24 @@ int bgemm_pack_sign_centered(const void* src, int src_dtype, int64_t rows, int64
  * `.transpose(0, 1).contiguous()` before its kernel can read it, are packed as they lie. */
 int bgemm_pack_sign_f16_transposed(const void* src, int64_t batch, int64_t rows, int64_t K, int64_t ld,
                                    int64_t src_batch_stride, void* dst_tiled, void* stream);
+/* The pack entry points above over a batch of batch_outer x batch_inner matrices in one launch, each of
+ * `rows` x K elements with rows ld elements apart; matrix (o, i) starts stride_outer*o + stride_inner*i
+ * elements into src and its tiled operand is written bgemm_tiled_words(rows, K) words after the one before it
+ * (o-major).  This reads the [B, H, S, d] views attention works on where they lie, e.g. the
+ * `permute(0, 2, 1, 3)` view of a [B, S, H*d] projection (tests/python/bert/bert.py:216-220: strides S*H*d, d
+ * and row stride H*d), for which the reference's 2-D kernel call needs a `.contiguous()` copy per matrix
+ * (tests/python/bgemm_linear.py:25, :60).  src_dtype BGEMM_SRC_F16 or BGEMM_SRC_F32 (an fp32 source is rounded
+ * to fp16 first, as `.to(torch.half)` does; the sign bit is the same).  ternary != 0 writes the (nonzero,
+ * sign & nonzero) planes to dst0 / dst1, otherwise dst1 is ignored; zero_point as in bgemm_pack_sign_centered
+ * (sign pack only), or NULL. */
+int bgemm_pack_batched(const void* src, int src_dtype, int ternary, const void* zero_point,
+                       int64_t batch_outer, int64_t batch_inner, int64_t rows, int64_t K, int64_t ld,
+                       int64_t stride_outer, int64_t stride_inner, void* dst0_tiled, void* dst1_tiled, void* stream);
+/* bgemm_pack_sign_f16_transposed over an outer x inner batch, fp16 or fp32 source: element (k, r) of matrix
+ * (o, i) is at src[stride_outer*o + stride_inner*i + k*ld + r]. */
+int bgemm_pack_transposed_batched(const void* src, int src_dtype, int64_t batch_outer, int64_t batch_inner,
+                                  int64_t rows, int64_t K, int64_t ld, int64_t stride_outer, int64_t stride_inner,
+                                  void* dst_tiled, void* stream);
 /* logical <-> tiled re-layout of already packed bits (device buffers). */
 int bgemm_tile_from_logical(const uint32_t* logical, int64_t rows, int64_t K,
                             void* dst_tiled, void* stream);

@@ -29,7 +29,7 @@ def test_header_symbols_exported():
 
 def test_layout_sizes():
     L = _lib.lib()
-    assert L.bgemm_abi_version() == _lib.ABI_VERSION == 5
+    assert L.bgemm_abi_version() == _lib.ABI_VERSION == 6
     assert L.bgemm_tiled_words(1, 1) == 256
     assert L.bgemm_tiled_words(32, 256) == 256
     assert L.bgemm_tiled_words(33, 257) == 4 * 256
@@ -123,6 +123,18 @@ def test_pack_and_f16_reject():
     assert L.bgemm_pack_sign_f16(None, 4, 128, 128, 0x2000, None) == _lib.ENULL
     assert L.bgemm_pack_sign_f16(0x1000, 4, 128, 128, 0x2004, None) == _lib.EALIGN
     assert L.bgemm_pack_ternary_f16(0x1000, 4, 128, 128, 0x2000, None, None) == _lib.ENULL
+    # batched packs: (src, dtype, ternary, zp, outer, inner, rows, K, ld, stride_outer, stride_inner, dst0, dst1, stream)
+    assert L.bgemm_pack_batched(0x1000, 0, 0, None, 2, 3, 4, 128, 128, 0, 0, None, None, None) == _lib.ENULL
+    assert L.bgemm_pack_batched(0x1000, 7, 0, None, 2, 3, 4, 128, 128, 0, 0, 0x2000, None, None) == _lib.EINVAL  # dtype
+    assert L.bgemm_pack_batched(0x1000, 0, 0, None, 2, 3, 4, 128, 128, -8, 0, 0x2000, None, None) == _lib.EINVAL  # stride
+    assert L.bgemm_pack_batched(0x1000, 0, 0, None, -1, 3, 4, 128, 128, 0, 0, 0x2000, None, None) == _lib.EINVAL
+    assert L.bgemm_pack_batched(0x1000, 0, 1, 0x3000, 1, 1, 4, 128, 128, 0, 0, 0x2000, 0x4000, None) == _lib.EINVAL  # ternary + zero point
+    assert L.bgemm_pack_batched(0x1000, 0, 1, None, 1, 1, 4, 128, 128, 0, 0, 0x2000, None, None) == _lib.ENULL     # second plane
+    assert L.bgemm_pack_batched(None, 0, 0, None, 0, 3, 4, 128, 128, 0, 0, None, None, None) == 0                  # empty batch
+    assert L.bgemm_pack_transposed_batched(0x1000, 0, 2, 3, 64, 128, 32, 0, 0, 0x2000, None) == _lib.EINVAL       # ld < rows
+    assert L.bgemm_pack_transposed_batched(0x1000, 2, 2, 3, 64, 128, 64, 0, 0, 0x2000, None) == _lib.EINVAL       # dtype
+    assert L.bgemm_pack_transposed_batched(0x1002, 1, 2, 3, 64, 128, 64, 0, 0, 0x2000, None) == _lib.EALIGN       # fp32 source
+    assert L.bgemm_pack_transposed_batched(None, 0, 2, 3, 64, 128, 64, 0, 0, 0x2000, None) == _lib.ENULL
     assert L.bgemm_f16_forward(0x1000, 0x2000, 0x3000, 32, 32, 128, None, 0, 1, 3, None) == _lib.EINVAL  # INSTR 3
     assert L.bgemm_f16_forward(0x1000, 0x2000, 0x3000, 32, 32, 128, None, 0, 1, 1, None) == _lib.EWORKSPACE
     assert L.bgemm_f16_forward(0x1000, 0x2000, None, 32, 32, 128, 0x4000, 1 << 20, 1, 1, None) == _lib.ENULL

@@ -66,6 +66,31 @@ def test_batched_attention_pair_bert_shape():
     assert torch.allclose(qg.grad[0, 0].float(), g @ k[0, 0].half().sign().float(), atol=0)   # backward uses torch.sign
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.half])
+def test_attention_pair_reads_head_split_views_where_they_lie(dtype):
+    """The [B, H, S, d] operands of BERT are `permute(0, 2, 1, 3)` views of [B, S, H*d] projections
+    (bert.py:216-234).  The pair takes the views as they are, fp32 or fp16, with or without gradients, and gives what
+    it gives for contiguous fp16 copies; ragged S and d included."""
+    torch.manual_seed(9)
+    for (B, H, S, D) in ((2, 12, 128, 64), (2, 3, 50, 40)):
+        split = lambda t: t.view(B, S, H, D).permute(0, 2, 1, 3)
+        q, k, v = (split(torch.randn(B, S, H * D, device=DEV, dtype=dtype)) for _ in range(3))
+        attn = torch.randn(B, H, S, S, device=DEV, dtype=dtype)
+        dense = lambda t: t.to(torch.half).contiguous()
+        with torch.no_grad():
+            scores = bl.bgemm_matmul.apply(q, k.transpose(-1, -2))
+            ctx = bl.bgemm_attn_matmul.apply(attn, v)
+            assert torch.equal(scores, bl.bgemm_matmul.apply(dense(q), dense(k).transpose(-1, -2)))
+            assert torch.equal(ctx, bl.bgemm_attn_matmul.apply(dense(attn), dense(v)))
+        pm = lambda t: torch.where(torch.signbit(t.half()), -1.0, 1.0)
+        assert torch.equal(scores.float(), torch.matmul(pm(q), pm(k).transpose(-1, -2)).half().float())
+        assert torch.equal(ctx.float(), torch.matmul((~torch.signbit(attn.half())).float(), pm(v)).half().float())
+        # with gradients the operands are saved as fp16 and the outputs are the same
+        qg, vg = q.detach().clone().requires_grad_(True), v.detach().clone().requires_grad_(True)
+        assert torch.equal(bl.bgemm_matmul.apply(qg, k.transpose(-1, -2)), scores)
+        assert torch.equal(bl.bgemm_attn_matmul.apply(attn, vg), ctx)
+
+
 def test_bgemm_linear_backward_shapes_and_values():
     torch.manual_seed(2)
     x = torch.randn(32, 128, device=DEV, requires_grad=True)

@@ -126,6 +126,50 @@ def test_pack_transposed_equals_pack_of_the_transpose(B, K, R, pad):
     assert torch.equal(lk.pack_sign_transposed(want_src := x.transpose(1, 2).contiguous().transpose(1, 2)).data, want.data)
 
 
+@pytest.mark.parametrize("B,H,S,d", [(2, 3, 40, 64), (1, 2, 33, 72), (3, 1, 5, 300), (16, 12, 128, 64)])
+@pytest.mark.parametrize("dtype", [torch.half, torch.float32])
+def test_pack_batched_strided_views_match_oracle(oracle, B, H, S, d, dtype):
+    """[B, H, S, d] views of a [B, S, H*d] tensor (what attention's head split produces) are packed where they lie, one
+    launch: every matrix's tiled block equals the oracle's pack of that matrix; sign, ternary, centred, transposed;
+    ragged rows (each matrix padded to whole tiles on its own), few tiles and many."""
+    g = torch.Generator(device=DEV).manual_seed(B * 1000 + S)
+    flat = torch.randn((B, S, H * d), generator=g, device=DEV, dtype=dtype)
+    flat[:, ::3, ::5] = -0.0
+    flat[:, 1::4, 1::7] = 0.0
+    flat[:, 2::5, 3::11] = 1e-9 if dtype == torch.float32 else 6e-8      # fp32: rounds to +0.0 in fp16
+    view = flat.view(B, S, H, d).permute(0, 2, 1, 3)
+    assert not view.is_contiguous() or H == 1
+    host = view.to(torch.half).cpu().numpy()
+    got = lk.pack_sign(view)
+    assert (got.batch, got.rows, got.K) == (B * H, S, d)
+    tern = lk.pack_ternary(view)
+
+    def logical(data, b):
+        return lk.logical_from_tiled(lk.PackedBits(data[b:b + 1], None, 1, S, d)).cpu().numpy().view(np.uint32)
+
+    for b in range(0, B * H, 1 if B * H <= 6 else 37):
+        m = host[b // H, b % H]
+        assert (logical(got.data, b) == oracle.c_pack_sign(m)).all(), b
+        nz, sg = oracle.c_pack_ternary(m)
+        assert (logical(tern.data, b) == nz).all() and (logical(tern.data2, b) == sg).all(), b
+    # the same bits as the pack of a contiguous fp16 copy, padding words included
+    assert torch.equal(got.data, lk.pack_sign(view.to(torch.half).contiguous()).data)
+    assert torch.equal(tern.data, lk.pack_ternary(view.to(torch.half).contiguous()).data)
+    assert torch.equal(tern.data2, lk.pack_ternary(view.to(torch.half).contiguous()).data2)
+    # centred
+    zp = flat.float().mean().to(dtype).reshape(1)
+    want_c = lk.pack_sign((view - zp).to(torch.half).contiguous())
+    assert torch.equal(lk.pack_sign(view, zero_point=zp).data, want_c.data)
+    # transposed: the view read as [.., K = S, rows = d]
+    got_t = lk.pack_sign_transposed(view)
+    assert (got_t.batch, got_t.rows, got_t.K) == (B * H, d, S)
+    assert torch.equal(got_t.data, lk.pack_sign(view.to(torch.half).transpose(-1, -2).contiguous()).data)
+    # 3-D slices with a batch stride and a row stride of their own
+    sl = flat[:, 1:, 8:8 + d]
+    assert torch.equal(lk.pack_sign(sl).data, lk.pack_sign(sl.to(torch.half).contiguous()).data)
+    assert torch.equal(lk.pack_sign_transposed(sl).data, lk.pack_sign(sl.to(torch.half).transpose(-1, -2).contiguous()).data)
+
+
 # ------------------------------------------------------------------ packed GEMM, small and ragged
 SMALL = [(1, 1, 1), (8, 5, 32), (33, 7, 40), (32, 32, 128), (10, 3, 784), (64, 1, 256), (65, 17, 300),
          (130, 70, 1000), (256, 256, 512), (40, 200, 2304),
