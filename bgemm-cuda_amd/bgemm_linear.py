@@ -171,8 +171,10 @@ def calculate_gradient_signed(qx, grad, grad_scale, is_act):
 
 
 def _elastic_prepare(input, weight, sa):
-    x = input - input.mean().item()
-    w = weight - weight.mean().item()
+    # the means stay on the device: subtracting the 0-dim tensor gives the values that subtracting its
+    # `.item()` gives (bgemm_linear.py:357-358) without the two host synchronisations
+    x = input - input.mean()
+    w = weight - weight.mean()
     return x / sa, w
 
 
@@ -358,15 +360,46 @@ class BGEMMLinear_bireal(BGEMMLinear):
 
 
 class BGEMMLinear_elastic_signed(_ScaledBinaryLinear):
-    """Learned-scale binary linear (bgemm_linear.py:538-564)."""
+    """Learned-scale binary linear (bgemm_linear.py:538-564).
+
+    When no gradient is being recorded the forward runs on packed operands: the kernel only sees the sign bits of
+    ``(x - mean(x)) / sa`` and ``w - mean(w)`` (bgemm_linear.py:357-373), and for a positive ``sa`` the division
+    does not change a sign, so the activations are centred and packed in one pass and the weight's bits are
+    packed once per weight version; the scaling stays in torch, in the reference's order ``out * sa * sw``."""
     _fn = bgemm_linear_elastic_signed
+    fuse_inference = True
 
     def __init__(self, in_channels, out_channels, bias=True):
         super().__init__(in_channels, out_channels, bias)
 
+    def _fusable(self, x):
+        if not (self.fuse_inference and self._fn is bgemm_linear_elastic_signed and not torch.is_grad_enabled()
+                and x.is_cuda and x.dtype in (torch.float32, torch.half) and self.weight.dtype in (torch.float32, torch.half)):
+            return False
+        key = (id(self.sa), self.sa._version, self.sa.data_ptr())
+        if self.__dict__.get("_sa_key") != key:          # one read-back per update of sa, none per forward
+            self._sa_positive, self._sa_key = bool((self.sa.detach() > 0).all()), key
+        return self._sa_positive
+
+    def _packed_weight(self):
+        w = self.weight
+        key = (w._version, w.data_ptr(), w.dtype)
+        if self.__dict__.get("_wp_key") != key:
+            self._wp = lowbit_kernel.pack_sign(w.detach(), zero_point=w.detach().mean().reshape(1))
+            self._wp_key = key
+        return self._wp
+
+    def _fused_forward(self, x):
+        x2 = x.reshape(-1, x.shape[-1])
+        xp = lowbit_kernel.pack_sign(x2, zero_point=x.mean().reshape(1))
+        out = lowbit_kernel.bgemm_packed_forward(self._packed_weight(), xp, lowbit_kernel.MODE_XOR, torch.half, splitK=8)[0]
+        return (out * self.sa * self.sw).reshape(*x.shape[:-1], self.weight.shape[0])
+
     def forward(self, x):
         if not self.initialized:
             self._initialize(x, self.weight)
+        if self._fusable(x):
+            return self._add_bias(self._fused_forward(x))
         return self._add_bias(self._fn.apply(x, self.weight, self.sa, self.sw, self.grad_scale))
 
 

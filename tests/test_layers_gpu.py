@@ -229,6 +229,42 @@ def test_elastic_module_matches_cpu_twin():
     assert a.weight.grad is not None and a.sa.grad is not None and a.sw.grad is not None
 
 
+@pytest.mark.filterwarnings("ignore:Synchronization debug mode")
+@pytest.mark.parametrize("dtype", [torch.float32, torch.half])
+def test_elastic_inference_runs_on_packed_operands_without_host_reads(dtype):
+    """Under no_grad the elastic layer centres and packs x in one pass and packs the weight once; the outputs are
+    those of the op-by-op forward, also for ragged shapes, after updates of the weight and the scales, and for a
+    negative sa (which the packed path leaves to the op-by-op one)."""
+    torch.manual_seed(6)
+    for (n, k, m) in ((64, 256, 128), (37, 300, 70), (1, 784, 10)):
+        lin = bl.BGEMMLinear_elastic_signed(k, m).to(DEV).to(dtype)
+        x = torch.randn(n, k, device=DEV, dtype=dtype) + 0.25
+        want = lin(x).detach()                               # records gradients: the op-by-op forward
+        with torch.no_grad():
+            got = lin(x)
+            assert got.dtype == want.dtype and torch.equal(got, want)
+            assert torch.equal(lin(x.reshape(1, n, k)), want.reshape(1, n, m))
+            # steady state: no host read-back in the forward
+            torch.cuda.set_sync_debug_mode("error")
+            try:
+                again = lin(x)
+            finally:
+                torch.cuda.set_sync_debug_mode("default")
+            assert torch.equal(again, want)
+            lin.weight.mul_(-0.5).add_(0.01)
+            lin.sw.mul_(1.5)
+            lin.sa.mul_(0.75)
+            lin.fuse_inference = False
+            want2 = lin(x)
+            lin.fuse_inference = True
+            assert not torch.equal(want2, want) and torch.equal(lin(x), want2)
+            lin.sa.neg_()
+            lin.fuse_inference = False
+            want3 = lin(x)
+            lin.fuse_inference = True
+            assert torch.equal(lin(x), want3)
+
+
 def test_config2_mlp_forward_bitwise(oracle):
     """Benchmark configuration 2: 784 -> 4096 -> 4096 -> 10, batch 128, fp16 outputs vs the CPU chain."""
     g = torch.Generator().manual_seed(1002)
