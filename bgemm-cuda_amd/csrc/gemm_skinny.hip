@@ -188,49 +188,38 @@ __global__ __launch_bounds__(256) void gemm_skinny_stream_kernel(const GemmArgs 
 }
 
 // ---- split-K kernel ----------------------------------------------------------------------------
-// NTL = activation tile rows handled by every wave (32 activation rows each).  More than one is
-// for shapes whose output has too few tiles to occupy the chip in the general kernel (a batch of
-// 128 rows against a few thousand weight rows): all KW * (weight row tiles) waves work, each on a
-// short K range, instead of a few waves walking all of K.
+// One block per (weight row tile, activation tile row): a 32 x 32 piece of the output, with K split over
+// the block's KW waves.  blockIdx.y walks the activation tile rows, so outputs of a few hundred such pieces
+// (a batch of 128 rows against a thousand weight rows, 512 x 512 with a long K) put KW waves on every piece,
+// each on a short K range with all of its loads in flight, instead of a few waves walking all of K.
 // FUSEX: the activations arrive unpacked (fp16 or fp32 rows, optionally minus a zero point): every wave
 // builds the activation tiles of its own K range itself, in LDS, while its weight loads are in flight,
-// which saves the separate pack launch of a decode step (a third of its time).  NTL == 1, batch == 1.
-template <typename Eng, int KW, int NTL, bool FUSEX = false>
+// which saves the separate pack launch of a decode step (a third of its time).  One tile row, batch == 1.
+template <typename Eng, int KW, bool FUSEX = false>
 __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_kernel(const GemmArgs a)
 {
     constexpr int NT = KW * 64;
-    constexpr int MAXT = (NTL == 1 && !FUSEX) ? 4 : 2;
-    static_assert(!FUSEX || NTL == 1, "in-kernel activation packing is built for one tile row");
-    __shared__ int sAcc[NTL][16][64];            // accumulator layout of the MFMA: [v][lane]
-    __shared__ int sPa[32], sPb[NTL][32];
+    constexpr int MAXT = FUSEX ? 2 : 4;
+    __shared__ int sAcc[16][64];                 // accumulator layout of the MFMA: [v][lane]
+    __shared__ int sPa[32], sPb[32];
     __shared__ __align__(16) unsigned char sX[FUSEX ? KW : 1][FUSEX ? MAXT : 1][FUSEX ? 1024 : 16];
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int h = lane >> 5;
     const int b = blockIdx.x / a.MT, rt = blockIdx.x % a.MT;
-    const bool two = a.mc.planes == 2;           // only with NTL == 1
+    const int nt = blockIdx.y, nbase = nt * 32;  // this block's activation tile row
+    const bool two = a.mc.planes == 2;           // only with one tile row
 
     int kt0, kt1;
     split_range(a.KT, KW, wave, &kt0, &kt1);
 
-    const uint4* xp[NTL];
-    if (FUSEX) xp[0] = nullptr;
-    else if (NTL == 1) xp[0] = skinny_x_ptr(a, b, lane);
-    else {
-#pragma unroll
-        for (int i = 0; i < NTL; i++)            // tile rows past the end re-read the last one (never stored)
-            xp[i] = a.X + (int64_t)b * a.strideX + (int64_t)min(i, a.NT - 1) * a.KT * TILE_U4 + lane;
-    }
+    const uint4* const xp = FUSEX ? nullptr : skinny_x_ptr(a, b, lane) + (int64_t)nt * a.KT * TILE_U4;
     const uint4* wp = a.W + (int64_t)b * a.strideW + (int64_t)rt * a.KT * TILE_U4 + lane;
 
-    typename Eng::Acc acc[NTL];
+    typename Eng::Acc acc;
 #pragma unroll
-    for (int i = 0; i < NTL; i++)
-#pragma unroll
-        for (int v = 0; v < 16; v++) acc[i][v] = 0;
-    int pa = 0, pb[NTL];
-#pragma unroll
-    for (int i = 0; i < NTL; i++) pb[i] = 0;
+    for (int v = 0; v < 16; v++) acc[v] = 0;
+    int pa = 0, pb = 0;
 
     // FUSEX: the activation tiles of this wave's K-tiles are built by the wave in its own LDS area: row n of
     // the source goes to operand row n (sign bits) or, with two planes, its nonzero bits to row n and
@@ -272,7 +261,7 @@ __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_ker
     // the wave's K range is short (K / KW) and requested MAXT K-tiles at a time: the kernel lives
     // on memory-level parallelism
     for (int kb = kt0; kb < kt1 || kb == kt0; kb += MAXT) {
-        uint4 xq[MAXT][NTL], wq[MAXT], xraw[FUSEX ? MAXT : 1][FUSEX ? 2 : 1];
+        uint4 xq[MAXT], wq[MAXT], xraw[FUSEX ? MAXT : 1][FUSEX ? 2 : 1];
         if (kb < kt1) {
             if (FUSEX && xfast) {
 #pragma unroll
@@ -289,10 +278,7 @@ __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_ker
 #pragma unroll
             for (int q = 0; q < MAXT; q++) {
                 const int64_t off = (int64_t)min(kb + q, kt1 - 1) * TILE_U4;
-                if (!FUSEX) {
-#pragma unroll
-                    for (int i = 0; i < NTL; i++) xq[q][i] = xp[i][off];
-                }
+                if (!FUSEX) xq[q] = xp[off];
                 wq[q] = load_stream(wp + off);
             }
             if (FUSEX) {
@@ -327,7 +313,7 @@ __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_ker
                 __builtin_amdgcn_wave_barrier();
                 __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-                for (int q = 0; q < MAXT; q++) xq[q][0] = reinterpret_cast<const uint4*>(sX[wave][min(q, kt1 - 1 - kb)])[lane];
+                for (int q = 0; q < MAXT; q++) xq[q] = reinterpret_cast<const uint4*>(sX[wave][min(q, kt1 - 1 - kb)])[lane];
                 __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");      // the next chunk overwrites the area
                 __builtin_amdgcn_wave_barrier();
             }
@@ -335,12 +321,8 @@ __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_ker
         if (kb == kt0) {
             // clear the meeting area while the first loads are in flight: every wave gets here at
             // once, so this barrier costs next to nothing
-            for (int i = threadIdx.x; i < NTL * 16 * 64; i += NT) (&sAcc[0][0][0])[i] = 0;
-            if (threadIdx.x < 32) {
-                sPa[threadIdx.x] = 0;
-#pragma unroll
-                for (int i = 0; i < NTL; i++) sPb[i][threadIdx.x] = 0;
-            }
+            for (int i = threadIdx.x; i < 16 * 64; i += NT) (&sAcc[0][0])[i] = 0;
+            if (threadIdx.x < 32) sPa[threadIdx.x] = sPb[threadIdx.x] = 0;
             __syncthreads();
         }
         if (kb < kt1) {
@@ -348,34 +330,25 @@ __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_ker
             for (int q = 0; q < MAXT; q++) {
                 if (kb + q >= kt1) break;
                 pa += popc4(wq[q]);
+                pb += popc4(xq[q]);
 #pragma unroll
-                for (int i = 0; i < NTL; i++) pb[i] += popc4(xq[q][i]);
-#pragma unroll
-                for (int s = 0; s < Eng::STEPS; s++) {
-                    const typename Eng::Frag bw = Eng::expand_w(wq[q], s);
-#pragma unroll
-                    for (int i = 0; i < NTL; i++) acc[i] = Eng::mma(Eng::expand_x(xq[q][i], s), bw, acc[i]);
-                }
+                for (int s = 0; s < Eng::STEPS; s++) acc = Eng::mma(Eng::expand_x(xq[q], s), Eng::expand_w(wq[q], s), acc);
             }
         }
     }
 
     // ---- meet in LDS: integer adds of the accumulator rows that carry outputs ------------------------
     pa += __shfl_xor(pa, 32);
-#pragma unroll
-    for (int i = 0; i < NTL; i++) pb[i] += __shfl_xor(pb[i], 32);
+    pb += __shfl_xor(pb, 32);
     if (kt0 < kt1) {
 #pragma unroll
-        for (int i = 0; i < NTL; i++)
-#pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const int n = 32 * i + 8 * (v >> 2) + 4 * h + (v & 3);
-                if ((two ? (n & 15) : n) < a.N) atomicAdd(&sAcc[i][v][lane], Eng::to_int(acc[i], v));
-            }
+        for (int v = 0; v < 16; v++) {
+            const int n = 8 * (v >> 2) + 4 * h + (v & 3);
+            if ((two ? (n & 15) : nbase + n) < a.N) atomicAdd(&sAcc[v][lane], Eng::to_int(acc, v));
+        }
         if (lane < 32) {
             atomicAdd(&sPa[lane], pa);
-#pragma unroll
-            for (int i = 0; i < NTL; i++) atomicAdd(&sPb[i][lane], pb[i]);
+            atomicAdd(&sPb[lane], pb);
         }
     }
     __syncthreads();
@@ -383,14 +356,14 @@ __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_ker
     // ---- rank-one terms and store: one output per thread and step, consecutive threads on one row ----
     const ModeCoef mc = a.mc;
     const int kbits = (int)a.K;
-    const int nout = (int)a.N * 32;
+    const int nout = min((int)a.N - nbase, 32) * 32;
     for (int o = threadIdx.x; o < nout; o += NT) {
-        const int n = o >> 5, c = o & 31, i = n >> 5, nl = n & 31;
+        const int nl = o >> 5, c = o & 31, n = nbase + nl;
         const int v = 4 * (nl >> 3) + (nl & 3), hh = (nl >> 2) & 1;   // accumulator slot of operand row nl
-        const int d = sAcc[i][v][hh * 32 + c];
-        const int d2 = two ? sAcc[0][v + 8][hh * 32 + c] : 0;
+        const int d = sAcc[v][hh * 32 + c];
+        const int d2 = two ? sAcc[v + 8][hh * 32 + c] : 0;
         const int64_t m = (int64_t)rt * 32 + c;
-        const int val = skinny_value(mc, two, kbits, sPa[c], sPb[i][nl], two ? sPb[0][nl + 16] : 0, d, d2);
+        const int val = skinny_value(mc, two, kbits, sPa[c], sPb[nl], two ? sPb[nl + 16] : 0, d, d2);
         if (bits_kind(a.out_kind))
             store_bits_word(a, b, n, (int64_t)rt * 32, m < a.M ? next_sign_bit(a, m, val) : 0u);
         else if (m < a.M)
@@ -398,18 +371,15 @@ __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_ker
     }
 }
 
-// Shapes the skinny kernels take: one activation tile row always.  Two to four tile rows only where
-// splitting K inside the block buys more than the general kernel's 32 x 128 tiles do (timed over a
-// sweep of shapes): few of those tiles and at least 16 K-tiles for up to 64 rows, a handful of tiles,
-// or a long K (from 32 K-tiles) on less than one tile per compute unit.
+// Shapes the skinny kernels take: one activation tile row always (two bit planes: up to 16 rows).  More
+// tile rows where splitting K inside the block buys more than the general kernel's 32 x 128 tiles do
+// (timed over a sweep of shapes): at least eight K-tiles and at most 512 pieces of 32 x 32 outputs, i.e.
+// about two blocks a compute unit; beyond that the general kernel's larger tiles re-read less.
 bool gemm_skinny_shape(int planes, int64_t batch, int64_t M, int64_t N, int64_t K)
 {
     if (planes == 2) return N <= 16;
     if (N <= 32) return true;
-    const int64_t tiles = batch * cdiv(N, 32) * cdiv(M, 128), KT = k_tiles(K);
-    if (N <= 64 && KT >= 16 && tiles < 128) return true;
-    if (N <= 128 && KT >= 8 && tiles < 32) return true;          // a handful of tiles: nothing else to spread over the chip
-    return N <= 128 && KT >= 32 && tiles < 256;
+    return k_tiles(K) >= 8 && batch * row_tiles(M) * row_tiles(N) <= 512;
 }
 
 template <typename Eng>
@@ -419,36 +389,29 @@ static int launch_splitk_fusex(const GemmArgs& a, hipStream_t st)
     int kw = 1;
     while (kw < 8 && (kw < a.splitK || blocks * kw < 4096) && kw * 2 <= a.KT) kw *= 2;
     const dim3 g((unsigned)blocks);
-    if (kw == 1) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 1, 1, true>), g, dim3(64), 0, st, a);
-    else if (kw == 2) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 2, 1, true>), g, dim3(128), 0, st, a);
-    else if (kw == 4) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 4, 1, true>), g, dim3(256), 0, st, a);
-    else hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 8, 1, true>), g, dim3(512), 0, st, a);
-    return check_launch("gemm_skinny");
-}
-
-template <typename Eng, int NTL>
-static int launch_splitk(const GemmArgs& a, hipStream_t st)
-{
-    const int64_t blocks = (int64_t)a.batch * a.MT;
-    if (blocks > 0x7fffffffLL) return fail(BGEMM_EINVAL, "gemm_skinny: grid of %lld blocks", (long long)blocks);
-    // K ways per block: at least what the caller asked for, more when the grid alone would leave the
-    // chip mostly idle (about four waves per SIMD wanted), never more than there are K-tiles
-    int kw = 1;
-    while (kw < 8 && (kw < a.splitK || blocks * kw < 4096) && kw * 2 <= a.KT) kw *= 2;
-    const dim3 g((unsigned)blocks);
-    if (kw == 1) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 1, NTL>), g, dim3(64), 0, st, a);
-    else if (kw == 2) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 2, NTL>), g, dim3(128), 0, st, a);
-    else if (kw == 4) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 4, NTL>), g, dim3(256), 0, st, a);
-    else hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 8, NTL>), g, dim3(512), 0, st, a);
+    if (kw == 1) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 1, true>), g, dim3(64), 0, st, a);
+    else if (kw == 2) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 2, true>), g, dim3(128), 0, st, a);
+    else if (kw == 4) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 4, true>), g, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 8, true>), g, dim3(512), 0, st, a);
     return check_launch("gemm_skinny");
 }
 
 template <typename Eng>
-static int launch_splitk_n(const GemmArgs& a, hipStream_t st)
+static int launch_splitk(const GemmArgs& a, hipStream_t st)
 {
-    if (a.NT <= 1) return launch_splitk<Eng, 1>(a, st);
-    if (a.NT == 2) return launch_splitk<Eng, 2>(a, st);
-    return launch_splitk<Eng, 4>(a, st);
+    const int64_t blocks = (int64_t)a.batch * a.MT;
+    if (blocks > 0x7fffffffLL || a.NT > 65535)
+        return fail(BGEMM_EINVAL, "gemm_skinny: grid of %lld x %lld blocks", (long long)blocks, (long long)a.NT);
+    // K ways per block: at least what the caller asked for, more when the grid alone would leave the
+    // chip mostly idle (about four waves per SIMD wanted), never more than there are K-tiles
+    int kw = 1;
+    while (kw < 8 && (kw < a.splitK || blocks * a.NT * kw < 4096) && kw * 2 <= a.KT) kw *= 2;
+    const dim3 g((unsigned)blocks, (unsigned)a.NT);
+    if (kw == 1) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 1>), g, dim3(64), 0, st, a);
+    else if (kw == 2) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 2>), g, dim3(128), 0, st, a);
+    else if (kw == 4) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 4>), g, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 8>), g, dim3(512), 0, st, a);
+    return check_launch("gemm_skinny");
 }
 
 template <typename Eng, int RT>
@@ -481,7 +444,7 @@ int launch_gemm_skinny(const GemmArgs& a, hipStream_t st, bool fp4)
         if (row_tiles >= 8192) return fp4 ? launch_stream<EngF4, 2>(a, st) : launch_stream<EngI8, 2>(a, st);
         if (row_tiles >= 4096) return fp4 ? launch_stream<EngF4, 1>(a, st) : launch_stream<EngI8, 1>(a, st);
     }
-    return fp4 ? launch_splitk_n<EngF4>(a, st) : launch_splitk_n<EngI8>(a, st);
+    return fp4 ? launch_splitk<EngF4>(a, st) : launch_splitk<EngI8>(a, st);
 }
 
 }  // namespace bgemm
