@@ -204,9 +204,9 @@ __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_ker
     __shared__ int sPa[32], sPb[32];
     __shared__ __align__(16) unsigned char sX[FUSEX ? KW : 1][FUSEX ? MAXT : 1][FUSEX ? 1024 : 16];
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: K ranges and their addresses stay scalar
     const int h = lane >> 5;
-    const int b = blockIdx.x / a.MT, rt = blockIdx.x % a.MT;
+    const int rt = blockIdx.x, b = blockIdx.z;   // weight row tile, matrix of the batch
     const int nt = blockIdx.y, nbase = nt * 32;  // this block's activation tile row
     const bool two = a.mc.planes == 2;           // only with one tile row
 
@@ -277,7 +277,8 @@ __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_ker
             }
 #pragma unroll
             for (int q = 0; q < MAXT; q++) {
-                const int64_t off = (int64_t)min(kb + q, kt1 - 1) * TILE_U4;
+                if (kb + q >= kt1) break;                       // wave-uniform: no load for a K-tile past the range
+                const int64_t off = (int64_t)(kb + q) * TILE_U4;
                 if (!FUSEX) xq[q] = xp[off];
                 wq[q] = load_stream(wp + off);
             }
@@ -341,10 +342,14 @@ __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_ker
     pa += __shfl_xor(pa, 32);
     pb += __shfl_xor(pb, 32);
     if (kt0 < kt1) {
+        // accumulator registers 4g .. 4g + 3 hold operand rows 8g .. 8g + 7: whole groups past the last real row
+        // are skipped (a branch the wave takes as one), rows past it inside a group are added and never read
+        const int nrows = (int)a.N - nbase;
 #pragma unroll
-        for (int v = 0; v < 16; v++) {
-            const int n = 8 * (v >> 2) + 4 * h + (v & 3);
-            if ((two ? (n & 15) : nbase + n) < a.N) atomicAdd(&sAcc[v][lane], Eng::to_int(acc, v));
+        for (int g = 0; g < 4; g++) {
+            if (8 * (two ? (g & 1) : g) >= nrows) continue;
+#pragma unroll
+            for (int v = 4 * g; v < 4 * g + 4; v++) atomicAdd(&sAcc[v][lane], Eng::to_int(acc, v));
         }
         if (lane < 32) {
             atomicAdd(&sPa[lane], pa);
@@ -357,17 +362,33 @@ __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_ker
     const ModeCoef mc = a.mc;
     const int kbits = (int)a.K;
     const int nout = min((int)a.N - nbase, 32) * 32;
-    for (int o = threadIdx.x; o < nout; o += NT) {
-        const int nl = o >> 5, c = o & 31, n = nbase + nl;
-        const int v = 4 * (nl >> 3) + (nl & 3), hh = (nl >> 2) & 1;   // accumulator slot of operand row nl
-        const int d = sAcc[v][hh * 32 + c];
-        const int d2 = two ? sAcc[v + 8][hh * 32 + c] : 0;
-        const int64_t m = (int64_t)rt * 32 + c;
-        const int val = skinny_value(mc, two, kbits, sPa[c], sPb[nl], two ? sPb[nl + 16] : 0, d, d2);
-        if (bits_kind(a.out_kind))
-            store_bits_word(a, b, n, (int64_t)rt * 32, m < a.M ? next_sign_bit(a, m, val) : 0u);
-        else if (m < a.M)
-            store_out(a, (int64_t)b * a.strideC + (int64_t)n * a.M, m, val);
+    // one copy of the loop per output kind: the kind's own addressing and parameters only
+    auto outputs = [&](auto store) {
+        for (int o = threadIdx.x; o < nout; o += NT) {
+            const int nl = o >> 5, c = o & 31;
+            const int v = 4 * (nl >> 3) + (nl & 3), hh = (nl >> 2) & 1;   // accumulator slot of operand row nl
+            const int d = sAcc[v][hh * 32 + c];
+            const int d2 = two ? sAcc[v + 8][hh * 32 + c] : 0;
+            store(nbase + nl, rt * 32 + c, skinny_value(mc, two, kbits, sPa[c], sPb[nl], two ? sPb[nl + 16] : 0, d, d2));
+        }
+    };
+    const int64_t out0 = (int64_t)b * a.strideC;
+    const int M = (int)a.M;
+    switch (a.out_kind) {
+    case BGEMM_OUT_I32:
+        outputs([&](const int n, const int m, const int val) { if (m < M) store_out_as<BGEMM_OUT_I32>(a, out0 + (int64_t)n * M, m, val); });
+        break;
+    case BGEMM_OUT_F16:
+        outputs([&](const int n, const int m, const int val) { if (m < M) store_out_as<BGEMM_OUT_F16>(a, out0 + (int64_t)n * M, m, val); });
+        break;
+    case BGEMM_OUT_F32_SCALED:
+        outputs([&](const int n, const int m, const int val) { if (m < M) store_out_as<BGEMM_OUT_F32_SCALED>(a, out0 + (int64_t)n * M, m, val); });
+        break;
+    case BGEMM_OUT_F16_SCALED:
+        outputs([&](const int n, const int m, const int val) { if (m < M) store_out_as<BGEMM_OUT_F16_SCALED>(a, out0 + (int64_t)n * M, m, val); });
+        break;
+    default:        // the bits kinds: every lane takes part in the ballot
+        outputs([&](const int n, const int m, const int val) { store_bits_word(a, b, n, (int64_t)rt * 32, m < M ? next_sign_bit(a, m, val) : 0u); });
     }
 }
 
@@ -400,13 +421,13 @@ template <typename Eng>
 static int launch_splitk(const GemmArgs& a, hipStream_t st)
 {
     const int64_t blocks = (int64_t)a.batch * a.MT;
-    if (blocks > 0x7fffffffLL || a.NT > 65535)
-        return fail(BGEMM_EINVAL, "gemm_skinny: grid of %lld x %lld blocks", (long long)blocks, (long long)a.NT);
+    if (a.MT > 0x7fffffffLL || a.NT > 65535 || a.batch > 65535)
+        return fail(BGEMM_EINVAL, "gemm_skinny: grid of %lld x %lld x %lld blocks", (long long)a.MT, (long long)a.NT, (long long)a.batch);
     // K ways per block: at least what the caller asked for, more when the grid alone would leave the
     // chip mostly idle (about four waves per SIMD wanted), never more than there are K-tiles
     int kw = 1;
     while (kw < 8 && (kw < a.splitK || blocks * a.NT * kw < 4096) && kw * 2 <= a.KT) kw *= 2;
-    const dim3 g((unsigned)blocks, (unsigned)a.NT);
+    const dim3 g((unsigned)a.MT, (unsigned)a.NT, (unsigned)a.batch);
     if (kw == 1) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 1>), g, dim3(64), 0, st, a);
     else if (kw == 2) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 2>), g, dim3(128), 0, st, a);
     else if (kw == 4) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 4>), g, dim3(256), 0, st, a);
