@@ -394,13 +394,16 @@ __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_ker
 
 // Shapes the skinny kernels take: one activation tile row always (two bit planes: up to 16 rows).  More
 // tile rows where splitting K inside the block buys more than the general kernel's 32 x 128 tiles do
-// (timed over a sweep of shapes): at least eight K-tiles and at most 512 pieces of 32 x 32 outputs, i.e.
-// about two blocks a compute unit; beyond that the general kernel's larger tiles re-read less.
+// (timed over a sweep of shapes, pieces = 32 x 32 outputs): up to 512 pieces from four K-tiles on, up to 1024
+// from eight, up to 1536 from 32 K-tiles; beyond that the general kernel's larger tiles re-read less.
 bool gemm_skinny_shape(int planes, int64_t batch, int64_t M, int64_t N, int64_t K)
 {
     if (planes == 2) return N <= 16;
     if (N <= 32) return true;
-    return k_tiles(K) >= 8 && batch * row_tiles(M) * row_tiles(N) <= 512;
+    const int64_t pieces = batch * row_tiles(M) * row_tiles(N), KT = k_tiles(K);
+    if (KT >= 32) return pieces <= 1536;
+    if (KT >= 8) return pieces <= 1024;
+    return KT >= 4 && pieces <= 512;
 }
 
 template <typename Eng>
