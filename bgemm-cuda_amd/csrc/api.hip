@@ -35,10 +35,10 @@ static int pick_variant(int mode, int64_t batch, int64_t M, int64_t N, int64_t K
 static void ws_needs(int variant, int planes, int64_t batch, int64_t M, int64_t N, int64_t K, int splitK,
                      size_t* part, size_t* counters)
 {
+    // Only the VALU family splits K across blocks.  The matrix-core family splits K among the waves of a block
+    // for outputs of few tiles (gemm_skinny_shape) and not at all for the rest, which fill the chip without.
     *part = *counters = 0;
-    if (variant != BGEMM_VARIANT_VALU && gemm_skinny_shape(planes, batch, M, N, K)) return;      // split inside the block
     if (variant == BGEMM_VARIANT_VALU) gemm_valu_ws(batch, M, N, K, splitK, planes, part, counters);
-    else gemm_mfma_ws(batch, M, N, K, splitK, planes, part, counters);
 }
 
 // one thread per counter
@@ -180,7 +180,7 @@ static int packed_forward(int mode, const void* W_tiled, const void* X_tiled, co
     const int v = variant == BGEMM_VARIANT_AUTO ? pick_variant(mode, batch, M, N, K) : variant;
     if (raw) return launch_gemm_skinny(a, (hipStream_t)stream, v == BGEMM_VARIANT_MFMA_F4);
     const bool skinny = v != BGEMM_VARIANT_VALU && gemm_skinny_shape(a.mc.planes, batch, M, N, K);
-    if (splitK > 1 && !skinny) {
+    if (splitK > 1 && v == BGEMM_VARIANT_VALU) {
         size_t part, cnt;
         ws_needs(v, a.mc.planes, batch, M, N, K, splitK, &part, &cnt);
         if (part) {       // this shape will really be split (splitK is an upper bound)

@@ -275,7 +275,6 @@ bool gemm_skinny_fusex_shape(int planes, int64_t M, int64_t N);
 int launch_gemm_skinny(const GemmArgs& a, hipStream_t st, bool fp4);
 // Split-K needs of each family for a shape: bytes of partial-tile scratch, number of counters.
 // (for the split that will actually be used: zero when the shape is not split at all)
-void gemm_mfma_ws(int64_t batch, int64_t M, int64_t N, int64_t K, int splitK, int planes, size_t* part_bytes, size_t* counters);
 void gemm_valu_ws(int64_t batch, int64_t M, int64_t N, int64_t K, int splitK, int planes, size_t* part_bytes, size_t* counters);
 
 }  // namespace bgemm

@@ -24,13 +24,10 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int wn = wave / WGM, wm = wave % WGM;
 
-    // logical block id: XCD-contiguous, split fastest (see xcd_contiguous_id / splitk_grid)
+    // logical block id: XCD-contiguous (see xcd_contiguous_id)
     const unsigned bid = xcd_contiguous_id(blockIdx.x, gridDim.x);
     const int per_gemm = tiles_n * tiles_m;
-    const int split = bid % a.splitK;
-    const unsigned rest = bid / a.splitK;
-    const int tile_id = rest % per_gemm, b = rest / per_gemm;
-    if (b >= a.batch) return;                    // padding blocks of a split-K grid
+    const int tile_id = bid % per_gemm, b = bid / per_gemm;
     // group tiles in bands of 8 along n so a band reuses its weight panels
     const int band = 8;
     const int band_id = tile_id / (band * tiles_m), in_band = tile_id % (band * tiles_m);
@@ -38,8 +35,9 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
     const int band_h = min(band, tiles_n - band_n0);
     const int tn = band_n0 + in_band % band_h, tm = in_band / band_h;
 
-    int kt0, kt1;
-    split_range(a.KT, a.splitK, split, &kt0, &kt1);
+    // K is never split across blocks here: outputs of so few tiles that a K split would pay go to the kernel
+    // that splits K among the waves of a block (gemm_skinny_shape)
+    const int kt0 = 0, kt1 = a.KT;
 
     const int nt0 = (tn * WGN + wn) * WN, mt0 = (tm * WGM + wm) * WM;
     const uint4* Wb = a.W + (int64_t)b * a.strideW;
@@ -191,11 +189,8 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
 
     }
 
-    // ---- epilogue: rank-one terms turn the AND-dot into this split's share of C ------------
-    const int64_t kbit0 = (int64_t)kt0 * TILE_KBITS;
-    int64_t kbit1 = (int64_t)kt1 * TILE_KBITS;
-    if (kbit1 > a.K) kbit1 = a.K;
-    const int bits = kbit1 > kbit0 ? (int)(kbit1 - kbit0) : 0;
+    // ---- epilogue: rank-one terms turn the AND-dot into C -----------------------------------------
+    const int bits = (int)a.K;
 #pragma unroll
     for (int j = 0; j < WM; j++) pa[j] += __shfl_xor(pa[j], 32);
 #pragma unroll
@@ -231,7 +226,7 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
         }
     }
     wave_sync();
-    // this split's share of C for tile row i (recomputed rather than kept: registers are tight)
+    // C for tile row i
     auto tile_row_vals = [&](const int i, int (&val)[WM][16]) {
         int4 r4[4];
 #pragma unroll
@@ -248,28 +243,6 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
             }
         }
     };
-
-    // ---- split-K: partial tiles go to the workspace in register order (lane-contiguous
-    // 16-byte stores); the last split to arrive on a tile adds the others to its own.
-    constexpr int TILE_I4 = WGN * WN * WGM * WM * 256;          // int4 per block tile
-    int4* tile_base = nullptr;
-    if (a.splitK > 1) {
-        tile_base = reinterpret_cast<int4*>(a.ws_part) + ((int64_t)b * per_gemm + tile_id) * a.splitK * TILE_I4;
-        int4* mine = tile_base + (int64_t)split * TILE_I4 + wave * (WN * WM * 256) + lane;
-#pragma unroll
-        for (int i = 0; i < WN; i++) {
-            int val[WM][16];
-            tile_row_vals(i, val);
-#pragma unroll
-            for (int j = 0; j < WM; j++)
-#pragma unroll
-                for (int g = 0; g < 4; g++)
-                    mine[((i * WM + j) * 4 + g) * 64] =
-                        make_int4(val[j][4 * g], val[j][4 * g + 1], val[j][4 * g + 2], val[j][4 * g + 3]);
-        }
-        __shared__ int s_last;
-        if (!splitk_arrive(a.ws_cnt + (int64_t)b * per_gemm + tile_id, (unsigned)a.splitK, &s_last)) return;
-    }
 
     // ---- store ------------------------------------------------------------------------------
     // Every 32-row strip of the wave's tile is transposed through the wave's own LDS area, so that
@@ -288,20 +261,6 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
     for (int i = 0; i < WN; i++) {
         int val[WM][16];
         tile_row_vals(i, val);
-        if (a.splitK > 1) {
-            for (int s = 0; s < a.splitK; s++) {
-                if (s == split) continue;
-                const int4* other = tile_base + (int64_t)s * TILE_I4;       // uniform: one split's tile
-#pragma unroll
-                for (int j = 0; j < WM; j++)
-#pragma unroll
-                    for (int g = 0; g < 4; g++) {
-                        const int4 o = load_partial(other, (unsigned)(wave * (WN * WM * 256) + lane + ((i * WM + j) * 4 + g) * 64) * 16u);
-                        val[j][4 * g] += o.x; val[j][4 * g + 1] += o.y;
-                        val[j][4 * g + 2] += o.z; val[j][4 * g + 3] += o.w;
-                    }
-            }
-        }
 #pragma unroll
         for (int v = 0; v < 16; v++)
 #pragma unroll
@@ -476,11 +435,8 @@ struct MfmaCfg { int id, bn, bm; };
 // per CU upwards, except on very short K (under 4 K-tiles), where 128 x 128 keeps more waves in
 // flight for what is then all prologue and epilogue; below that the smaller tiles, down to
 // 32 x 128, are chosen so that every CU gets a block.
-static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int splitK, int planes)
+static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int planes)
 {
-    // The tile is chosen for the output and the length of K, not for splitK: K ranges are only added (effective_split) where
-    // the tiles of the smallest efficient size still leave compute units idle.
-    (void)splitK;
     auto blocks = [&](int bn, int bm) { return batch * cdiv(N, bn) * cdiv(M, bm); };
     if (M <= 64) return blocks(128, 64) >= 512 ? MfmaCfg{7, 128, 64} : MfmaCfg{6, 64, 64};   // narrow outputs
     if (planes == 1 && blocks(256, 256) >= 512 && KT >= 32) return {0, 256, 256};
@@ -490,22 +446,12 @@ static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int spl
     return {3, 32, 128};
 }
 
-void gemm_mfma_ws(int64_t batch, int64_t M, int64_t N, int64_t K, int splitK, int planes, size_t* part_bytes,
-                  size_t* counters)
-{
-    const MfmaCfg c = pick_cfg(batch, M, N, k_tiles(K), splitK, planes);
-    const int64_t tiles = batch * cdiv(N, c.bn) * cdiv(M, c.bm);
-    const int s = effective_split(tiles, splitK, (int)k_tiles(K));       // as launch_eng will split
-    *part_bytes = s > 1 ? (size_t)tiles * s * c.bn * c.bm * 4 : 0;
-    *counters = s > 1 ? (size_t)tiles : 0;
-}
-
 template <typename Eng, int WGN, int WGM, int WN, int WM>
 static int launch_cfg(const GemmArgs& a, hipStream_t st)
 {
     constexpr int BN = WGN * WN * 32, BM = WGM * WM * 32;
     const int tiles_n = (int)cdiv(a.N, BN), tiles_m = (int)cdiv(a.M, BM);
-    const int64_t grid = splitk_grid((int64_t)a.batch * a.splitK * tiles_n * tiles_m, a.splitK);
+    const int64_t grid = (int64_t)a.batch * tiles_n * tiles_m;
     if (grid <= 0 || grid > 0x7fffffffLL) return fail(BGEMM_EINVAL, "gemm_mfma: grid of %lld blocks", (long long)grid);
     if (a.mc.planes == 2) {
         // two accumulator sets: only the tiles whose registers fit are built for two planes
@@ -521,11 +467,9 @@ static int launch_cfg(const GemmArgs& a, hipStream_t st)
 }
 
 template <typename Eng>
-static int launch_eng(const GemmArgs& a_in, hipStream_t st)
+static int launch_eng(const GemmArgs& a, hipStream_t st)
 {
-    GemmArgs a = a_in;
-    const MfmaCfg cfg = pick_cfg(a.batch, a.M, a.N, a.KT, a.splitK, a.mc.planes);   // as the workspace was sized
-    a.splitK = effective_split((int64_t)a.batch * cdiv(a.N, cfg.bn) * cdiv(a.M, cfg.bm), a.splitK, a.KT);
+    const MfmaCfg cfg = pick_cfg(a.batch, a.M, a.N, a.KT, a.mc.planes);
     switch (cfg.id) {
     case 0: return launch_cfg<Eng, 2, 2, 4, 4>(a, st);    // 256 x 256
     case 4: return launch_cfg<Eng, 2, 2, 4, 2>(a, st);    // 256 x 128, two blocks per CU

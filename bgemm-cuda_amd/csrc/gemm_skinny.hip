@@ -31,11 +31,12 @@ __device__ __forceinline__ uint4 load_stream(const uint4* p)
 // Pointer to this lane's slot of the activation operand's first K-tile.  With two planes, rows
 // 0..15 of the operand come from the nonzero plane and rows 16..31 from the sign&nonzero plane
 // (both hold at most 16 real rows), so one MFMA yields both dots.
-__device__ __forceinline__ const uint4* skinny_x_ptr(const GemmArgs& a, const int b, const int lane)
+// `half` picks rows 0..15 or 16..31 of the activation tile row for the two-plane operand.
+__device__ __forceinline__ const uint4* skinny_x_ptr(const GemmArgs& a, const int b, const int lane, const int half = 0)
 {
     const int h = lane >> 5, r = lane & 31;
-    const bool two = a.mc.planes == 2;
-    return (two && r >= 16 ? a.X2 + (h * 32 + r - 16) : a.X + lane) + (int64_t)b * a.strideX;
+    if (a.mc.planes != 2) return a.X + lane + (int64_t)b * a.strideX;
+    return (r >= 16 ? a.X2 : a.X) + (h * 32 + half * 16 + (r & 15)) + (int64_t)b * a.strideX;
 }
 
 // Output of one (activation row, weight row) pair from the AND-dots d (and d2 of the second plane).
@@ -205,15 +206,16 @@ __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_ker
     __shared__ __align__(16) unsigned char sX[FUSEX ? KW : 1][FUSEX ? MAXT : 1][FUSEX ? 1024 : 16];
 
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: K ranges and their addresses stay scalar
-    const int h = lane >> 5;
     const int rt = blockIdx.x, b = blockIdx.z;   // weight row tile, matrix of the batch
-    const int nt = blockIdx.y, nbase = nt * 32;  // this block's activation tile row
-    const bool two = a.mc.planes == 2;           // only with one tile row
+    // this block's activation rows: tile row blockIdx.y, or with two bit planes its half blockIdx.y & 1 (16 rows
+    // of both planes fill the 32 operand rows)
+    const bool two = a.mc.planes == 2;
+    const int nt = two ? blockIdx.y >> 1 : blockIdx.y, nbase = two ? blockIdx.y * 16 : blockIdx.y * 32;
 
     int kt0, kt1;
     split_range(a.KT, KW, wave, &kt0, &kt1);
 
-    const uint4* const xp = FUSEX ? nullptr : skinny_x_ptr(a, b, lane) + (int64_t)nt * a.KT * TILE_U4;
+    const uint4* const xp = FUSEX ? nullptr : skinny_x_ptr(a, b, lane, blockIdx.y & 1) + (int64_t)nt * a.KT * TILE_U4;
     const uint4* wp = a.W + (int64_t)b * a.strideW + (int64_t)rt * a.KT * TILE_U4 + lane;
 
     typename Eng::Acc acc;
@@ -361,7 +363,7 @@ __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_ker
     // ---- rank-one terms and store: one output per thread and step, consecutive threads on one row ----
     const ModeCoef mc = a.mc;
     const int kbits = (int)a.K;
-    const int nout = min((int)a.N - nbase, 32) * 32;
+    const int nout = min((int)a.N - nbase, two ? 16 : 32) * 32;
     // one copy of the loop per output kind: the kind's own addressing and parameters only
     auto outputs = [&](auto store) {
         for (int o = threadIdx.x; o < nout; o += NT) {
@@ -392,16 +394,19 @@ __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_ker
     }
 }
 
-// Shapes the skinny kernels take: one activation tile row always (two bit planes: up to 16 rows).  More
-// tile rows where splitting K inside the block buys more than the general kernel's 32 x 128 tiles do
-// (timed over a sweep of shapes, pieces = 32 x 32 outputs): up to 512 pieces from four K-tiles on, up to 1024
-// from eight, up to 1536 from 32 K-tiles; beyond that the general kernel's larger tiles re-read less.
+// Shapes the skinny kernels take: one group of activation rows always (32 rows, or 16 rows of two bit planes).
+// More groups where splitting K inside the block buys more than the general kernel's 32 x 128 tiles do (timed
+// over sweeps of shapes, pieces = 32 x 32 outputs resp. 16 x 32 of two planes): up to 512 pieces from four
+// K-tiles on, up to 1024 from eight, up to 2048 from sixteen.  The last bound is set by weights that come from
+// HBM rather than from a warm cache (a model's layers): there the general kernel's serial K loop pays the
+// full memory latency per step and loses by 15 to 50 %, while on cache-resident operands it would win the
+// range from 1024 to 2048 pieces by up to 7 %.  Beyond that the general kernel's larger tiles re-read less.
 bool gemm_skinny_shape(int planes, int64_t batch, int64_t M, int64_t N, int64_t K)
 {
-    if (planes == 2) return N <= 16;
-    if (N <= 32) return true;
-    const int64_t pieces = batch * row_tiles(M) * row_tiles(N), KT = k_tiles(K);
-    if (KT >= 32) return pieces <= 1536;
+    const int rows = planes == 2 ? 16 : 32;      // activation rows of one piece
+    if (N <= rows) return true;
+    const int64_t pieces = batch * row_tiles(M) * cdiv(N, rows), KT = k_tiles(K);
+    if (KT >= 16) return pieces <= 2048;
     if (KT >= 8) return pieces <= 1024;
     return KT >= 4 && pieces <= 512;
 }
@@ -424,13 +429,14 @@ template <typename Eng>
 static int launch_splitk(const GemmArgs& a, hipStream_t st)
 {
     const int64_t blocks = (int64_t)a.batch * a.MT;
-    if (a.MT > 0x7fffffffLL || a.NT > 65535 || a.batch > 65535)
-        return fail(BGEMM_EINVAL, "gemm_skinny: grid of %lld x %lld x %lld blocks", (long long)a.MT, (long long)a.NT, (long long)a.batch);
+    const int64_t groups = a.mc.planes == 2 ? cdiv(a.N, 16) : a.NT;      // activation rows a block takes: 16 of two planes, or 32
+    if (groups > 65535 || a.batch > 65535)
+        return fail(BGEMM_EINVAL, "gemm_skinny: grid of %lld x %lld x %lld blocks", (long long)a.MT, (long long)groups, (long long)a.batch);
     // K ways per block: at least what the caller asked for, more when the grid alone would leave the
     // chip mostly idle (about four waves per SIMD wanted), never more than there are K-tiles
     int kw = 1;
-    while (kw < 8 && (kw < a.splitK || blocks * a.NT * kw < 4096) && kw * 2 <= a.KT) kw *= 2;
-    const dim3 g((unsigned)a.MT, (unsigned)a.NT, (unsigned)a.batch);
+    while (kw < 8 && (kw < a.splitK || blocks * groups * kw < 4096) && kw * 2 <= a.KT) kw *= 2;
+    const dim3 g((unsigned)a.MT, (unsigned)groups, (unsigned)a.batch);
     if (kw == 1) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 1>), g, dim3(64), 0, st, a);
     else if (kw == 2) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 2>), g, dim3(128), 0, st, a);
     else if (kw == 4) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 4>), g, dim3(256), 0, st, a);
@@ -464,7 +470,7 @@ int launch_gemm_skinny(const GemmArgs& a, hipStream_t st, bool fp4)
     // Enough row tiles for about four waves on every SIMD: no K split needed (the result does not
     // depend on it).  Two row tiles per wave share one expansion of the activation tiles.
     const int64_t row_tiles = (int64_t)a.batch * a.MT;
-    if (a.NT <= 1) {
+    if (a.mc.planes == 2 ? a.N <= 16 : a.NT <= 1) {
         if (row_tiles >= 8192) return fp4 ? launch_stream<EngF4, 2>(a, st) : launch_stream<EngI8, 2>(a, st);
         if (row_tiles >= 4096) return fp4 ? launch_stream<EngF4, 1>(a, st) : launch_stream<EngI8, 1>(a, st);
     }

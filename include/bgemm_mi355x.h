@@ -138,10 +138,12 @@ int bgemm_logical_from_tiled(const void* tiled, int64_t rows, int64_t K,
  *   splitK   : >= 1, an upper bound on the number of contiguous K ranges (partitioned as in
  *              kernel_matmul.cuh:397-404) that are reduced inside the same launch with integer
  *              adds, so the result does not depend on it.  K is only split where the output
- *              tiles alone leave compute units idle and every range stays long enough to pay
- *              for the hand-over; few activation rows are split inside the block.
+ *              tiles alone leave compute units idle: the matrix-core kernels then split it
+ *              among the waves of a block (no workspace); the VALU family splits it across
+ *              blocks while every range stays long enough to pay for the hand-over.
  *   ws       : scratch for split-K partial tiles, bgemm_packed_workspace_bytes() bytes for the
- *              same arguments (0 when the shape will not be split), no initialisation needed
+ *              same arguments (0 when the shape will not be split across blocks: always for
+ *              BGEMM_VARIANT_AUTO and the matrix-core variants), no initialisation needed
  *              (NULL when that is 0).
  *   counters : split-K arrival counters, bgemm_packed_counter_bytes() bytes.  Must be
  *              zero-filled once before first use; every call leaves them zero again.

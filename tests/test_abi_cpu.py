@@ -35,22 +35,20 @@ def test_layout_sizes():
     assert L.bgemm_tiled_words(33, 257) == 4 * 256
     assert L.bgemm_tiled_words(11008, 4096) == 11008 * 4096 // 32
     assert L.bgemm_tiled_words(0, 128) == 0
-    # splitK is an upper bound: the needs are those of the split that will be used (K ranges of >= 24 K-tiles).
-    # One bit plane on few output tiles goes to the kernel that splits K inside a block (no workspace); two bit
-    # planes beyond 16 rows stay with the general kernel, which splits K across blocks
-    assert L.bgemm_packed_workspace_bytes(3, 1, 64, 256, 16384, 1, 0) == 0
-    assert L.bgemm_packed_workspace_bytes(3, 1, 64, 256, 16384, 4, 0) >= 2 * 64 * 256 * 4
-    assert L.bgemm_packed_counter_bytes(3, 1, 64, 256, 16384, 4, 0) >= 4
-    assert L.bgemm_packed_counter_bytes(3, 1, 64, 256, 16384, 1, 0) == 0
-    assert L.bgemm_packed_workspace_bytes(3, 1, 64, 256, 1024, 4, 0) == 0            # K too short to split
-    assert L.bgemm_packed_workspace_bytes(3, 1, 8192, 8192, 65536, 8, 0) == 0        # enough tiles without
-    assert L.bgemm_packed_workspace_bytes(1, 1, 64, 256, 16384, 4, 0) == 0
-    assert L.bgemm_packed_workspace_bytes(1, 1, 1030, 570, 16384, 4, 0) == 0
-    assert L.bgemm_packed_workspace_bytes(1, 1, 11008, 16, 4096, 8, 0) == 0
-    assert L.bgemm_packed_workspace_bytes(1, 1, 4096, 128, 4096, 8, 0) == 0
-    assert L.bgemm_packed_workspace_bytes(1, 1, 128, 128, 65536, 8, 1) > 0           # the VALU family still needs one
-    for variant in (1, 2, 3):           # every family states its needs for the same shape
-        assert L.bgemm_packed_workspace_bytes(3, 2, 100, 270, 40000, 3, variant) >= 2 * 3 * 100 * 270 * 4
+    # splitK is an upper bound, and only the VALU family (variant 1) splits K across blocks, through a workspace:
+    # the matrix-core family splits K among the waves of a block for outputs of few tiles and not at all otherwise
+    assert L.bgemm_packed_workspace_bytes(1, 1, 64, 256, 16384, 1, 1) == 0
+    assert L.bgemm_packed_workspace_bytes(1, 1, 64, 256, 16384, 4, 1) >= 2 * 64 * 256 * 4
+    assert L.bgemm_packed_counter_bytes(1, 1, 64, 256, 16384, 4, 1) >= 4
+    assert L.bgemm_packed_counter_bytes(1, 1, 64, 256, 16384, 1, 1) == 0
+    assert L.bgemm_packed_workspace_bytes(1, 1, 64, 256, 1024, 4, 1) == 0            # K too short to split
+    assert L.bgemm_packed_workspace_bytes(1, 1, 8192, 8192, 65536, 8, 1) == 0        # enough tiles without
+    assert L.bgemm_packed_workspace_bytes(3, 2, 100, 270, 40000, 3, 1) >= 2 * 3 * 100 * 270 * 4
+    for variant in (0, 2, 3):
+        for shape in ((1, 1, 64, 256, 16384), (3, 1, 64, 256, 16384), (1, 1, 11008, 16, 4096), (1, 1, 4096, 128, 4096),
+                      (1, 1, 128, 128, 65536), (3, 2, 100, 270, 40000), (1, 1, 8192, 8192, 65536)):
+            assert L.bgemm_packed_workspace_bytes(*shape, 8, variant) == 0
+            assert L.bgemm_packed_counter_bytes(*shape, 8, variant) == 0
     assert L.bgemm_f16_workspace_bytes(64, 32, 256, 1) >= (64 + 32) * 256 // 8
 
 
@@ -67,12 +65,12 @@ def test_layout_sizes():
     (dict(W=0x1008), _lib.EALIGN),
     (dict(out=0x3002), _lib.EALIGN),                  # int32 output on a 2-byte boundary
     (dict(out=0x3001, out_dtype=1), _lib.EALIGN),     # fp16 output on an odd address
-    # two bit planes on 64 x 256 outputs with a long K: the general kernel, which splits K across blocks
-    (dict(mode=3, X2=0x4000, splitK=2), _lib.EWORKSPACE),                # no workspace given
-    (dict(mode=3, X2=0x4000, splitK=2, ws=0x10000, ws_bytes=1 << 24), _lib.EWORKSPACE),            # no counters given
-    (dict(mode=3, X2=0x4000, splitK=2, ws=0x10000, ws_bytes=16, cnt=0x20000, cnt_bytes=4096), _lib.EWORKSPACE),
-    (dict(mode=3, X2=0x4000, splitK=2, ws=0x10000, ws_bytes=1 << 24, cnt=0x20000, cnt_bytes=0), _lib.EWORKSPACE),
-    (dict(mode=3, X2=0x4000, splitK=2, ws=0x10004, ws_bytes=1 << 24, cnt=0x20000, cnt_bytes=4096), _lib.EALIGN),
+    # the VALU family on 64 x 256 outputs with a long K splits K across blocks
+    (dict(variant=1, splitK=2), _lib.EWORKSPACE),                # no workspace given
+    (dict(variant=1, splitK=2, ws=0x10000, ws_bytes=1 << 24), _lib.EWORKSPACE),            # no counters given
+    (dict(variant=1, splitK=2, ws=0x10000, ws_bytes=16, cnt=0x20000, cnt_bytes=4096), _lib.EWORKSPACE),
+    (dict(variant=1, splitK=2, ws=0x10000, ws_bytes=1 << 24, cnt=0x20000, cnt_bytes=0), _lib.EWORKSPACE),
+    (dict(variant=1, splitK=2, ws=0x10004, ws_bytes=1 << 24, cnt=0x20000, cnt_bytes=4096), _lib.EALIGN),
     (dict(strideW=2), _lib.EINVAL),
 ])
 def test_packed_forward_rejects(kwargs, code):

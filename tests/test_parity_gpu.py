@@ -256,6 +256,28 @@ def test_config4_decode_bwta(N):
     assert (goth.view(np.uint16) == f16_of(want).view(np.uint16)).all()
 
 
+@pytest.mark.parametrize("M,N,K", [(11008, 17, 4096), (11008, 40, 4096), (4096, 100, 4096), (1000, 130, 2304), (70, 250, 1000)])
+def test_decode_batches_of_ternary_rows(M, N, K):
+    """More than 16 ternary rows (a batch of decode steps): the two bit planes are taken 16 rows at a time by the
+    kernel that splits K inside a block, also over ragged M, N and K; same integers as the dense reference, and the
+    same through the other kernel families."""
+    rng = np.random.default_rng(M + N)
+    w = np.where(rng.integers(0, 2, (M, K)) == 1, np.float16(-1), np.float16(1)).astype(np.float16)
+    t = rng.choice(np.array([-1, 0, 0, 1], dtype=np.float16), size=(N, K)).astype(np.float16)
+    want = dense_ref(MODE_BWTA, w, t)
+    wp, xt = lk.pack_sign(to_dev(w)), lk.pack_ternary(to_dev(t))
+    for variant in [VARIANT_AUTO] + VARIANTS:
+        got = lk.bgemm_packed_forward(wp, xt, MODE_BWTA, torch.int32, 1, variant)[0].cpu().numpy()
+        assert (got == want).all(), variant
+    goth = lk.bgemm_packed_forward(wp, xt, MODE_BWTA, torch.half, 8)[0].cpu().numpy()
+    assert (goth.view(np.uint16) == f16_of(want).view(np.uint16)).all()
+    # a batch of weight matrices against shared rows
+    wp3 = lk.PackedBits(torch.cat([wp.data, wp.data.flip(1)], 0), None, 2, M, K)
+    got3 = lk.bgemm_packed_forward(wp3, xt, MODE_BWTA, torch.int32)
+    assert (got3[0].cpu().numpy() == want).all()
+    assert torch.equal(got3[1], lk.bgemm_packed_forward(lk.PackedBits(wp.data.flip(1).contiguous(), None, 1, M, K), xt, MODE_BWTA, torch.int32)[0])
+
+
 def test_config3_attention_av_batched():
     rng = np.random.default_rng(3000)
     B, S, D = 24, 512, 64                      # 24 of the 192 heads element by element
@@ -402,10 +424,9 @@ def test_dropin_argument_errors():
 @pytest.mark.parametrize("variant", VARIANTS)
 @pytest.mark.parametrize("M,N,K,splits", [(130, 170, 16384, (2,)), (100, 200, 40000, (3, 5, 8)), (300, 260, 24800, (2, 4))])
 def test_split_k_handover_long_k(oracle, variant, M, N, K, splits):
-    """Shapes with few output tiles and a long K, where the cross-block split-K really happens (K is only
-    split while every range keeps 24 K-tiles): partial tiles through the workspace, tickets, all output kinds.
-    With two bit planes the general kernel takes these shapes (and so does the VALU family with one); with one
-    plane the matrix-core family hands them to the kernel that splits K inside a block, without a workspace."""
+    """Shapes with few output tiles and a long K, where K is really split: across blocks in the VALU family (K is
+    only split while every range keeps 24 K-tiles; partial tiles through the workspace, tickets), among the waves
+    of a block, without a workspace, in the matrix-core family.  All modes and output kinds."""
     import _lib
     rng = np.random.default_rng(M + N + K)
     w, x = rand_f16(rng, M, K), rand_f16(rng, N, K)
@@ -416,7 +437,7 @@ def test_split_k_handover_long_k(oracle, variant, M, N, K, splits):
     wp, xp, xt = lk.pack_sign(to_dev(w)), lk.pack_sign(to_dev(x)), lk.pack_ternary(to_dev(x))
     L = _lib.lib()
     for sk in splits:
-        assert L.bgemm_packed_workspace_bytes(MODE_BWTA, 1, M, N, K, sk, variant) > 0      # it does split
+        assert (L.bgemm_packed_workspace_bytes(MODE_BWTA, 1, M, N, K, sk, variant) > 0) == (variant == VARIANT_VALU)
         for mode in (MODE_XOR, MODE_ATTN, MODE_BWTA):
             got = lk.bgemm_packed_forward(wp, xt if mode == MODE_BWTA else xp, mode, torch.int32, sk, variant)
             assert (got[0].cpu().numpy() == want[mode]).all(), (mode, sk)
