@@ -397,16 +397,17 @@ __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_ker
 // Shapes the skinny kernels take: one group of activation rows always (32 rows, or 16 rows of two bit planes).
 // More groups where splitting K inside the block buys more than the general kernel's 32 x 128 tiles do (timed
 // over sweeps of shapes, pieces = 32 x 32 outputs resp. 16 x 32 of two planes): up to 512 pieces from four
-// K-tiles on, up to 1024 from eight, up to 2048 from sixteen.  The last bound is set by weights that come from
-// HBM rather than from a warm cache (a model's layers): there the general kernel's serial K loop pays the
-// full memory latency per step and loses by 15 to 50 %, while on cache-resident operands it would win the
-// range from 1024 to 2048 pieces by up to 7 %.  Beyond that the general kernel's larger tiles re-read less.
+// K-tiles on, up to 1024 from eight, up to 1792 from sixteen and 2048 from 32.  The last bounds are set by
+// weights that come from HBM rather than from a warm cache (a model's layers): there the general kernel's
+// serial K loop pays the full memory latency per step and loses by 15 to 50 %, while on cache-resident
+// operands it would win the range from 1024 pieces on by up to 7 %.  Beyond that the general kernel's
+// larger tiles re-read less.
 bool gemm_skinny_shape(int planes, int64_t batch, int64_t M, int64_t N, int64_t K)
 {
     const int rows = planes == 2 ? 16 : 32;      // activation rows of one piece
     if (N <= rows) return true;
     const int64_t pieces = batch * row_tiles(M) * cdiv(N, rows), KT = k_tiles(K);
-    if (KT >= 16) return pieces <= 2048;
+    if (KT >= 16) return pieces <= (KT >= 32 ? 2048 : 1792);
     if (KT >= 8) return pieces <= 1024;
     return KT >= 4 && pieces <= 512;
 }
