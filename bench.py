@@ -25,7 +25,7 @@ for _p in (ROOT, os.path.join(ROOT, "bgemm-cuda_amd")):
 INT8_MFMA_PEAK_TOPS = 5000.0      # MI355X dense int8 MFMA, published
 FP4_MFMA_PEAK_TOPS = 10100.0      # MI355X dense fp4 MFMA, published
 HBM_PEAK_GBS = 8000.0             # MI355X HBM3E, published
-MEASURED_TRAFFIC_BYTES_C5_FP4 = int((101.9 + 265.0) * 2 ** 20)   # fetched + written, rocprofv3 --pmc
+MEASURED_TRAFFIC_BYTES_C5_FP4 = int((96.5 + 257.0) * 2 ** 20)   # fetched + written, rocprofv3 --pmc
 
 
 def log(*a):
