@@ -16,6 +16,7 @@
 #include "common.h"
 #include "mfma_engines.h"
 #include "pack_bits.h"
+#include <type_traits>
 
 namespace bgemm {
 
@@ -205,7 +206,8 @@ __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_ker
     __shared__ int sPa[32], sPb[32];
     __shared__ __align__(16) unsigned char sX[FUSEX ? KW : 1][FUSEX ? MAXT : 1][FUSEX ? 1024 : 16];
 
-    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: K ranges and their addresses stay scalar
+    // the wave index as a scalar: the wave's K range and every address derived from it stay on the scalar unit
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int rt = blockIdx.x, b = blockIdx.z;   // weight row tile, matrix of the batch
     // this block's activation rows: tile row blockIdx.y, or with two bit planes its half blockIdx.y & 1 (16 rows
     // of both planes fill the 32 operand rows)
@@ -376,21 +378,20 @@ __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_ker
     };
     const int64_t out0 = (int64_t)b * a.strideC;
     const int M = (int)a.M;
+    auto elements = [&](auto kind) {
+        outputs([&](const int n, const int m, const int val) {
+            if (m < M) store_out_as<decltype(kind)::value>(a, out0 + (int64_t)n * M, m, val);
+        });
+    };
     switch (a.out_kind) {
-    case BGEMM_OUT_I32:
-        outputs([&](const int n, const int m, const int val) { if (m < M) store_out_as<BGEMM_OUT_I32>(a, out0 + (int64_t)n * M, m, val); });
-        break;
-    case BGEMM_OUT_F16:
-        outputs([&](const int n, const int m, const int val) { if (m < M) store_out_as<BGEMM_OUT_F16>(a, out0 + (int64_t)n * M, m, val); });
-        break;
-    case BGEMM_OUT_F32_SCALED:
-        outputs([&](const int n, const int m, const int val) { if (m < M) store_out_as<BGEMM_OUT_F32_SCALED>(a, out0 + (int64_t)n * M, m, val); });
-        break;
-    case BGEMM_OUT_F16_SCALED:
-        outputs([&](const int n, const int m, const int val) { if (m < M) store_out_as<BGEMM_OUT_F16_SCALED>(a, out0 + (int64_t)n * M, m, val); });
-        break;
+    case BGEMM_OUT_I32: elements(std::integral_constant<int, BGEMM_OUT_I32>{}); break;
+    case BGEMM_OUT_F16: elements(std::integral_constant<int, BGEMM_OUT_F16>{}); break;
+    case BGEMM_OUT_F32_SCALED: elements(std::integral_constant<int, BGEMM_OUT_F32_SCALED>{}); break;
+    case BGEMM_OUT_F16_SCALED: elements(std::integral_constant<int, BGEMM_OUT_F16_SCALED>{}); break;
     default:        // the bits kinds: every lane takes part in the ballot
-        outputs([&](const int n, const int m, const int val) { store_bits_word(a, b, n, (int64_t)rt * 32, m < M ? next_sign_bit(a, m, val) : 0u); });
+        outputs([&](const int n, const int m, const int val) {
+            store_bits_word(a, b, n, (int64_t)rt * 32, m < M ? next_sign_bit(a, m, val) : 0u);
+        });
     }
 }
 
