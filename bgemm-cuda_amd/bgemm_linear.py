@@ -354,6 +354,41 @@ class BGEMMChain(nn.Sequential):
                                                     next_zero_point=layers[i + 1].zpa.detach().reshape(1))
 
 
+class GraphedInference:
+    """``module(x)`` under ``no_grad`` captured once into a HIP graph and replayed per call: the launches of a
+    binary layer, chain or block are a few microseconds each, less than it costs to issue them from Python, so a
+    replay (one call into the runtime) is what makes a small model run at the speed of its kernels.
+
+    The capture fixes the input's shape and dtype, the packed weights and every buffer: parameters updated in
+    place afterwards (scales, biases) are seen, a changed or replaced weight is not (capture again).  The
+    returned tensor is the graph's own output buffer, overwritten by the next call.  Not in the reference."""
+
+    def __init__(self, module, example):
+        if not example.is_cuda:
+            raise ValueError("the example input must be on the GPU")
+        self.module = module
+        self._x = example.detach().clone()
+        with torch.no_grad():
+            side = torch.cuda.Stream(device=example.device)
+            side.wait_stream(torch.cuda.current_stream(example.device))
+            with torch.cuda.stream(side):
+                for _ in range(2):                 # initialises scales, packs weights, grows cached buffers
+                    module(self._x)
+                side.synchronize()
+                self._graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(self._graph, stream=side):
+                    self._y = module(self._x)
+            torch.cuda.current_stream(example.device).wait_stream(side)
+
+    def __call__(self, x):
+        if x.shape != self._x.shape or x.dtype != self._x.dtype or x.device != self._x.device:
+            raise ValueError("captured for %s %s on %s, got %s %s on %s" % (tuple(self._x.shape), self._x.dtype,
+                             self._x.device, tuple(x.shape), x.dtype, x.device))
+        self._x.copy_(x)
+        self._graph.replay()
+        return self._y
+
+
 class BGEMMLinear_bireal(BGEMMLinear):
     """BGEMMLinear with the Bi-Real backward (bgemm_linear.py:489-516)."""
     _fn = bgemm_linear_bireal

@@ -265,6 +265,37 @@ def test_elastic_inference_runs_on_packed_operands_without_host_reads(dtype):
             assert torch.equal(lin(x), want3)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.half])
+def test_graphed_inference_replays_equal_eager(dtype):
+    """A chain captured into a HIP graph gives, replay after replay and with eager work in between, what the eager
+    forward gives for the same input; scales changed in place are seen; another shape is refused."""
+    torch.manual_seed(12)
+    chain = bl.BGEMMChain(bl.BGEMMLinear(300, 256, bias=True), bl.BGEMMLinear(256, 512), bl.BGEMMLinear(512, 10, bias=True)).to(DEV).to(dtype)
+    xs = [torch.randn(64, 300, device=DEV, dtype=dtype) for _ in range(4)]
+    with torch.no_grad():
+        chain(xs[0])                                  # first call initialises the layers
+        fast = bl.GraphedInference(chain, xs[0])
+        for i in (1, 2, 0, 3, 1):
+            want = chain(xs[i])                       # eager launches between the replays
+            got = fast(xs[i])
+            assert got.dtype == want.dtype and torch.equal(got, want), i
+        chain[1].sw.mul_(0.5)
+        chain[2].bias.add_(1.0)
+        assert torch.equal(fast(xs[2]), chain(xs[2]))
+        with pytest.raises(ValueError):
+            fast(xs[0][:32])
+    # a single layer and the attention block capture the same way
+    import attention_demo
+    block = attention_demo.BinarySelfAttention(128, 4).to(DEV)
+    x = torch.randn(2, 64, 128, device=DEV)
+    with torch.no_grad():
+        block(x)
+        fast = bl.GraphedInference(lambda t: block(t)[0], x)
+        for _ in range(3):
+            x = torch.randn(2, 64, 128, device=DEV)
+            assert torch.equal(fast(x), block(x)[0])
+
+
 def test_config2_mlp_forward_bitwise(oracle):
     """Benchmark configuration 2: 784 -> 4096 -> 4096 -> 10, batch 128, fp16 outputs vs the CPU chain."""
     g = torch.Generator().manual_seed(1002)
