@@ -5,7 +5,7 @@ The reference vendors a quantised BERT whose self-attention still multiplies wit
 wiring the binary kernels in as open work.  This block is that wiring, forward and backward:
 the four projections are ``BGEMMLinear`` layers, the scores are ``bgemm_matmul(q, k^T)`` on the
 sign bits of Q and K, and the context is ``bgemm_attn_matmul(a, v)`` with the probabilities binarised
-to {0,1} (1 where a probability is at least its row's mean) and V to {-1,+1}.  ``kernels=False``
+to {0,1} (1 where a probability is at least the uniform level 1/S, its row's mean) and V to {-1,+1}.  ``kernels=False``
 evaluates the same block with dense torch matmuls on the de-binarised tensors, which is what the
 tests compare against, bit for bit.
 
@@ -53,11 +53,13 @@ class BinarySelfAttention(nn.Module):
             scores = bgemm_matmul.apply(q, k.transpose(-1, -2))
         else:
             scores = torch.matmul(_pm1(q.half()).float(), _pm1(k.half()).float().transpose(-1, -2)).half()
-        scores = scores.float() / math.sqrt(self.attention_head_size)
+        # the scores are small integers held in fp16 (the kernel's output type); the elementwise work between the
+        # two matmuls stays in fp16 storage, which is a third of the memory traffic of an fp32 round trip
+        scores = scores / math.sqrt(self.attention_head_size)
         if attention_mask is not None:
-            scores = scores + attention_mask
+            scores = scores + attention_mask.to(scores.dtype)
         probs = torch.softmax(scores, dim=-1)
-        centred = probs - probs.mean(dim=-1, keepdim=True)          # {0,1}: at least the row's mean
+        centred = probs - 1.0 / probs.shape[-1]                     # {0,1}: at least the uniform level 1/S
         if self.kernels:
             context = bgemm_attn_matmul.apply(centred, v)
         else:

@@ -356,6 +356,8 @@ extern "C" int bgemm_pack_batched(const void* src, int src_dtype, int ternary, c
                        "bgemm_pack_batched", batch_outer, batch_inner, stride_outer, stride_inner);
 }
 
+namespace bgemm {
+
 // Transposed source ([K][rows] in memory): a wave builds one 32-row x 256-bit tile.  For each of its
 // four words, lane (h, k') reads the 32 consecutive fp16 of source row k = 256 kt + 128 h + 32 q + k'
 // (four 16-byte loads when the source allows, all sixteen in flight), gathers their sign bits into a
@@ -431,6 +433,8 @@ __global__ __launch_bounds__(256) void pack_transposed_kernel(const void* __rest
     for (int q = 0; q < 4; q++) w[q] = __brev(transpose32(w[q], lane));
     dst[tile * TILE_U4 + lane] = make_uint4(w[0], w[1], w[2], w[3]);
 }
+
+}  // namespace bgemm
 
 extern "C" int bgemm_pack_transposed_batched(const void* src, int src_dtype, int64_t batch_outer, int64_t batch_inner,
                                              int64_t rows, int64_t K, int64_t ld, int64_t stride_outer,
