@@ -197,33 +197,40 @@ __global__ __launch_bounds__(256) void gemm_skinny_stream_kernel(const GemmArgs 
 // FUSEX: the activations arrive unpacked (fp16 or fp32 rows, optionally minus a zero point): every wave
 // builds the activation tiles of its own K range itself, in LDS, while its weight loads are in flight,
 // which saves the separate pack launch of a decode step (a third of its time).  One tile row, batch == 1.
-template <typename Eng, int KW, bool FUSEX = false>
+// Two bit planes (a ternary operand): 16 rows of both planes share one 32-row operand, rows 0..15 from the
+// nonzero plane and 16..31 from the sign plane, so one MFMA yields both dots; up to 32 rows are taken that way,
+// 16 a block (blockIdx.y & 1 picks the half of the tile row).  PL2: more rows than that; every block takes 32
+// rows of each plane as two operands against one expansion of the weight tile, two accumulators, which halves
+// the blocks and the weight traffic (64 to 128 rows: 8 to 15 % faster; up to 32 rows the half blocks win by
+// 10 to 20 %, twice the blocks with half the matrix-core chain each).
+template <typename Eng, int KW, bool FUSEX = false, bool PL2 = false>
 __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_kernel(const GemmArgs a)
 {
-    constexpr int NT = KW * 64;
+    static_assert(!(FUSEX && PL2), "in-kernel activation packing is built for up to four rows");
+    constexpr int NT = KW * 64, NP = PL2 ? 2 : 1;
     constexpr int MAXT = FUSEX ? 2 : 4;
-    __shared__ int sAcc[16][64];                 // accumulator layout of the MFMA: [v][lane]
-    __shared__ int sPa[32], sPb[32];
+    __shared__ int sAcc[NP][16][64];             // accumulator layout of the MFMA: [v][lane]
+    __shared__ int sPa[32], sPb[NP][32];
     __shared__ __align__(16) unsigned char sX[FUSEX ? KW : 1][FUSEX ? MAXT : 1][FUSEX ? 1024 : 16];
 
     // the wave index as a scalar: the wave's K range and every address derived from it stay on the scalar unit
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int rt = blockIdx.x, b = blockIdx.z;   // weight row tile, matrix of the batch
-    // this block's activation rows: tile row blockIdx.y, or with two bit planes its half blockIdx.y & 1 (16 rows
-    // of both planes fill the 32 operand rows)
-    const bool two = a.mc.planes == 2;
+    const bool two = !PL2 && a.mc.planes == 2;   // both planes in one operand, 16 rows a block
     const int nt = two ? blockIdx.y >> 1 : blockIdx.y, nbase = two ? blockIdx.y * 16 : blockIdx.y * 32;
 
     int kt0, kt1;
     split_range(a.KT, KW, wave, &kt0, &kt1);
 
-    const uint4* const xp = FUSEX ? nullptr : skinny_x_ptr(a, b, lane, blockIdx.y & 1) + (int64_t)nt * a.KT * TILE_U4;
+    const uint4* const xp = FUSEX ? nullptr
+                            : (PL2 ? a.X + lane + (int64_t)b * a.strideX : skinny_x_ptr(a, b, lane, blockIdx.y & 1)) + (int64_t)nt * a.KT * TILE_U4;
+    const uint4* const xp2 = PL2 ? a.X2 + lane + (int64_t)b * a.strideX + (int64_t)nt * a.KT * TILE_U4 : nullptr;
     const uint4* wp = a.W + (int64_t)b * a.strideW + (int64_t)rt * a.KT * TILE_U4 + lane;
 
-    typename Eng::Acc acc;
+    typename Eng::Acc acc, acc2;                 // acc2: the second plane's dots (PL2)
 #pragma unroll
-    for (int v = 0; v < 16; v++) acc[v] = 0;
-    int pa = 0, pb = 0;
+    for (int v = 0; v < 16; v++) acc[v] = acc2[v] = 0;
+    int pa = 0, pb = 0, pb2 = 0;
 
     // FUSEX: the activation tiles of this wave's K-tiles are built by the wave in its own LDS area: row n of
     // the source goes to operand row n (sign bits) or, with two planes, its nonzero bits to row n and
@@ -265,7 +272,7 @@ __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_ker
     // the wave's K range is short (K / KW) and requested MAXT K-tiles at a time: the kernel lives
     // on memory-level parallelism
     for (int kb = kt0; kb < kt1 || kb == kt0; kb += MAXT) {
-        uint4 xq[MAXT], wq[MAXT], xraw[FUSEX ? MAXT : 1][FUSEX ? 2 : 1];
+        uint4 xq[MAXT], xq2[PL2 ? MAXT : 1], wq[MAXT], xraw[FUSEX ? MAXT : 1][FUSEX ? 2 : 1];
         if (kb < kt1) {
             if (FUSEX && xfast) {
 #pragma unroll
@@ -284,6 +291,7 @@ __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_ker
                 if (kb + q >= kt1) break;                       // wave-uniform: no load for a K-tile past the range
                 const int64_t off = (int64_t)(kb + q) * TILE_U4;
                 if (!FUSEX) xq[q] = xp[off];
+                if (PL2) xq2[q] = xp2[off];
                 wq[q] = load_stream(wp + off);
             }
             if (FUSEX) {
@@ -326,8 +334,11 @@ __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_ker
         if (kb == kt0) {
             // clear the meeting area while the first loads are in flight: every wave gets here at
             // once, so this barrier costs next to nothing
-            for (int i = threadIdx.x; i < 16 * 64; i += NT) (&sAcc[0][0])[i] = 0;
-            if (threadIdx.x < 32) sPa[threadIdx.x] = sPb[threadIdx.x] = 0;
+            for (int i = threadIdx.x; i < NP * 16 * 64; i += NT) (&sAcc[0][0][0])[i] = 0;
+            if (threadIdx.x < 32) {
+                sPa[threadIdx.x] = sPb[0][threadIdx.x] = 0;
+                if (PL2) sPb[NP - 1][threadIdx.x] = 0;
+            }
             __syncthreads();
         }
         if (kb < kt1) {
@@ -336,8 +347,13 @@ __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_ker
                 if (kb + q >= kt1) break;
                 pa += popc4(wq[q]);
                 pb += popc4(xq[q]);
+                if (PL2) pb2 += popc4(xq2[q]);
 #pragma unroll
-                for (int s = 0; s < Eng::STEPS; s++) acc = Eng::mma(Eng::expand_x(xq[q], s), Eng::expand_w(wq[q], s), acc);
+                for (int s = 0; s < Eng::STEPS; s++) {
+                    const typename Eng::Frag bw = Eng::expand_w(wq[q], s);
+                    acc = Eng::mma(Eng::expand_x(xq[q], s), bw, acc);
+                    if (PL2) acc2 = Eng::mma(Eng::expand_x(xq2[PL2 ? q : 0], s), bw, acc2);
+                }
             }
         }
     }
@@ -345,6 +361,7 @@ __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_ker
     // ---- meet in LDS: integer adds of the accumulator rows that carry outputs ------------------------
     pa += __shfl_xor(pa, 32);
     pb += __shfl_xor(pb, 32);
+    if (PL2) pb2 += __shfl_xor(pb2, 32);
     if (kt0 < kt1) {
         // accumulator registers 4g .. 4g + 3 hold operand rows 8g .. 8g + 7: whole groups past the last real row
         // are skipped (a branch the wave takes as one), rows past it inside a group are added and never read
@@ -353,11 +370,15 @@ __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_ker
         for (int g = 0; g < 4; g++) {
             if (8 * (two ? (g & 1) : g) >= nrows) continue;
 #pragma unroll
-            for (int v = 4 * g; v < 4 * g + 4; v++) atomicAdd(&sAcc[v][lane], Eng::to_int(acc, v));
+            for (int v = 4 * g; v < 4 * g + 4; v++) {
+                atomicAdd(&sAcc[0][v][lane], Eng::to_int(acc, v));
+                if (PL2) atomicAdd(&sAcc[NP - 1][v][lane], Eng::to_int(acc2, v));
+            }
         }
         if (lane < 32) {
             atomicAdd(&sPa[lane], pa);
-            atomicAdd(&sPb[lane], pb);
+            atomicAdd(&sPb[0][lane], pb);
+            if (PL2) atomicAdd(&sPb[NP - 1][lane], pb2);
         }
     }
     __syncthreads();
@@ -371,9 +392,10 @@ __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_ker
         for (int o = threadIdx.x; o < nout; o += NT) {
             const int nl = o >> 5, c = o & 31;
             const int v = 4 * (nl >> 3) + (nl & 3), hh = (nl >> 2) & 1;   // accumulator slot of operand row nl
-            const int d = sAcc[v][hh * 32 + c];
-            const int d2 = two ? sAcc[v + 8][hh * 32 + c] : 0;
-            store(nbase + nl, rt * 32 + c, skinny_value(mc, two, kbits, sPa[c], sPb[nl], two ? sPb[nl + 16] : 0, d, d2));
+            const int d = sAcc[0][v][hh * 32 + c];
+            const int d2 = PL2 ? sAcc[NP - 1][v][hh * 32 + c] : two ? sAcc[0][v + 8][hh * 32 + c] : 0;
+            const int rb2 = PL2 ? sPb[NP - 1][nl] : two ? sPb[0][nl + 16] : 0;
+            store(nbase + nl, rt * 32 + c, skinny_value(mc, two || PL2, kbits, sPa[c], sPb[0][nl], rb2, d, d2));
         }
     };
     const int64_t out0 = (int64_t)b * a.strideC;
@@ -397,17 +419,15 @@ __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_ker
 
 // Shapes the skinny kernels take: one group of activation rows always (32 rows, or 16 rows of two bit planes).
 // More groups where splitting K inside the block buys more than the general kernel's 32 x 128 tiles do (timed
-// over sweeps of shapes, pieces = 32 x 32 outputs resp. 16 x 32 of two planes): up to 512 pieces from four
-// K-tiles on, up to 1024 from eight, up to 1792 from sixteen and 2048 from 32.  The last bounds are set by
-// weights that come from HBM rather than from a warm cache (a model's layers): there the general kernel's
-// serial K loop pays the full memory latency per step and loses by 15 to 50 %, while on cache-resident
-// operands it would win the range from 1024 pieces on by up to 7 %.  Beyond that the general kernel's
-// larger tiles re-read less.
+// over sweeps of shapes, pieces = 32 x 32 outputs): up to 512 pieces from four K-tiles on, up to 1024 from
+// eight, up to 1792 from sixteen and 2048 from 32.  The last bounds are set by weights that come from HBM
+// rather than from a warm cache (a model's layers): there the general kernel's serial K loop pays the full
+// memory latency per step and loses by 15 to 50 %, while on cache-resident operands it would win the range
+// from 1024 pieces on by up to 7 %.  Beyond that the general kernel's larger tiles re-read less.
 bool gemm_skinny_shape(int planes, int64_t batch, int64_t M, int64_t N, int64_t K)
 {
-    const int rows = planes == 2 ? 16 : 32;      // activation rows of one piece
-    if (N <= rows) return true;
-    const int64_t pieces = batch * row_tiles(M) * cdiv(N, rows), KT = k_tiles(K);
+    if (N <= (planes == 2 ? 16 : 32)) return true;
+    const int64_t pieces = batch * row_tiles(M) * row_tiles(N), KT = k_tiles(K);
     if (KT >= 16) return pieces <= (KT >= 32 ? 2048 : 1792);
     if (KT >= 8) return pieces <= 1024;
     return KT >= 4 && pieces <= 512;
@@ -431,7 +451,8 @@ template <typename Eng>
 static int launch_splitk(const GemmArgs& a, hipStream_t st)
 {
     const int64_t blocks = (int64_t)a.batch * a.MT;
-    const int64_t groups = a.mc.planes == 2 ? cdiv(a.N, 16) : a.NT;      // activation rows a block takes: 16 of two planes, or 32
+    const bool pl2 = a.mc.planes == 2 && a.N > 32;      // two operands a block
+    const int64_t groups = a.mc.planes == 2 && !pl2 ? cdiv(a.N, 16) : a.NT;      // 16 rows of two planes a block, else 32 rows
     if (groups > 65535 || a.batch > 65535)
         return fail(BGEMM_EINVAL, "gemm_skinny: grid of %lld x %lld x %lld blocks", (long long)a.MT, (long long)groups, (long long)a.batch);
     // K ways per block: at least what the caller asked for, more when the grid alone would leave the
@@ -439,7 +460,12 @@ static int launch_splitk(const GemmArgs& a, hipStream_t st)
     int kw = 1;
     while (kw < 8 && (kw < a.splitK || blocks * groups * kw < 4096) && kw * 2 <= a.KT) kw *= 2;
     const dim3 g((unsigned)a.MT, (unsigned)groups, (unsigned)a.batch);
-    if (kw == 1) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 1>), g, dim3(64), 0, st, a);
+    if (pl2) {
+        if (kw == 1) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 1, false, true>), g, dim3(64), 0, st, a);
+        else if (kw == 2) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 2, false, true>), g, dim3(128), 0, st, a);
+        else if (kw == 4) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 4, false, true>), g, dim3(256), 0, st, a);
+        else hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 8, false, true>), g, dim3(512), 0, st, a);
+    } else if (kw == 1) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 1>), g, dim3(64), 0, st, a);
     else if (kw == 2) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 2>), g, dim3(128), 0, st, a);
     else if (kw == 4) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 4>), g, dim3(256), 0, st, a);
     else hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 8>), g, dim3(512), 0, st, a);
