@@ -284,6 +284,15 @@ def test_graphed_inference_replays_equal_eager(dtype):
         assert torch.equal(fast(xs[2]), chain(xs[2]))
         with pytest.raises(ValueError):
             fast(xs[0][:32])
+    # a decode step (one row: the kernel that packs its own activations) captures too
+    lin = bl.BGEMMLinear(4096, 1000, bias=True).to(DEV).to(dtype)
+    with torch.no_grad():
+        lin(torch.randn(8, 4096, device=DEV, dtype=dtype))
+        x1 = torch.randn(1, 4096, device=DEV, dtype=dtype)
+        step = bl.GraphedInference(lin, x1)
+        for _ in range(3):
+            x1 = torch.randn(1, 4096, device=DEV, dtype=dtype)
+            assert torch.equal(step(x1), lin(x1))
     # a single layer and the attention block capture the same way
     import attention_demo
     block = attention_demo.BinarySelfAttention(128, 4).to(DEV)
