@@ -152,6 +152,9 @@ __global__ __launch_bounds__(256) void gemm_skinny_stream_kernel(const GemmArgs 
     };
     if (a.out_kind == BGEMM_OUT_I32 || a.out_kind == BGEMM_OUT_F16) {
         const bool wide = a.out_kind == BGEMM_OUT_I32;
+        // from a handful of rows on the output is a noticeable share of the traffic and is written past the
+        // caches (timed: 5 to 7 % at 6 to 16 rows, while at 1 to 4 rows ordinary stores are 3 % faster)
+        const bool past_cache = wide && a.N > 4;
         const int sh = wide ? 2 : 1;
         const int64_t row_bytes = a.M << sh;
         char* const base = reinterpret_cast<char*>(a.out) + ((out_row0 + m0) << sh) + 4 * h * row_bytes;
@@ -165,7 +168,8 @@ __global__ __launch_bounds__(256) void gemm_skinny_stream_kernel(const GemmArgs 
             for (int t = 0; t < RT; t++) {
                 if (!col_ok[t]) continue;
                 const int val = value(v, t, rowterm);
-                if (wide) *reinterpret_cast<int*>(rowp + t * 128) = val;
+                if (past_cache) __builtin_nontemporal_store(val, reinterpret_cast<int*>(rowp + t * 128));
+                else if (wide) *reinterpret_cast<int*>(rowp + t * 128) = val;
                 else *reinterpret_cast<__half*>(rowp + t * 64) = __float2half_rn((float)val);
             }
         }
