@@ -177,6 +177,7 @@ static int packed_forward(int mode, const void* W_tiled, const void* X_tiled, co
     a.batch = (int)batch; a.splitK = splitK;
     a.vec_store = !bits && (M % 4 == 0) && (strideC % 4 == 0) && (((uintptr_t)out & 15) == 0) ? 4 : 0;
     if (a.vec_store && out_elem_shift(a.out_kind) == 1 && M % 8 == 0 && strideC % 8 == 0) a.vec_store = 8;
+    a.nt_store = batch * N * M * 4 <= (32LL << 20);
     const int v = variant == BGEMM_VARIANT_AUTO ? pick_variant(mode, batch, M, N, K) : variant;
     if (raw) return launch_gemm_skinny(a, (hipStream_t)stream, v == BGEMM_VARIANT_MFMA_F4);
     const bool skinny = v != BGEMM_VARIANT_VALU && gemm_skinny_shape(a.mc.planes, batch, M, N, K);

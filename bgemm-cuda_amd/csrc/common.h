@@ -54,6 +54,7 @@ struct GemmArgs {
     void* out; int out_kind;       // BGEMM_OUT_*
     const void* ep_sw; const void* ep_sa; const void* ep_bias;   // scaled output kinds: per-column scale, scalar, bias
     const void* ep_zp;    // bits kinds: the next layer's zero point (null = 0)
+    int nt_store;         // general kernel: 4-byte outputs are stored past the caches (set for outputs of up to 32 MiB)
     int vec_store;        // 0, or the elements per lane the epilogue may store at once: 4 (rows of `out` 16-byte aligned
                           // for int32, 8-byte for fp16) or 8 (fp16 kinds with rows of a multiple of 8)
     int64_t M, N, K;

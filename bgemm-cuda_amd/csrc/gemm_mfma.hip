@@ -269,6 +269,17 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
         const int64_t nrow0 = (int64_t)(nt0 + i) * 32, mcol0 = (int64_t)mt0 * 32;
         constexpr int C4 = WM * 8;               // int4 per staged row
         constexpr int NP = 32 * C4 / 64;
+        // Stores past the caches (non-temporal) where timing favours them: always for the 2-byte kinds, for the
+        // 4-byte kinds on outputs of up to 32 MiB (a.nt_store); larger int32 outputs are faster with ordinary stores.
+        // (The non-temporal store is written as an instruction: as a builtin next to an ordinary store of the same
+        // value the optimiser merges the two into one ordinary store.)
+        auto store16 = [&](char* const to, const int4 v, const bool past_cache) {
+            if (past_cache) {
+                const v4i x = {v.x, v.y, v.z, v.w};
+                asm volatile("global_store_dwordx4 %0, %1, off nt" : : "v"(to), "v"(x) : "memory");
+            } else
+                *reinterpret_cast<int4*>(to) = v;
+        };
         if (a.vec_store && a.out_kind == BGEMM_OUT_I32) {
             // 16-byte stores: one instruction covers 64 * 4 consecutive elements of the strip.  Eight
             // LDS reads are issued together, then their stores; the address advances by whole rows.
@@ -284,12 +295,17 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
                         int4 q[CHUNK];
 #pragma unroll
                         for (int p = 0; p < CHUNK; p++) q[p] = *reinterpret_cast<const int4*>(sp + (p0 + p) * RSTEP * ROW_I);
+                        if (a.nt_store) {
 #pragma unroll
-                        for (int p = 0; p < CHUNK; p++, dst += dstep) *reinterpret_cast<int4*>(dst) = q[p];
+                            for (int p = 0; p < CHUNK; p++, dst += dstep) store16(dst, q[p], true);
+                        } else {
+#pragma unroll
+                            for (int p = 0; p < CHUNK; p++, dst += dstep) store16(dst, q[p], false);
+                        }
                     }
                 } else {
                     for (int row = row0; nrow0 + row < a.N; row += RSTEP, sp += RSTEP * ROW_I, dst += dstep)
-                        *reinterpret_cast<int4*>(dst) = *reinterpret_cast<const int4*>(sp);
+                        store16(dst, *reinterpret_cast<const int4*>(sp), a.nt_store != 0);
                 }
             }
         } else if (a.vec_store == 8) {
@@ -314,7 +330,7 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
                 union { __half h[8]; uint4 u; } pk;
 #pragma unroll
                 for (int e = 0; e < 8; e++) pk.h[e] = sc ? scaled_f16(q[e], cp[e], saf, has_bias) : __float2half_rn((float)q[e]);
-                *reinterpret_cast<uint4*>(to) = pk.u;
+                store16(to, make_int4((int)pk.u.x, (int)pk.u.y, (int)pk.u.z, (int)pk.u.w), true);
             };
             if (m < a.M) {
                 if (nrow0 + 32 <= a.N && !scaled) {  // uniform: whole strip, plain conversion: reads issued in pairs of rows
@@ -356,7 +372,7 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
                     union { __half h[4]; uint2 u; } pk;
                     switch (a.out_kind) {
                     case BGEMM_OUT_I32:
-                        *reinterpret_cast<int4*>(dst) = q;
+                        store16(dst, q, a.nt_store != 0);
                         break;
                     case BGEMM_OUT_F16:
                         pk.h[0] = __float2half_rn((float)q.x); pk.h[1] = __float2half_rn((float)q.y);
@@ -364,8 +380,9 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
                         *reinterpret_cast<uint2*>(dst) = pk.u;
                         break;
                     case BGEMM_OUT_F32_SCALED:
-                        *reinterpret_cast<float4*>(dst) = make_float4(scaled_f32(q.x, cp[0], saf, has_bias), scaled_f32(q.y, cp[1], saf, has_bias),
-                                                                      scaled_f32(q.z, cp[2], saf, has_bias), scaled_f32(q.w, cp[3], saf, has_bias));
+                        store16(dst, make_int4(__float_as_int(scaled_f32(q.x, cp[0], saf, has_bias)), __float_as_int(scaled_f32(q.y, cp[1], saf, has_bias)),
+                                               __float_as_int(scaled_f32(q.z, cp[2], saf, has_bias)), __float_as_int(scaled_f32(q.w, cp[3], saf, has_bias))),
+                                a.nt_store != 0);
                         break;
                     default:
                         pk.h[0] = scaled_f16(q.x, cp[0], saf, has_bias); pk.h[1] = scaled_f16(q.y, cp[1], saf, has_bias);
