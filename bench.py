@@ -363,6 +363,9 @@ def run_extra(which, quick=False, variant=0):
             for sk in (1, 8):
                 extra.append(bench_c4(2000 // div, 200 // div, N, sk, variant))
                 log(json.dumps(extra[-1]))
+        for N in (32, 64, 128):             # a batch of decode steps, beyond the configuration's row counts
+            extra.append(bench_c4(1000 // div, 100 // div, N, 1, variant))
+            log(json.dumps(extra[-1]))
         for N in (1, 4, 16):
             extra.append(bench_c4_batched(400 // div, N))
             log(json.dumps(extra[-1]))
