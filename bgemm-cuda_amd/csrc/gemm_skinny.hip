@@ -4,15 +4,17 @@
 // read once and streamed past the caches (non-temporal loads); the activation tiles are
 // re-read by every wave and stay cached.
 //
-// Two kernels:
+// Three kernels:
 //  * gemm_skinny_stream_kernel: every wave owns RT weight row tiles over the whole K and keeps
 //    its accumulators to the end: no LDS, no barriers, nothing shared between waves.  Used when
 //    there are enough row tiles (a batch of weight matrices, a very tall one) to fill the chip.
 //  * gemm_skinny_splitk_kernel: a block owns one row tile and its KW waves split K between them
 //    (the in-kernel split-K: no workspace, no second launch, no atomics on global memory); the
 //    partial sums meet in LDS through ds_add.  Used for a single decode-size matrix, which has
-//    too few row tiles to occupy every SIMD otherwise, and, with up to four activation tile rows
-//    per wave, for small batches (N <= 128) against a few thousand weight rows.
+//    too few row tiles to occupy every SIMD otherwise, and, one 32 x 32 piece of the output per
+//    block, for outputs of up to about a thousand such pieces.
+//  * gemm_skinny_splitk_quad_kernel: the same with a 64 x 64 piece per block (four accumulators a
+//    wave), for a few thousand pieces over a long K.
 #include "common.h"
 #include "mfma_engines.h"
 #include "pack_bits.h"
@@ -425,18 +427,167 @@ __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_ker
     }
 }
 
+// ---- split-K kernel, four pieces a block ---------------------------------------------------------
+// The same scheme for outputs of a few thousand pieces (a few hundred activation rows against a few
+// thousand weight rows): a block owns two weight row tiles and two activation tile rows, a 64 x 64 piece
+// of the output, and every wave runs four accumulators over its K range.  Each expanded fragment then
+// feeds two matrix-core instructions instead of one and every tile is fetched by half as many blocks:
+// the 32 x 32 scheme spends more vector-ALU time on expansion than the matrix cores spend on the
+// products.  One bit plane only.  The K range is walked two K-tiles at a time with the next pair in flight.
+template <typename Eng, int KW>
+__global__ __launch_bounds__(KW * 64) void gemm_skinny_splitk_quad_kernel(const GemmArgs a)
+{
+    constexpr int NT = KW * 64, CH = 2;
+    __shared__ int sAcc[2][2][16][64];           // [weight tile][activation tile], then the MFMA's [v][lane]
+    __shared__ int sPa[2][32], sPb[2][32];
+
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int rt0 = blockIdx.x * 2, nt0 = blockIdx.y * 2, b = blockIdx.z;
+    const bool has_w1 = rt0 + 1 < a.MT, has_x1 = nt0 + 1 < a.NT;      // the second tiles exist (else: the first again, unused)
+    int kt0, kt1;
+    split_range(a.KT, KW, wave, &kt0, &kt1);
+
+    const int64_t tile_row = (int64_t)a.KT * TILE_U4;
+    const uint4* const wp0 = a.W + (int64_t)b * a.strideW + rt0 * tile_row + lane;
+    const uint4* const wp1 = wp0 + (has_w1 ? tile_row : 0);
+    const uint4* const xp0 = a.X + (int64_t)b * a.strideX + nt0 * tile_row + lane;
+    const uint4* const xp1 = xp0 + (has_x1 ? tile_row : 0);
+
+    typename Eng::Acc acc[2][2];
+#pragma unroll
+    for (int v = 0; v < 16; v++) acc[0][0][v] = acc[0][1][v] = acc[1][0][v] = acc[1][1][v] = 0;
+    int pa[2] = {0, 0}, pb[2] = {0, 0};
+
+    uint4 wA[CH][2], xA[CH][2], wB[CH][2], xB[CH][2];
+    auto fetch = [&](uint4 (&wq)[CH][2], uint4 (&xq)[CH][2], const int kb) {
+#pragma unroll
+        for (int q = 0; q < CH; q++) {
+            if (kb + q >= kt1) break;                       // wave-uniform: no load for a K-tile past the range
+            const int64_t off = (int64_t)(kb + q) * TILE_U4;
+            xq[q][0] = xp0[off]; xq[q][1] = xp1[off];
+            wq[q][0] = wp0[off]; wq[q][1] = wp1[off];
+        }
+    };
+    auto consume = [&](const uint4 (&wq)[CH][2], const uint4 (&xq)[CH][2], const int kb) {
+#pragma unroll
+        for (int q = 0; q < CH; q++) {
+            if (kb + q >= kt1) break;
+            pa[0] += popc4(wq[q][0]); pa[1] += popc4(wq[q][1]);
+            pb[0] += popc4(xq[q][0]); pb[1] += popc4(xq[q][1]);
+#pragma unroll
+            for (int s = 0; s < Eng::STEPS; s++) {
+                const typename Eng::Frag bw0 = Eng::expand_w(wq[q][0], s), bw1 = Eng::expand_w(wq[q][1], s);
+                const typename Eng::Frag ax0 = Eng::expand_x(xq[q][0], s), ax1 = Eng::expand_x(xq[q][1], s);
+                acc[0][0] = Eng::mma(ax0, bw0, acc[0][0]);
+                acc[1][0] = Eng::mma(ax0, bw1, acc[1][0]);
+                acc[0][1] = Eng::mma(ax1, bw0, acc[0][1]);
+                acc[1][1] = Eng::mma(ax1, bw1, acc[1][1]);
+            }
+        }
+    };
+    fetch(wA, xA, kt0);
+    // the meeting area is cleared while the first loads are in flight
+    for (int i = threadIdx.x; i < 4 * 16 * 64; i += NT) (&sAcc[0][0][0][0])[i] = 0;
+    if (threadIdx.x < 64) (&sPa[0][0])[threadIdx.x] = (&sPb[0][0])[threadIdx.x] = 0;
+    __syncthreads();
+    for (int kb = kt0; kb < kt1; kb += 2 * CH) {
+        fetch(wB, xB, kb + CH);
+        consume(wA, xA, kb);
+        fetch(wA, xA, kb + 2 * CH);
+        consume(wB, xB, kb + CH);
+    }
+
+    // ---- meet in LDS ------------------------------------------------------------------------------
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        pa[i] += __shfl_xor(pa[i], 32);
+        pb[i] += __shfl_xor(pb[i], 32);
+    }
+    if (kt0 < kt1) {
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int nrows = (int)a.N - (nt0 + j) * 32;      // accumulator registers 4g .. 4g + 3 hold operand rows 8g .. 8g + 7
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                if (i && !has_w1) continue;
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    if (8 * g >= nrows) continue;
+#pragma unroll
+                    for (int v = 4 * g; v < 4 * g + 4; v++) atomicAdd(&sAcc[i][j][v][lane], Eng::to_int(acc[i][j], v));
+                }
+            }
+        }
+        if (lane < 32) {
+            atomicAdd(&sPa[0][lane], pa[0]); atomicAdd(&sPa[1][lane], pa[1]);
+            atomicAdd(&sPb[0][lane], pb[0]); atomicAdd(&sPb[1][lane], pb[1]);
+        }
+    }
+    __syncthreads();
+
+    // ---- rank-one terms and store: a wave takes one output row of the piece, 64 consecutive columns ----
+    const ModeCoef mc = a.mc;
+    const int kbits = (int)a.K;
+    const int nout = min((int)a.N - nt0 * 32, 64) * 64;
+    auto outputs = [&](auto store) {
+        for (int o = threadIdx.x; o < nout; o += NT) {
+            const int mm = o & 63, nn = o >> 6;
+            const int i = mm >> 5, c = mm & 31, j = nn >> 5, nl = nn & 31;
+            const int v = 4 * (nl >> 3) + (nl & 3), hh = (nl >> 2) & 1;       // accumulator slot of operand row nl
+            const int d = sAcc[i][j][v][hh * 32 + c];
+            store(nt0 * 32 + nn, rt0 * 32 + mm, i, skinny_value(mc, false, kbits, sPa[i][c], sPb[j][nl], 0, d, 0));
+        }
+    };
+    const int64_t out0 = (int64_t)b * a.strideC;
+    const int M = (int)a.M;
+    auto elements = [&](auto kind) {
+        outputs([&](const int n, const int m, const int, const int val) {
+            if (m < M) store_out_as<decltype(kind)::value>(a, out0 + (int64_t)n * M, m, val);
+        });
+    };
+    switch (a.out_kind) {
+    case BGEMM_OUT_I32:
+        if (a.nt_store)     // a small output that nothing here reads again: written past the caches
+            outputs([&](const int n, const int m, const int, const int val) {
+                if (m < M) __builtin_nontemporal_store(val, reinterpret_cast<int*>(a.out) + out0 + (int64_t)n * M + m);
+            });
+        else
+            elements(std::integral_constant<int, BGEMM_OUT_I32>{});
+        break;
+    case BGEMM_OUT_F16: elements(std::integral_constant<int, BGEMM_OUT_F16>{}); break;
+    case BGEMM_OUT_F32_SCALED: elements(std::integral_constant<int, BGEMM_OUT_F32_SCALED>{}); break;
+    case BGEMM_OUT_F16_SCALED: elements(std::integral_constant<int, BGEMM_OUT_F16_SCALED>{}); break;
+    default:        // the bits kinds: a half-wave holds the 32 columns of one weight row tile, every lane takes part
+        outputs([&](const int n, const int m, const int i, const int val) {
+            store_bits_word(a, b, n, (int64_t)(rt0 + i) * 32, m < M ? next_sign_bit(a, m, val) : 0u);
+        });
+    }
+}
+
+// Shapes the four-pieces kernel takes: one bit plane, at least two tile rows on either side, enough blocks
+// to give every compute unit one, and a K long enough for the shared expansions to outweigh the larger
+// meeting area (timed against both neighbours, weights from HBM and from a warm cache, pieces = 32 x 32
+// outputs): up to 1024 pieces from 16 K-tiles on, 2048 from 24, 3072 from 32, 6144 from 48.  Beyond that
+// the general kernel's 128- and 256-row tiles re-read less.
+static bool skinny_quad_shape(int planes, int64_t batch, int64_t MT, int64_t NT, int64_t KT)
+{
+    if (planes != 1 || MT < 2 || NT < 2 || batch * cdiv(MT, 2) * cdiv(NT, 2) < 256) return false;
+    return batch * MT * NT <= (KT >= 48 ? 6144 : KT >= 32 ? 3072 : KT >= 24 ? 2048 : KT >= 16 ? 1024 : 0);
+}
+
 // Shapes the skinny kernels take: one group of activation rows always (32 rows, or 16 rows of two bit planes).
 // More groups where splitting K inside the block buys more than the general kernel's 32 x 128 tiles do (timed
-// over sweeps of shapes, pieces = 32 x 32 outputs): up to 512 pieces from four K-tiles on, up to 1024 from
-// eight, up to 1792 from sixteen and 2048 from 32.  The last bounds are set by weights that come from HBM
-// rather than from a warm cache (a model's layers): there the general kernel's serial K loop pays the full
-// memory latency per step and loses by 15 to 50 %, while on cache-resident operands it would win the range
-// from 1024 pieces on by up to 7 %.  Beyond that the general kernel's larger tiles re-read less.
+// over sweeps of shapes, pieces = 32 x 32 outputs): up to 512 pieces from four K-tiles on and up to 1024 from
+// eight; two bit planes (two operands a block against one weight expansion) up to 1792 from sixteen and 2048
+// from 32.  The last bounds are set by weights that come from HBM rather than from a warm cache (a model's
+// layers): there the general kernel's serial K loop pays the full memory latency per step.  One bit plane
+// beyond 1024 pieces goes to the four-pieces kernel where that pays (see above), else to the general kernel.
 bool gemm_skinny_shape(int planes, int64_t batch, int64_t M, int64_t N, int64_t K)
 {
     if (N <= (planes == 2 ? 16 : 32)) return true;
     const int64_t pieces = batch * row_tiles(M) * row_tiles(N), KT = k_tiles(K);
-    if (KT >= 16) return pieces <= (KT >= 32 ? 2048 : 1792);
+    if (skinny_quad_shape(planes, batch, row_tiles(M), row_tiles(N), KT)) return true;
+    if (KT >= 16 && planes == 2) return pieces <= (KT >= 32 ? 2048 : 1792);
     if (KT >= 8) return pieces <= 1024;
     return KT >= 4 && pieces <= 512;
 }
@@ -455,9 +606,29 @@ static int launch_splitk_fusex(const GemmArgs& a, hipStream_t st)
     return check_launch("gemm_skinny");
 }
 
+static bool skinny_quad(const GemmArgs& a) { return skinny_quad_shape(a.mc.planes, a.batch, a.MT, a.NT, a.KT); }
+
+template <typename Eng>
+static int launch_splitk_quad(const GemmArgs& a, hipStream_t st)
+{
+    const int64_t gx = cdiv(a.MT, 2), gy = cdiv(a.NT, 2);
+    if (gy > 65535 || a.batch > 65535)
+        return fail(BGEMM_EINVAL, "gemm_skinny: grid of %lld x %lld x %lld blocks", (long long)gx, (long long)gy, (long long)a.batch);
+    // K ways per block: the kernel's registers allow two waves a SIMD, 2048 on the chip
+    int kw = 1;
+    while (kw < 8 && gx * gy * a.batch * kw < 2048 && kw * 2 <= a.KT) kw *= 2;
+    const dim3 g((unsigned)gx, (unsigned)gy, (unsigned)a.batch);
+    if (kw == 1) hipLaunchKernelGGL((gemm_skinny_splitk_quad_kernel<Eng, 1>), g, dim3(64), 0, st, a);
+    else if (kw == 2) hipLaunchKernelGGL((gemm_skinny_splitk_quad_kernel<Eng, 2>), g, dim3(128), 0, st, a);
+    else if (kw == 4) hipLaunchKernelGGL((gemm_skinny_splitk_quad_kernel<Eng, 4>), g, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((gemm_skinny_splitk_quad_kernel<Eng, 8>), g, dim3(512), 0, st, a);
+    return check_launch("gemm_skinny");
+}
+
 template <typename Eng>
 static int launch_splitk(const GemmArgs& a, hipStream_t st)
 {
+    if (skinny_quad(a)) return launch_splitk_quad<Eng>(a, st);
     const int64_t blocks = (int64_t)a.batch * a.MT;
     const bool pl2 = a.mc.planes == 2 && a.N > 32;      // two operands a block
     const int64_t groups = a.mc.planes == 2 && !pl2 ? cdiv(a.N, 16) : a.NT;      // 16 rows of two planes a block, else 32 rows

@@ -278,6 +278,40 @@ def test_decode_batches_of_ternary_rows(M, N, K):
     assert torch.equal(got3[1], lk.bgemm_packed_forward(lk.PackedBits(wp.data.flip(1).contiguous(), None, 1, M, K), xt, MODE_BWTA, torch.int32)[0])
 
 
+@pytest.mark.parametrize("batch,M,N,K", [(1, 4040, 270, 6200), (4, 1000, 250, 4100), (1, 8192, 256, 8192)])
+def test_split_k_in_block_four_pieces_a_block(oracle, batch, M, N, K):
+    """Outputs of one to two thousand 32 x 32 pieces over a long K: a block takes two weight row tiles and two
+    activation tile rows (odd tile counts, ragged M, N and K, batches); every one-plane mode, both engines,
+    every output kind, against the dense reference and the oracle's epilogue."""
+    rng = np.random.default_rng(batch + M + N + K)
+    w = rand_f16(rng, batch * M, K).reshape(batch, M, K)
+    x = rand_f16(rng, batch * N, K).reshape(batch, N, K)
+    wp, xp = lk.pack_sign(to_dev(w)), lk.pack_sign(to_dev(x))
+    for mode in (MODE_XOR, MODE_AND, MODE_ATTN, MODE_ATTN_X):
+        want = np.stack([dense_ref(mode, w[b], x[b]) for b in range(batch)])
+        for variant in (VARIANT_AUTO, VARIANT_MFMA):
+            got = lk.bgemm_packed_forward(wp, xp, mode, torch.int32, 8, variant).cpu().numpy()
+            assert (got == want).all(), (mode, variant)
+        goth = lk.bgemm_packed_forward(wp, xp, mode, torch.half, 1).cpu().numpy()
+        assert (goth.view(np.uint16) == f16_of(want).view(np.uint16)).all(), mode
+    acc = np.stack([dense_ref(MODE_XOR, w[b], x[b]) for b in range(batch)])
+    for dtype in (np.float32, np.float16):
+        sw = rng.uniform(1e-4, 3e-3, M).astype(dtype)
+        sa = np.asarray(1.7371, dtype=dtype)
+        bias = rng.standard_normal(M).astype(dtype)
+        scale = (to_dev(sw), to_dev(sa.reshape(1)), to_dev(bias))
+        y = oracle.np_scale_epilogue(acc.reshape(batch * N, M), sw, sa, bias)
+        got = lk.bgemm_packed_forward(wp, xp, MODE_XOR, scale=scale).cpu().numpy()
+        assert (_bits(got.reshape(batch * N, M)) == _bits(y)).all(), dtype
+        zp = np.asarray(0.013, dtype=dtype)
+        out = lk.bgemm_packed_forward(wp, xp, MODE_XOR, scale=scale, bits_out=lk.zeros_packed(N, M, batch, DEV),
+                                      next_zero_point=to_dev(zp.reshape(1)))
+        wantb = oracle.c_pack_sign(oracle.np_center_to_f16(y, zp))
+        for b in range(batch):
+            one = lk.PackedBits(out.data[b:b + 1], None, 1, N, M)
+            assert (lk.logical_from_tiled(one).cpu().numpy().view(np.uint32) == wantb[b * N:(b + 1) * N]).all(), (dtype, b)
+
+
 def test_config3_attention_av_batched():
     rng = np.random.default_rng(3000)
     B, S, D = 24, 512, 64                      # 24 of the 192 heads element by element
