@@ -458,12 +458,14 @@ __global__ __launch_bounds__(KW * 64) void gemm_skinny_splitk_quad_kernel(const 
     for (int v = 0; v < 16; v++) acc[0][0][v] = acc[0][1][v] = acc[1][0][v] = acc[1][1][v] = 0;
     int pa[2] = {0, 0}, pb[2] = {0, 0};
 
-    uint4 wA[CH][2], xA[CH][2], wB[CH][2], xB[CH][2];
+    uint4 wA[CH][2], xA[CH][2], wB[CH][2], xB[CH][2], wC[CH][2], xC[CH][2];
+    // Every fetch issues all of its loads, a K-tile past the range as the range's last one again (a cache hit,
+    // never multiplied): with loads under a branch the compiler can no longer count how many are in flight
+    // at a use and waits for all of them, the pairs requested ahead included.
     auto fetch = [&](uint4 (&wq)[CH][2], uint4 (&xq)[CH][2], const int kb) {
 #pragma unroll
         for (int q = 0; q < CH; q++) {
-            if (kb + q >= kt1) break;                       // wave-uniform: no load for a K-tile past the range
-            const int64_t off = (int64_t)(kb + q) * TILE_U4;
+            const int64_t off = (int64_t)min(kb + q, kt1 - 1) * TILE_U4;
             xq[q][0] = xp0[off]; xq[q][1] = xp1[off];
             wq[q][0] = wp0[off]; wq[q][1] = wp1[off];
         }
@@ -490,11 +492,14 @@ __global__ __launch_bounds__(KW * 64) void gemm_skinny_splitk_quad_kernel(const 
     for (int i = threadIdx.x; i < 4 * 16 * 64; i += NT) (&sAcc[0][0][0][0])[i] = 0;
     if (threadIdx.x < 64) (&sPa[0][0])[threadIdx.x] = (&sPb[0][0])[threadIdx.x] = 0;
     __syncthreads();
-    for (int kb = kt0; kb < kt1; kb += 2 * CH) {
-        fetch(wB, xB, kb + CH);
+    fetch(wB, xB, kt0 + CH);
+    for (int kb = kt0; kb < kt1; kb += 3 * CH) {       // two pairs ahead of the one being multiplied
+        fetch(wC, xC, kb + 2 * CH);
         consume(wA, xA, kb);
-        fetch(wA, xA, kb + 2 * CH);
+        fetch(wA, xA, kb + 3 * CH);
         consume(wB, xB, kb + CH);
+        fetch(wB, xB, kb + 4 * CH);
+        consume(wC, xC, kb + 2 * CH);
     }
 
     // ---- meet in LDS ------------------------------------------------------------------------------
