@@ -427,6 +427,166 @@ __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_ker
     }
 }
 
+// ---- split-K kernel on the vector ALU: one or two activation vectors ------------------------------
+// With one or two rows the matrix cores have nothing to amortise the bit expansion over (13 vector-ALU
+// instructions per MFMA, of whose 32 output rows a few are used).  Here a lane keeps the weight words of
+// its row and K-half and ANDs them with the same words of each activation vector (NVEC = rows x bit planes,
+// TWO = two planes: vector 2n is row n's nonzero plane, 2n + 1 its sign plane; all lanes of a half-wave read
+// one address), popcounts accumulate per lane, and the meeting in LDS is one integer per lane and vector
+// instead of a 32 x 32 accumulator.  Same grid, K split and epilogue as the matrix-core kernel above.
+// FUSEX: the activations arrive unpacked.  A wave walks its K range 512 elements at a time: lane L loads
+// elements 8L .. 8L + 7 of every row, turns them into a byte of sign (and nonzero) bits, and the 64 bytes of
+// a vector, stored through the wave's own 64 bytes of LDS in big-endian word order, are the sixteen packed
+// words of two K-tiles, which every lane reads back as the two 16-byte pieces its K-half needs.
+template <int KW, int NVEC, bool TWO, bool FUSEX>
+__global__ __launch_bounds__(KW * 64) void gemm_skinny_popc_kernel(const GemmArgs a)
+{
+    static_assert(!TWO || NVEC % 2 == 0, "two planes come in pairs of vectors");
+    constexpr int NT = KW * 64, MAXT = FUSEX ? 2 : 4, ROWS = TWO ? NVEC / 2 : NVEC;
+    __shared__ int sD[NVEC][32], sPa[32], sPb[NVEC];
+    __shared__ __align__(16) unsigned char sXb[FUSEX ? KW : 1][FUSEX ? NVEC : 1][64];
+
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int h = lane >> 5;
+    const int rt = blockIdx.x, b = blockIdx.z;
+    int kt0, kt1;
+    split_range(a.KT, KW, wave, &kt0, &kt1);
+
+    const uint4* const wp = a.W + (int64_t)b * a.strideW + (int64_t)rt * a.KT * TILE_U4 + lane;
+    const uint4* xp[NVEC];
+#pragma unroll
+    for (int j = 0; j < NVEC; j++) {             // a vector past the last row reads the last row again and is not stored
+        const int n = min(TWO ? j >> 1 : j, (int)a.N - 1);
+        xp[j] = FUSEX ? nullptr : ((TWO && (j & 1)) ? a.X2 : a.X) + (int64_t)b * a.strideX + h * 32 + n;
+    }
+    float xzf = 0.f;
+    if (FUSEX && a.xzp)
+        xzf = a.xsrc_f32 ? *reinterpret_cast<const float*>(a.xzp) : __half2float(*reinterpret_cast<const __half*>(a.xzp));
+    const bool xfast = FUSEX && !a.xsrc_f32 && !a.xzp && (a.K & 7) == 0 && ((((uintptr_t)a.xsrc) | (uintptr_t)(a.xld * 2)) & 15) == 0;
+    int d[NVEC], pb[NVEC], pa = 0;
+#pragma unroll
+    for (int j = 0; j < NVEC; j++) d[j] = pb[j] = 0;
+
+    for (int kb = kt0; kb < kt1 || kb == kt0; kb += MAXT) {
+        uint4 wq[MAXT], xq[MAXT][NVEC];
+        if (kb < kt1) {
+            uint32_t xbyte[NVEC];
+            if (FUSEX) {                                        // the rows first: loads return in order
+                const int64_t k0 = (int64_t)kb * TILE_KBITS + 8 * lane;
+                const bool mine = kb + h < kt1;                 // the second K-tile of the pair may be another wave's
+#pragma unroll
+                for (int rr = 0; rr < ROWS; rr++) {
+                    const int n = min(rr, (int)a.N - 1);
+                    uint32_t sg, nz;
+                    if (xfast) {                                // aligned fp16 rows, no zero point: bits straight from one 16-byte load
+                        const uint4 v = (mine && k0 < a.K) ? *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(a.xsrc) + (int64_t)n * a.xld + k0)
+                                                           : make_uint4(0u, 0u, 0u, 0u);
+                        bits8(v, sg, nz);
+                    } else {
+                        uint16_t hb[8];
+                        load8_as_half(reinterpret_cast<const char*>(a.xsrc) + (int64_t)n * a.xld * (a.xsrc_f32 ? 4 : 2), a.xsrc_f32 != 0,
+                                      mine ? k0 : a.K, a.K, a.xzp != nullptr, xzf, hb);
+                        bits8(hb, sg, nz);
+                    }
+                    if (TWO) { xbyte[2 * rr] = nz; xbyte[TWO ? 2 * rr + 1 : 0] = sg & nz; }
+                    else xbyte[rr] = sg;
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < MAXT; q++) {
+                if (kb + q >= kt1) break;                       // wave-uniform: no load for a K-tile past the range
+                const int64_t off = (int64_t)(kb + q) * TILE_U4;
+                if (!FUSEX) {
+#pragma unroll
+                    for (int j = 0; j < NVEC; j++) xq[q][j] = xp[j][off];
+                }
+                wq[q] = load_stream(wp + off);
+            }
+            if (FUSEX) {
+#pragma unroll
+                for (int j = 0; j < NVEC; j++) sXb[wave][j][lane ^ 3] = (unsigned char)xbyte[j];
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+                for (int q = 0; q < MAXT; q++)
+#pragma unroll
+                    for (int j = 0; j < NVEC; j++) xq[q][j] = *reinterpret_cast<const uint4*>(&sXb[wave][j][32 * q + 16 * h]);
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");      // the next pair overwrites the area
+                __builtin_amdgcn_wave_barrier();
+            }
+        }
+        if (kb == kt0) {                                        // cleared while the first loads are in flight
+            if (threadIdx.x < 32) {
+                sPa[threadIdx.x] = 0;
+#pragma unroll
+                for (int j = 0; j < NVEC; j++) sD[j][threadIdx.x] = 0;
+                if (threadIdx.x < NVEC) sPb[threadIdx.x] = 0;
+            }
+            __syncthreads();
+        }
+        if (kb < kt1) {
+#pragma unroll
+            for (int q = 0; q < MAXT; q++) {
+                if (kb + q >= kt1) break;
+                const uint4 w = wq[q];
+                pa += popc4(w);
+#pragma unroll
+                for (int j = 0; j < NVEC; j++) {
+                    const uint4 x = xq[q][j];
+                    pb[j] += popc4(x);
+                    d[j] += popc4(make_uint4(w.x & x.x, w.y & x.y, w.z & x.z, w.w & x.w));
+                }
+            }
+        }
+    }
+
+    // ---- meet in LDS: lane r of either half now adds what its wave found for weight row r -----------
+    pa += __shfl_xor(pa, 32);
+#pragma unroll
+    for (int j = 0; j < NVEC; j++) {
+        d[j] += __shfl_xor(d[j], 32);
+        pb[j] += __shfl_xor(pb[j], 32);
+    }
+    if (kt0 < kt1 && lane < 32) {
+        atomicAdd(&sPa[lane], pa);
+#pragma unroll
+        for (int j = 0; j < NVEC; j++) {
+            atomicAdd(&sD[j][lane], d[j]);
+            if (lane == 0) atomicAdd(&sPb[j], pb[j]);
+        }
+    }
+    __syncthreads();
+
+    // ---- rank-one terms and store: one output per thread ----------------------------------------------
+    const ModeCoef mc = a.mc;
+    const int kbits = (int)a.K;
+    const int nout = (int)a.N * 32;
+    auto outputs = [&](auto store) {
+        for (int o = threadIdx.x; o < nout; o += NT) {
+            const int nl = o >> 5, c = o & 31, j = TWO ? 2 * nl : nl, j2 = TWO ? j + 1 : j;
+            store(nl, rt * 32 + c, skinny_value(mc, TWO, kbits, sPa[c], sPb[j], sPb[j2], sD[j][c], sD[j2][c]));
+        }
+    };
+    const int64_t out0 = (int64_t)b * a.strideC;
+    const int M = (int)a.M;
+    auto elements = [&](auto kind) {
+        outputs([&](const int n, const int m, const int val) {
+            if (m < M) store_out_as<decltype(kind)::value>(a, out0 + (int64_t)n * M, m, val);
+        });
+    };
+    switch (a.out_kind) {
+    case BGEMM_OUT_I32: elements(std::integral_constant<int, BGEMM_OUT_I32>{}); break;
+    case BGEMM_OUT_F16: elements(std::integral_constant<int, BGEMM_OUT_F16>{}); break;
+    case BGEMM_OUT_F32_SCALED: elements(std::integral_constant<int, BGEMM_OUT_F32_SCALED>{}); break;
+    case BGEMM_OUT_F16_SCALED: elements(std::integral_constant<int, BGEMM_OUT_F16_SCALED>{}); break;
+    default:        // the bits kinds: every lane takes part in the ballot
+        outputs([&](const int n, const int m, const int val) {
+            store_bits_word(a, b, n, (int64_t)rt * 32, m < M ? next_sign_bit(a, m, val) : 0u);
+        });
+    }
+}
+
 // ---- split-K kernel, four pieces a block ---------------------------------------------------------
 // The same scheme for outputs of a few thousand pieces (a few hundred activation rows against a few
 // thousand weight rows): a block owns two weight row tiles and two activation tile rows, a 64 x 64 piece
@@ -656,6 +816,36 @@ static int launch_splitk(const GemmArgs& a, hipStream_t st)
     return check_launch("gemm_skinny");
 }
 
+// Vector-ALU kernel: one matrix of the batch per grid plane, one block per weight row tile.
+template <int NVEC, bool TWO, bool FUSEX>
+static int launch_popc(const GemmArgs& a, hipStream_t st)
+{
+    const int64_t blocks = (int64_t)a.batch * a.MT;
+    if (a.batch > 65535) return fail(BGEMM_EINVAL, "gemm_skinny: grid of %lld x 1 x %lld blocks", (long long)a.MT, (long long)a.batch);
+    int kw = 1;
+    while (kw < 8 && (kw < a.splitK || blocks * kw < 4096) && kw * 2 <= a.KT) kw *= 2;
+    const dim3 g((unsigned)a.MT, 1u, (unsigned)a.batch);
+    if (kw == 1) hipLaunchKernelGGL((gemm_skinny_popc_kernel<1, NVEC, TWO, FUSEX>), g, dim3(64), 0, st, a);
+    else if (kw == 2) hipLaunchKernelGGL((gemm_skinny_popc_kernel<2, NVEC, TWO, FUSEX>), g, dim3(128), 0, st, a);
+    else if (kw == 4) hipLaunchKernelGGL((gemm_skinny_popc_kernel<4, NVEC, TWO, FUSEX>), g, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((gemm_skinny_popc_kernel<8, NVEC, TWO, FUSEX>), g, dim3(512), 0, st, a);
+    return check_launch("gemm_skinny");
+}
+
+// One or two vectors (rows x bit planes), packed or not.  From three on the matrix-core kernels are faster:
+// with unpacked activations every further row costs this kernel about a microsecond (all waves of the grid
+// fetch the same few lines of the row at once), timed on W[11008,4096], popcount / matrix cores: one sign row
+// 4.1 / 5.5 us, two 5.1 / 5.6, three 6.7 / 5.9; one ternary row 4.4 / 5.8, two 5.9 / 5.8.
+template <bool FUSEX>
+static bool launch_popc_for(const GemmArgs& a, hipStream_t st, int* rc)
+{
+    const int64_t nvec = a.N * a.mc.planes;
+    if (nvec > 2) return false;
+    if (a.mc.planes == 2) *rc = launch_popc<2, true, FUSEX>(a, st);
+    else *rc = nvec == 1 ? launch_popc<1, false, FUSEX>(a, st) : launch_popc<2, false, FUSEX>(a, st);
+    return true;
+}
+
 template <typename Eng, int RT>
 static int launch_stream(const GemmArgs& a, hipStream_t st)
 {
@@ -678,10 +868,17 @@ bool gemm_skinny_fusex_shape(int planes, int64_t M, int64_t N)
 
 int launch_gemm_skinny(const GemmArgs& a, hipStream_t st, bool fp4)
 {
-    if (a.xsrc) return fp4 ? launch_splitk_fusex<EngF4>(a, st) : launch_splitk_fusex<EngI8>(a, st);
+    // a few vectors: the vector ALU does it with less work than the expansion costs (the int8-engine variant
+    // keeps the matrix-core kernels for every row count)
+    int rc;
+    const int64_t row_tiles = (int64_t)a.batch * a.MT;
+    if (a.xsrc) {
+        if (fp4 && launch_popc_for<true>(a, st, &rc)) return rc;
+        return fp4 ? launch_splitk_fusex<EngF4>(a, st) : launch_splitk_fusex<EngI8>(a, st);
+    }
+    if (fp4 && row_tiles < 4096 && launch_popc_for<false>(a, st, &rc)) return rc;
     // Enough row tiles for about four waves on every SIMD: no K split needed (the result does not
     // depend on it).  Two row tiles per wave share one expansion of the activation tiles.
-    const int64_t row_tiles = (int64_t)a.batch * a.MT;
     if (a.mc.planes == 2 ? a.N <= 16 : a.NT <= 1) {
         if (row_tiles >= 8192) return fp4 ? launch_stream<EngF4, 2>(a, st) : launch_stream<EngI8, 2>(a, st);
         if (row_tiles >= 4096) return fp4 ? launch_stream<EngF4, 1>(a, st) : launch_stream<EngI8, 1>(a, st);

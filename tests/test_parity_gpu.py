@@ -582,6 +582,52 @@ def test_decode_step_packs_its_own_activations(variant, M, N, K):
     assert torch.equal(lk.bgemm_packed_weight_forward(wp, x, MODE_XOR, torch.half), lk.bgemm_packed_forward(wp, lk.pack_sign(x), MODE_XOR, torch.half)[0])
 
 
+@pytest.mark.parametrize("batch,M,N,K", [(1, 11008, 1, 4096), (1, 4100, 2, 1000), (3, 70, 2, 5000), (1, 33, 1, 8), (2, 1000, 1, 11008)])
+def test_one_or_two_rows_on_the_vector_alu(oracle, batch, M, N, K):
+    """One or two activation vectors (rows x bit planes) take the AND-popcount kernel: every mode against the dense
+    reference (batches, ragged M and K, one to 43 K-tiles), fp16, the layer epilogue and the bits output against
+    the oracle, and the same from unpacked fp16 / fp32 rows with a zero point."""
+    rng = np.random.default_rng(batch + M + N + K)
+    w = rand_f16(rng, batch * M, K).reshape(batch, M, K)
+    x = rand_f16(rng, batch * N, K).reshape(batch, N, K)
+    wp, xp = lk.pack_sign(to_dev(w)), lk.pack_sign(to_dev(x))
+    for mode in (MODE_XOR, MODE_AND, MODE_ATTN, MODE_ATTN_X, MODE_BWTA):
+        if mode == MODE_BWTA and N > 1:
+            continue                                    # two ternary rows are four vectors: the matrix-core kernel's
+        want = np.stack([dense_ref(mode, w[b], x[b]) for b in range(batch)])
+        xo = lk.pack_ternary(to_dev(x)) if mode == MODE_BWTA else xp
+        for splitK in (1, 8):
+            got = lk.bgemm_packed_forward(wp, xo, mode, torch.int32, splitK).cpu().numpy()
+            assert (got == want).all(), (mode, splitK)
+        goth = lk.bgemm_packed_forward(wp, xo, mode, torch.half, 1).cpu().numpy()
+        assert (goth.view(np.uint16) == f16_of(want).view(np.uint16)).all(), mode
+        if batch == 1:                                  # the same from the rows as they are
+            for dt in (torch.half, torch.float32):
+                got1 = lk.bgemm_packed_weight_forward(lk.PackedBits(wp.data, None, 1, M, K), to_dev(x[0]).to(dt), mode, torch.int32)
+                assert (got1.cpu().numpy() == want[0]).all(), (mode, dt)
+    acc = np.stack([dense_ref(MODE_XOR, w[b], x[b]) for b in range(batch)]).reshape(batch * N, M)
+    for dtype in (np.float32, np.float16):
+        sw = rng.uniform(1e-4, 3e-3, M).astype(dtype)
+        sa = np.asarray(1.7371, dtype=dtype)
+        bias = rng.standard_normal(M).astype(dtype)
+        scale = (to_dev(sw), to_dev(sa.reshape(1)), to_dev(bias))
+        y = oracle.np_scale_epilogue(acc, sw, sa, bias)
+        got = lk.bgemm_packed_forward(wp, xp, MODE_XOR, scale=scale).cpu().numpy()
+        assert (_bits(got.reshape(batch * N, M)) == _bits(y)).all(), dtype
+        zp = np.asarray(0.013, dtype=dtype)
+        out = lk.bgemm_packed_forward(wp, xp, MODE_XOR, scale=scale, bits_out=lk.zeros_packed(N, M, batch, DEV),
+                                      next_zero_point=to_dev(zp.reshape(1)))
+        wantb = oracle.c_pack_sign(oracle.np_center_to_f16(y, zp))
+        for b in range(batch):
+            one = lk.PackedBits(out.data[b:b + 1], None, 1, N, M)
+            assert (lk.logical_from_tiled(one).cpu().numpy().view(np.uint32) == wantb[b * N:(b + 1) * N]).all(), (dtype, b)
+    if batch == 1:      # unpacked rows with a zero point: the sign bits of (x - zp).half(), as the centring pack forms them
+        xd = to_dev(x[0]).float()
+        zpt = xd.mean().reshape(1)
+        want = lk.bgemm_packed_forward(wp, lk.pack_sign(xd, zero_point=zpt), MODE_XOR, torch.int32, 1, VARIANT_MFMA)[0]
+        assert torch.equal(lk.bgemm_packed_weight_forward(wp, xd, MODE_XOR, torch.int32, x_zero_point=zpt), want)
+
+
 def test_decode_step_larger_batches_fall_back_to_two_launches():
     g = torch.Generator(device=DEV).manual_seed(3)
     w = torch.randn((500, 700), generator=g, device=DEV, dtype=torch.half)
