@@ -594,7 +594,9 @@ __global__ __launch_bounds__(KW * 64) void gemm_skinny_popc_kernel(const GemmArg
 // feeds two matrix-core instructions instead of one and every tile is fetched by half as many blocks:
 // the 32 x 32 scheme spends more vector-ALU time on expansion than the matrix cores spend on the
 // products.  One bit plane only.  The K range is walked two K-tiles at a time with the next pair in flight.
-template <typename Eng, int KW>
+// TWO: a ternary operand; the block's two activation tiles are the two bit planes of ONE tile row (32 rows), so a
+// block is a 32 x 64 piece of the output and the two accumulators of a weight tile combine in the epilogue.
+template <typename Eng, int KW, bool TWO = false>
 __global__ __launch_bounds__(KW * 64) void gemm_skinny_splitk_quad_kernel(const GemmArgs a)
 {
     constexpr int NT = KW * 64, CH = 2;
@@ -602,8 +604,8 @@ __global__ __launch_bounds__(KW * 64) void gemm_skinny_splitk_quad_kernel(const 
     __shared__ int sPa[2][32], sPb[2][32];
 
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int rt0 = blockIdx.x * 2, nt0 = blockIdx.y * 2, b = blockIdx.z;
-    const bool has_w1 = rt0 + 1 < a.MT, has_x1 = nt0 + 1 < a.NT;      // the second tiles exist (else: the first again, unused)
+    const int rt0 = blockIdx.x * 2, nt0 = TWO ? blockIdx.y : blockIdx.y * 2, b = blockIdx.z;
+    const bool has_w1 = rt0 + 1 < a.MT, has_x1 = TWO || nt0 + 1 < a.NT;      // the second tiles exist (else: the first again, unused)
     int kt0, kt1;
     split_range(a.KT, KW, wave, &kt0, &kt1);
 
@@ -611,7 +613,7 @@ __global__ __launch_bounds__(KW * 64) void gemm_skinny_splitk_quad_kernel(const 
     const uint4* const wp0 = a.W + (int64_t)b * a.strideW + rt0 * tile_row + lane;
     const uint4* const wp1 = wp0 + (has_w1 ? tile_row : 0);
     const uint4* const xp0 = a.X + (int64_t)b * a.strideX + nt0 * tile_row + lane;
-    const uint4* const xp1 = xp0 + (has_x1 ? tile_row : 0);
+    const uint4* const xp1 = TWO ? a.X2 + (int64_t)b * a.strideX + nt0 * tile_row + lane : xp0 + (has_x1 ? tile_row : 0);
 
     typename Eng::Acc acc[2][2];
 #pragma unroll
@@ -671,7 +673,7 @@ __global__ __launch_bounds__(KW * 64) void gemm_skinny_splitk_quad_kernel(const 
     if (kt0 < kt1) {
 #pragma unroll
         for (int j = 0; j < 2; j++) {
-            const int nrows = (int)a.N - (nt0 + j) * 32;      // accumulator registers 4g .. 4g + 3 hold operand rows 8g .. 8g + 7
+            const int nrows = (int)a.N - (nt0 + (TWO ? 0 : j)) * 32;      // accumulator registers 4g .. 4g + 3 hold operand rows 8g .. 8g + 7
 #pragma unroll
             for (int i = 0; i < 2; i++) {
                 if (i && !has_w1) continue;
@@ -693,14 +695,15 @@ __global__ __launch_bounds__(KW * 64) void gemm_skinny_splitk_quad_kernel(const 
     // ---- rank-one terms and store: a wave takes one output row of the piece, 64 consecutive columns ----
     const ModeCoef mc = a.mc;
     const int kbits = (int)a.K;
-    const int nout = min((int)a.N - nt0 * 32, 64) * 64;
+    const int nout = min((int)a.N - nt0 * 32, TWO ? 32 : 64) * 64;
     auto outputs = [&](auto store) {
         for (int o = threadIdx.x; o < nout; o += NT) {
             const int mm = o & 63, nn = o >> 6;
-            const int i = mm >> 5, c = mm & 31, j = nn >> 5, nl = nn & 31;
+            const int i = mm >> 5, c = mm & 31, j = TWO ? 0 : nn >> 5, nl = nn & 31;
             const int v = 4 * (nl >> 3) + (nl & 3), hh = (nl >> 2) & 1;       // accumulator slot of operand row nl
             const int d = sAcc[i][j][v][hh * 32 + c];
-            store(nt0 * 32 + nn, rt0 * 32 + mm, i, skinny_value(mc, false, kbits, sPa[i][c], sPb[j][nl], 0, d, 0));
+            const int d2 = TWO ? sAcc[i][1][v][hh * 32 + c] : 0, pb2 = TWO ? sPb[1][nl] : 0;
+            store(nt0 * 32 + nn, rt0 * 32 + mm, i, skinny_value(mc, TWO, kbits, sPa[i][c], sPb[j][nl], pb2, d, d2));
         }
     };
     const int64_t out0 = (int64_t)b * a.strideC;
@@ -729,30 +732,35 @@ __global__ __launch_bounds__(KW * 64) void gemm_skinny_splitk_quad_kernel(const 
     }
 }
 
-// Shapes the four-pieces kernel takes: one bit plane, at least two tile rows on either side, enough blocks
-// to give every compute unit one, and a K long enough for the shared expansions to outweigh the larger
-// meeting area (timed against both neighbours, weights from HBM and from a warm cache, pieces = 32 x 32
-// outputs): up to 1024 pieces from 16 K-tiles on, 2048 from 24, 3072 from 32, 6144 from 48.  Beyond that
+// Shapes the four-pieces kernel takes: at least two tile rows on either side, enough blocks to give every
+// compute unit one, and a K long enough for the shared expansions to outweigh the larger meeting area (timed
+// against both neighbours, weights from HBM and from a warm cache, pieces = 32 x 32 outputs).  One bit plane:
+// up to 1024 pieces from 16 K-tiles on, 2048 from 24, 3072 from 32, 6144 from 48.  Two planes (twice the
+// matrix-core work per piece): up to 2048 pieces from 24 K-tiles on, 3072 from 32, 4096 from 40.  Beyond that
 // the general kernel's 128- and 256-row tiles re-read less.
 static bool skinny_quad_shape(int planes, int64_t batch, int64_t MT, int64_t NT, int64_t KT)
 {
-    if (planes != 1 || MT < 2 || NT < 2 || batch * cdiv(MT, 2) * cdiv(NT, 2) < 256) return false;
-    return batch * MT * NT <= (KT >= 48 ? 6144 : KT >= 32 ? 3072 : KT >= 24 ? 2048 : KT >= 16 ? 1024 : 0);
+    if (MT < 2 || NT < 2) return false;
+    const int64_t pieces = batch * MT * NT;
+    if (planes == 2)
+        return batch * cdiv(MT, 2) * NT >= 256 && pieces <= (KT >= 40 ? 4096 : KT >= 32 ? 3072 : KT >= 24 ? 2048 : 0);
+    if (batch * cdiv(MT, 2) * cdiv(NT, 2) < 256) return false;
+    return pieces <= (KT >= 48 ? 6144 : KT >= 32 ? 3072 : KT >= 24 ? 2048 : KT >= 16 ? 1024 : 0);
 }
 
 // Shapes the skinny kernels take: one group of activation rows always (32 rows, or 16 rows of two bit planes).
 // More groups where splitting K inside the block buys more than the general kernel's 32 x 128 tiles do (timed
 // over sweeps of shapes, pieces = 32 x 32 outputs): up to 512 pieces from four K-tiles on and up to 1024 from
-// eight; two bit planes (two operands a block against one weight expansion) up to 1792 from sixteen and 2048
-// from 32.  The last bounds are set by weights that come from HBM rather than from a warm cache (a model's
-// layers): there the general kernel's serial K loop pays the full memory latency per step.  One bit plane
-// beyond 1024 pieces goes to the four-pieces kernel where that pays (see above), else to the general kernel.
+// eight; two bit planes (two operands a block against one weight expansion) up to 1792 from sixteen K-tiles on
+// (1024 from 24 on, where the four-pieces kernel takes over).  The last bounds are set by weights that come
+// from HBM rather than from a warm cache (a model's layers): there the general kernel's serial K loop pays the
+// full memory latency per step.  Beyond, the four-pieces kernel where that pays (see above), else the general one.
 bool gemm_skinny_shape(int planes, int64_t batch, int64_t M, int64_t N, int64_t K)
 {
     if (N <= (planes == 2 ? 16 : 32)) return true;
     const int64_t pieces = batch * row_tiles(M) * row_tiles(N), KT = k_tiles(K);
     if (skinny_quad_shape(planes, batch, row_tiles(M), row_tiles(N), KT)) return true;
-    if (KT >= 16 && planes == 2) return pieces <= (KT >= 32 ? 2048 : 1792);
+    if (KT >= 16 && planes == 2) return pieces <= (KT >= 24 ? 1024 : 1792);
     if (KT >= 8) return pieces <= 1024;
     return KT >= 4 && pieces <= 512;
 }
@@ -773,27 +781,35 @@ static int launch_splitk_fusex(const GemmArgs& a, hipStream_t st)
 
 static bool skinny_quad(const GemmArgs& a) { return skinny_quad_shape(a.mc.planes, a.batch, a.MT, a.NT, a.KT); }
 
-template <typename Eng>
+template <typename Eng, bool TWO>
 static int launch_splitk_quad(const GemmArgs& a, hipStream_t st)
 {
-    const int64_t gx = cdiv(a.MT, 2), gy = cdiv(a.NT, 2);
+    const int64_t gx = cdiv(a.MT, 2), gy = TWO ? a.NT : cdiv(a.NT, 2);
     if (gy > 65535 || a.batch > 65535)
         return fail(BGEMM_EINVAL, "gemm_skinny: grid of %lld x %lld x %lld blocks", (long long)gx, (long long)gy, (long long)a.batch);
-    // K ways per block: the kernel's registers allow two waves a SIMD, 2048 on the chip
-    int kw = 1;
-    while (kw < 8 && gx * gy * a.batch * kw < 2048 && kw * 2 <= a.KT) kw *= 2;
+    // K ways per block: the kernel's registers allow two waves a SIMD, 2048 on the chip at once, and the grid
+    // should come out as whole rounds of that (1536 blocks: four ways are three full rounds, two ways one and
+    // a half).  Fewest ways among the best fits; one plane at least four (two were not faster anywhere).
+    const int64_t blocks = gx * gy * a.batch;
+    int kw = 8;
+    int64_t best_w = blocks * 8, best_r = cdiv(best_w, 2048);
+    for (int c = 4; c >= (TWO ? 2 : 4); c /= 2) {
+        const int64_t w = blocks * c, r = cdiv(w, 2048);
+        if (w * best_r >= best_w * r) { kw = c; best_w = w; best_r = r; }      // w / r: waves per round
+    }
+    while (kw > 1 && kw > a.KT) kw /= 2;
     const dim3 g((unsigned)gx, (unsigned)gy, (unsigned)a.batch);
-    if (kw == 1) hipLaunchKernelGGL((gemm_skinny_splitk_quad_kernel<Eng, 1>), g, dim3(64), 0, st, a);
-    else if (kw == 2) hipLaunchKernelGGL((gemm_skinny_splitk_quad_kernel<Eng, 2>), g, dim3(128), 0, st, a);
-    else if (kw == 4) hipLaunchKernelGGL((gemm_skinny_splitk_quad_kernel<Eng, 4>), g, dim3(256), 0, st, a);
-    else hipLaunchKernelGGL((gemm_skinny_splitk_quad_kernel<Eng, 8>), g, dim3(512), 0, st, a);
+    if (kw == 1) hipLaunchKernelGGL((gemm_skinny_splitk_quad_kernel<Eng, 1, TWO>), g, dim3(64), 0, st, a);
+    else if (kw == 2) hipLaunchKernelGGL((gemm_skinny_splitk_quad_kernel<Eng, 2, TWO>), g, dim3(128), 0, st, a);
+    else if (kw == 4) hipLaunchKernelGGL((gemm_skinny_splitk_quad_kernel<Eng, 4, TWO>), g, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((gemm_skinny_splitk_quad_kernel<Eng, 8, TWO>), g, dim3(512), 0, st, a);
     return check_launch("gemm_skinny");
 }
 
 template <typename Eng>
 static int launch_splitk(const GemmArgs& a, hipStream_t st)
 {
-    if (skinny_quad(a)) return launch_splitk_quad<Eng>(a, st);
+    if (skinny_quad(a)) return a.mc.planes == 2 ? launch_splitk_quad<Eng, true>(a, st) : launch_splitk_quad<Eng, false>(a, st);
     const int64_t blocks = (int64_t)a.batch * a.MT;
     const bool pl2 = a.mc.planes == 2 && a.N > 32;      // two operands a block
     const int64_t groups = a.mc.planes == 2 && !pl2 ? cdiv(a.N, 16) : a.NT;      // 16 rows of two planes a block, else 32 rows

@@ -287,14 +287,20 @@ def test_split_k_in_block_four_pieces_a_block(oracle, batch, M, N, K):
     w = rand_f16(rng, batch * M, K).reshape(batch, M, K)
     x = rand_f16(rng, batch * N, K).reshape(batch, N, K)
     wp, xp = lk.pack_sign(to_dev(w)), lk.pack_sign(to_dev(x))
-    for mode in (MODE_XOR, MODE_AND, MODE_ATTN, MODE_ATTN_X):
+    xt = lk.pack_ternary(to_dev(x))
+    for mode in (MODE_XOR, MODE_AND, MODE_ATTN, MODE_ATTN_X, MODE_BWTA):     # ternary: the two planes of a tile row are the block's two operands
         want = np.stack([dense_ref(mode, w[b], x[b]) for b in range(batch)])
+        xo = xt if mode == MODE_BWTA else xp
         for variant in (VARIANT_AUTO, VARIANT_MFMA):
-            got = lk.bgemm_packed_forward(wp, xp, mode, torch.int32, 8, variant).cpu().numpy()
+            got = lk.bgemm_packed_forward(wp, xo, mode, torch.int32, 8, variant).cpu().numpy()
             assert (got == want).all(), (mode, variant)
-        goth = lk.bgemm_packed_forward(wp, xp, mode, torch.half, 1).cpu().numpy()
+        goth = lk.bgemm_packed_forward(wp, xo, mode, torch.half, 1).cpu().numpy()
         assert (goth.view(np.uint16) == f16_of(want).view(np.uint16)).all(), mode
     acc = np.stack([dense_ref(MODE_XOR, w[b], x[b]) for b in range(batch)])
+    acct = np.stack([dense_ref(MODE_BWTA, w[b], x[b]) for b in range(batch)]).reshape(batch * N, M)
+    swt, sat = rng.uniform(1e-4, 3e-3, M).astype(np.float32), np.asarray(0.61, dtype=np.float32)
+    gott = lk.bgemm_packed_forward(wp, xt, MODE_BWTA, scale=(to_dev(swt), to_dev(sat.reshape(1)), None)).cpu().numpy()
+    assert (_bits(gott.reshape(batch * N, M)) == _bits(oracle.np_scale_epilogue(acct, swt, sat, None))).all()
     for dtype in (np.float32, np.float16):
         sw = rng.uniform(1e-4, 3e-3, M).astype(dtype)
         sa = np.asarray(1.7371, dtype=dtype)
