@@ -735,7 +735,7 @@ __global__ __launch_bounds__(KW * 64) void gemm_skinny_splitk_quad_kernel(const 
 // Shapes the four-pieces kernel takes: at least two tile rows on either side, enough blocks to give every
 // compute unit one, and a K long enough for the shared expansions to outweigh the larger meeting area (timed
 // against both neighbours, weights from HBM and from a warm cache, pieces = 32 x 32 outputs).  One bit plane:
-// up to 1024 pieces from 16 K-tiles on, 2048 from 24, 3072 from 32, 6144 from 48.  Two planes (twice the
+// up to 1024 pieces from 16 K-tiles on, 2048 from 24, 4096 from 32, 6144 from 48.  Two planes (twice the
 // matrix-core work per piece): up to 2048 pieces from 24 K-tiles on, 3072 from 32, 4096 from 40.  Beyond that
 // the general kernel's 128- and 256-row tiles re-read less.
 static bool skinny_quad_shape(int planes, int64_t batch, int64_t MT, int64_t NT, int64_t KT)
@@ -745,7 +745,7 @@ static bool skinny_quad_shape(int planes, int64_t batch, int64_t MT, int64_t NT,
     if (planes == 2)
         return batch * cdiv(MT, 2) * NT >= 256 && pieces <= (KT >= 40 ? 4096 : KT >= 32 ? 3072 : KT >= 24 ? 2048 : 0);
     if (batch * cdiv(MT, 2) * cdiv(NT, 2) < 256) return false;
-    return pieces <= (KT >= 48 ? 6144 : KT >= 32 ? 3072 : KT >= 24 ? 2048 : KT >= 16 ? 1024 : 0);
+    return pieces <= (KT >= 48 ? 6144 : KT >= 32 ? 4096 : KT >= 24 ? 2048 : KT >= 16 ? 1024 : 0);
 }
 
 // Shapes the skinny kernels take: one group of activation rows always (32 rows, or 16 rows of two bit planes).
@@ -789,11 +789,11 @@ static int launch_splitk_quad(const GemmArgs& a, hipStream_t st)
         return fail(BGEMM_EINVAL, "gemm_skinny: grid of %lld x %lld x %lld blocks", (long long)gx, (long long)gy, (long long)a.batch);
     // K ways per block: the kernel's registers allow two waves a SIMD, 2048 on the chip at once, and the grid
     // should come out as whole rounds of that (1536 blocks: four ways are three full rounds, two ways one and
-    // a half).  Fewest ways among the best fits; one plane at least four (two were not faster anywhere).
+    // a half).  Fewest ways among the best fits.
     const int64_t blocks = gx * gy * a.batch;
     int kw = 8;
     int64_t best_w = blocks * 8, best_r = cdiv(best_w, 2048);
-    for (int c = 4; c >= (TWO ? 2 : 4); c /= 2) {
+    for (int c = 4; c >= 2; c /= 2) {
         const int64_t w = blocks * c, r = cdiv(w, 2048);
         if (w * best_r >= best_w * r) { kw = c; best_w = w; best_r = r; }      // w / r: waves per round
     }
