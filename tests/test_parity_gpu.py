@@ -278,7 +278,8 @@ def test_decode_batches_of_ternary_rows(M, N, K):
     assert torch.equal(got3[1], lk.bgemm_packed_forward(lk.PackedBits(wp.data.flip(1).contiguous(), None, 1, M, K), xt, MODE_BWTA, torch.int32)[0])
 
 
-@pytest.mark.parametrize("batch,M,N,K", [(1, 4040, 270, 6200), (4, 1000, 250, 4100), (1, 8192, 256, 8192)])
+@pytest.mark.parametrize("batch,M,N,K", [(1, 4040, 270, 6200), (4, 1000, 250, 4100), (1, 8192, 256, 8192),
+                                         (1, 4096, 1024, 8192), (1, 4096, 512, 8192)])      # the last two: two K ways, one plane / two planes
 def test_split_k_in_block_four_pieces_a_block(oracle, batch, M, N, K):
     """Outputs of one to two thousand 32 x 32 pieces over a long K: a block takes two weight row tiles and two
     activation tile rows (odd tile counts, ragged M, N and K, batches); every one-plane mode, both engines,
