@@ -13,8 +13,18 @@ OK, EINVAL, ENULL, EWORKSPACE, ELAUNCH, EALIGN = 0, -1, -2, -3, -4, -5
 MODE_AND, MODE_XOR, MODE_ATTN, MODE_BWTA, MODE_ATTN_X = 0, 1, 2, 3, 4
 OUT_I32, OUT_F16, OUT_F32_SCALED, OUT_F16_SCALED, OUT_BITS_F32, OUT_BITS_F16 = 0, 1, 2, 3, 4, 5
 SRC_F16, SRC_F32 = 0, 1
-ABI_VERSION = 6
+ABI_VERSION = 7
 VARIANT_AUTO, VARIANT_VALU, VARIANT_MFMA, VARIANT_MFMA_F4 = 0, 1, 2, 3
+# BGEMM_KERNEL_*: what bgemm_packed_kernel_id() returns and force_kernel() takes
+KERNEL_MFMA_256x256, KERNEL_MFMA_128x128, KERNEL_MFMA_64x128, KERNEL_MFMA_32x128, KERNEL_MFMA_256x128 = 0, 1, 2, 3, 4
+KERNEL_MFMA_64x64, KERNEL_MFMA_128x64 = 6, 7
+KERNEL_SKINNY_STREAM, KERNEL_SKINNY_SPLITK, KERNEL_SKINNY_QUAD, KERNEL_SKINNY_POPC, KERNEL_VALU = 16, 17, 18, 19, 32
+
+
+def force_kernel(kernel_id, family=VARIANT_AUTO):
+    """BGEMM_FORCE_KERNEL(id) | family: a `variant` that runs the named kernel whatever the shape (tests, benchmarks)."""
+    return ((kernel_id + 1) << 8) | family
+
 
 _i64, _p, _int, _sz = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
 
@@ -33,6 +43,7 @@ SIGNATURES = {
     "bgemm_packed_counter_bytes": (_sz, [_int, _i64, _i64, _i64, _i64, _int, _int]),
     "bgemm_packed_forward": (_int, [_int, _p, _p, _p, _p, _int, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
                                     _int, _int, _p, _sz, _p, _sz, _p]),
+    "bgemm_packed_kernel_id": (_int, [_int, _i64, _i64, _i64, _i64, _int, _int]),
     "bgemm_packed_forward_scaled": (_int, [_int, _p, _p, _p, _p, _int, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
                                            _int, _int, _p, _sz, _p, _sz, _p, _p, _p, _p]),
     "bgemm_packed_forward_bits": (_int, [_int, _p, _p, _p, _p, _int, _i64, _i64, _i64, _i64, _i64, _i64, _i64,

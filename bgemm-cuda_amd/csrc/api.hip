@@ -32,6 +32,23 @@ static int pick_variant(int mode, int64_t batch, int64_t M, int64_t N, int64_t K
     return BGEMM_VARIANT_MFMA_F4;
 }
 
+// `variant` = kernel family in the low byte, BGEMM_FORCE_KERNEL(id) above it.
+static bool split_variant(int variant, int* family, int* force)
+{
+    *family = variant & 0xff;
+    *force = (variant >> 8) - 1;
+    if (variant < 0 || (variant >> 16) || *family > BGEMM_VARIANT_MFMA_F4) return false;
+    if (*force < 0) return true;
+    if (*family == BGEMM_VARIANT_VALU) return false;
+    switch (*force) {
+    case BGEMM_KERNEL_MFMA_256x256: case BGEMM_KERNEL_MFMA_128x128: case BGEMM_KERNEL_MFMA_64x128:
+    case BGEMM_KERNEL_MFMA_32x128: case BGEMM_KERNEL_MFMA_256x128: case BGEMM_KERNEL_MFMA_64x64:
+    case BGEMM_KERNEL_MFMA_128x64: case BGEMM_KERNEL_SKINNY_STREAM: case BGEMM_KERNEL_SKINNY_SPLITK:
+    case BGEMM_KERNEL_SKINNY_QUAD: case BGEMM_KERNEL_SKINNY_POPC: return true;
+    default: return false;
+    }
+}
+
 static void ws_needs(int variant, int planes, int64_t batch, int64_t M, int64_t N, int64_t K, int splitK,
                      size_t* part, size_t* counters)
 {
@@ -53,7 +70,7 @@ __global__ void clear_counters_kernel(uint32_t* c, int64_t n)
 using namespace bgemm;
 
 extern "C" const char* bgemm_last_error(void) { return g_err; }
-extern "C" int bgemm_abi_version(void) { return 6; }
+extern "C" int bgemm_abi_version(void) { return 7; }
 
 static bool ws_query(int mode, int64_t batch, int64_t M, int64_t N, int64_t K, int splitK, int variant,
                      size_t* part, size_t* counters)
@@ -61,8 +78,9 @@ static bool ws_query(int mode, int64_t batch, int64_t M, int64_t N, int64_t K, i
     ModeCoef mc;
     *part = *counters = 0;
     if (!mode_coef(mode, &mc) || splitK <= 1 || batch <= 0 || M <= 0 || N <= 0 || K <= 0) return false;
-    if (variant < BGEMM_VARIANT_AUTO || variant > BGEMM_VARIANT_MFMA_F4) return false;
-    const int v = variant == BGEMM_VARIANT_AUTO ? pick_variant(mode, batch, M, N, K) : variant;
+    int family, force;
+    if (!split_variant(variant, &family, &force)) return false;
+    const int v = family == BGEMM_VARIANT_AUTO ? pick_variant(mode, batch, M, N, K) : family;
     ws_needs(v, mc.planes, batch, M, N, K, splitK, part, counters);
     return true;
 }
@@ -90,7 +108,7 @@ __global__ void fill_empty_sum_kernel(const GemmArgs a)
 {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= a.N * a.M) return;
-    store_out(a, (int64_t)blockIdx.y * a.strideC + (i / a.M) * a.M, i % a.M, 0);
+    for (int64_t b = blockIdx.y; b < a.batch; b += gridDim.y) store_out(a, b * a.strideC + (i / a.M) * a.M, i % a.M, 0);
 }
 
 // K = 0 with a bits kind: one thread per output word, the 32 columns in turn.
@@ -102,7 +120,8 @@ __global__ void fill_empty_bits_kernel(const GemmArgs a)
     unsigned w = 0;
     for (int c = 0; c < 32; c++)
         if (jw * 32 + c < a.M) w |= next_sign_bit(a, jw * 32 + c, 0) << (31 - c);
-    reinterpret_cast<uint32_t*>(a.out)[(int64_t)blockIdx.y * a.strideC + tiled_word_offset(n, jw, k_tiles(a.M))] = w;
+    for (int64_t b = blockIdx.y; b < a.batch; b += gridDim.y)
+        reinterpret_cast<uint32_t*>(a.out)[b * a.strideC + tiled_word_offset(n, jw, k_tiles(a.M))] = w;
 }
 
 // Unpacked activations for the decode kernel that packs them itself (null = X_tiled / X2_tiled are used).
@@ -114,7 +133,7 @@ static int packed_forward(int mode, const void* W_tiled, const void* X_tiled, co
                           int splitK, int variant, void* ws, size_t ws_bytes,
                           void* counters, size_t counter_bytes,
                           const void* sw, const void* sa, const void* bias, const void* zp, void* stream,
-                          const RawActivations* raw = nullptr)
+                          const RawActivations* raw = nullptr, const bool kernel_id_only = false)
 {
     g_err[0] = 0;
     GemmArgs a;
@@ -124,7 +143,8 @@ static int packed_forward(int mode, const void* W_tiled, const void* X_tiled, co
         return fail(BGEMM_EINVAL, "bgemm_packed_forward: unknown output dtype %d", out_dtype);
     const bool bits = out_dtype == BGEMM_OUT_BITS_F32 || out_dtype == BGEMM_OUT_BITS_F16;
     const bool scaled = bits || out_dtype == BGEMM_OUT_F32_SCALED || out_dtype == BGEMM_OUT_F16_SCALED;
-    if (variant < BGEMM_VARIANT_AUTO || variant > BGEMM_VARIANT_MFMA_F4)
+    int family, force;
+    if (!split_variant(variant, &family, &force))
         return fail(BGEMM_EINVAL, "bgemm_packed_forward: unknown variant %d", variant);
     if (batch < 0 || M < 0 || N < 0 || K < 0 || splitK < 1 || splitK > 65535)
         return fail(BGEMM_EINVAL, "bgemm_packed_forward: bad shape batch=%lld M=%lld N=%lld K=%lld splitK=%d",
@@ -135,7 +155,8 @@ static int packed_forward(int mode, const void* W_tiled, const void* X_tiled, co
         return fail(BGEMM_EINVAL, "bgemm_packed_forward: dimension too large");
     if (strideW < 0 || strideX < 0 || strideC < 0 || (strideW & 3) || (strideX & 3))
         return fail(BGEMM_EINVAL, "bgemm_packed_forward: operand strides must be non-negative multiples of 4 words");
-    if (batch == 0 || M == 0 || N == 0) return BGEMM_OK;
+    if (batch == 0 || M == 0 || N == 0)
+        return kernel_id_only ? fail(BGEMM_EINVAL, "bgemm_packed_kernel_id: an empty output runs no kernel") : BGEMM_OK;
     if (!out) return fail(BGEMM_ENULL, "bgemm_packed_forward: out is NULL");
     if (scaled && (!sw || !sa)) return fail(BGEMM_ENULL, "bgemm_packed_forward_scaled: sw or sa is NULL");
     if (batch > 1 && strideC < (bits ? bgemm_tiled_words(N, M) : M * N))
@@ -147,20 +168,24 @@ static int packed_forward(int mode, const void* W_tiled, const void* X_tiled, co
     a.ep_sw = sw; a.ep_sa = sa; a.ep_bias = bias; a.ep_zp = zp;
     a.M = M; a.N = N; a.K = K;
     a.strideC = strideC;
+    a.batch = (int)batch;
+    a.force = force;
     if (K == 0) {   // empty sum: every mode gives 0
-        if (batch > 65535 || cdiv(N * M, 256) > 0x7fffffffLL) return fail(BGEMM_EINVAL, "bgemm_packed_forward: output too large");
+        if (cdiv(N * M, 256) > 0x7fffffffLL) return fail(BGEMM_EINVAL, "bgemm_packed_forward: output too large");
+        const unsigned gy = (unsigned)(batch < 65535 ? batch : 65535);      // the kernels walk the rest of the batch
+        if (kernel_id_only) return fail(BGEMM_EINVAL, "bgemm_packed_kernel_id: K = 0 runs no GEMM kernel");
         if (bits)
-            hipLaunchKernelGGL(fill_empty_bits_kernel, dim3((unsigned)cdiv(N * cdiv(M, 32), 256), (unsigned)batch), dim3(256), 0,
+            hipLaunchKernelGGL(fill_empty_bits_kernel, dim3((unsigned)cdiv(N * cdiv(M, 32), 256), gy), dim3(256), 0,
                                (hipStream_t)stream, a);
         else
-            hipLaunchKernelGGL(fill_empty_sum_kernel, dim3((unsigned)cdiv(N * M, 256), (unsigned)batch), dim3(256), 0,
+            hipLaunchKernelGGL(fill_empty_sum_kernel, dim3((unsigned)cdiv(N * M, 256), gy), dim3(256), 0,
                                (hipStream_t)stream, a);
         return check_launch("bgemm_packed_forward: fill");
     }
     if (raw) {
         if (!W_tiled || !raw->src) return fail(BGEMM_ENULL, "bgemm_packed_weight_forward: operand pointer is NULL");
         if (raw->ld < K) return fail(BGEMM_EINVAL, "bgemm_packed_weight_forward: row stride %lld < K", (long long)raw->ld);
-        if (batch != 1 || !gemm_skinny_fusex_shape(a.mc.planes, M, N) || variant == BGEMM_VARIANT_VALU)
+        if (batch != 1 || !gemm_skinny_fusex_shape(a.mc.planes, M, N) || family == BGEMM_VARIANT_VALU)
             return fail(BGEMM_EINVAL, "bgemm_packed_weight_forward: shape M=%lld N=%lld not taken by the decode kernel "
                                       "(see bgemm_packed_weight_forward_supported)", (long long)M, (long long)N);
         if ((uintptr_t)raw->src & (raw->f32 ? 3 : 1))
@@ -174,13 +199,26 @@ static int packed_forward(int mode, const void* W_tiled, const void* X_tiled, co
     a.W = (const uint4*)W_tiled; a.X = (const uint4*)X_tiled; a.X2 = (const uint4*)X2_tiled;
     a.MT = (int)row_tiles(M); a.NT = (int)row_tiles(N); a.KT = (int)k_tiles(K);
     a.strideW = strideW / 4; a.strideX = strideX / 4;
-    a.batch = (int)batch; a.splitK = splitK;
+    a.splitK = splitK;
     a.vec_store = !bits && (M % 4 == 0) && (strideC % 4 == 0) && (((uintptr_t)out & 15) == 0) ? 4 : 0;
     if (a.vec_store && out_elem_shift(a.out_kind) == 1 && M % 8 == 0 && strideC % 8 == 0) a.vec_store = 8;
     a.nt_store = batch * N * M * 4 <= (32LL << 20);
-    const int v = variant == BGEMM_VARIANT_AUTO ? pick_variant(mode, batch, M, N, K) : variant;
-    if (raw) return launch_gemm_skinny(a, (hipStream_t)stream, v == BGEMM_VARIANT_MFMA_F4);
-    const bool skinny = v != BGEMM_VARIANT_VALU && gemm_skinny_shape(a.mc.planes, batch, M, N, K);
+    const int v = family == BGEMM_VARIANT_AUTO ? pick_variant(mode, batch, M, N, K) : family;
+    const bool fp4 = v == BGEMM_VARIANT_MFMA_F4;
+    if (raw) {
+        if (force >= 0 && force < BGEMM_KERNEL_SKINNY_STREAM)
+            return fail(BGEMM_EINVAL, "bgemm_packed_weight_forward: kernel %d does not pack activations", force);
+        return launch_gemm_skinny(a, (hipStream_t)stream, fp4);
+    }
+    const bool skinny = force >= 0 ? force >= BGEMM_KERNEL_SKINNY_STREAM
+                                   : v != BGEMM_VARIANT_VALU && gemm_skinny_shape(a.mc.planes, batch, M, N, K);
+    if (skinny && batch > 65535)
+        return fail(BGEMM_EINVAL, "bgemm_packed_forward: the decode kernels take batches of up to 65535");
+    if (kernel_id_only)
+        return v == BGEMM_VARIANT_VALU ? BGEMM_KERNEL_VALU
+               : force >= 0            ? force
+               : skinny                ? gemm_skinny_kernel_id(a, fp4)
+                                       : gemm_mfma_kernel_id(batch, M, N, a.KT, a.mc.planes);
     if (splitK > 1 && v == BGEMM_VARIANT_VALU) {
         size_t part, cnt;
         ws_needs(v, a.mc.planes, batch, M, N, K, splitK, &part, &cnt);
@@ -198,8 +236,18 @@ static int packed_forward(int mode, const void* W_tiled, const void* X_tiled, co
         }
     }
     if (v == BGEMM_VARIANT_VALU) return launch_gemm_valu(a, (hipStream_t)stream);
-    if (skinny) return launch_gemm_skinny(a, (hipStream_t)stream, v == BGEMM_VARIANT_MFMA_F4);
-    return launch_gemm_mfma(a, (hipStream_t)stream, v == BGEMM_VARIANT_MFMA_F4);
+    if (skinny) return launch_gemm_skinny(a, (hipStream_t)stream, fp4);
+    return launch_gemm_mfma(a, (hipStream_t)stream, fp4);
+}
+
+extern "C" int bgemm_packed_kernel_id(int mode, int64_t batch, int64_t M, int64_t N, int64_t K, int splitK, int variant)
+{
+    // the same checks and the same choice as a call, with stand-in pointers that are never dereferenced
+    // and a workspace that is never too small
+    alignas(16) static char stand_in[16];
+    return packed_forward(mode, stand_in, stand_in, stand_in, stand_in, BGEMM_OUT_I32, batch, M, N, K, 0, 0, M * N,
+                          splitK, variant, stand_in, (size_t)-1, stand_in, (size_t)-1, nullptr, nullptr, nullptr, nullptr,
+                          nullptr, nullptr, true);
 }
 
 extern "C" int bgemm_packed_forward(int mode, const void* W_tiled, const void* X_tiled, const void* X2_tiled,

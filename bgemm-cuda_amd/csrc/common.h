@@ -49,6 +49,20 @@ static inline bool mode_coef(int mode, ModeCoef* mc)
     }
 }
 
+// Rank-one terms on the device.  K, the row popcounts and the AND-dot all reach 2^24 - 1, past the SIGNED
+// 24-bit operands of __mul24 (which would read 2^23 as -2^23).  The few per-row and per-column terms use the
+// plain 32-bit multiply.  The per-element term keeps a full-rate multiply-add through the UNSIGNED 24-bit
+// one, whose operand range the dots fit; the signs of its coefficients are fixed by the number of planes
+// (one plane: cd > 0; two planes, BWTA: cd < 0 < cd2), which mode_coef's table obeys.
+__device__ __forceinline__ int dot_term(const ModeCoef& mc, const int d)
+{
+    return (int)__umul24((unsigned)mc.cd, (unsigned)d);
+}
+__device__ __forceinline__ int dot_terms2(const ModeCoef& mc, const int d, const int d2)
+{
+    return (int)__umul24((unsigned)mc.cd2, (unsigned)d2) - (int)__umul24((unsigned)-mc.cd, (unsigned)d);
+}
+
 struct GemmArgs {
     const uint4* W; const uint4* X; const uint4* X2;
     void* out; int out_kind;       // BGEMM_OUT_*
@@ -61,6 +75,7 @@ struct GemmArgs {
     int MT, NT, KT;
     int64_t strideW, strideX, strideC;   // uint4 units for W/X, elements for C
     int batch, splitK;
+    int force;            // BGEMM_KERNEL_* the caller insists on (BGEMM_FORCE_KERNEL), or -1: chosen by shape
     ModeCoef mc;
     // activations not packed yet (the decode kernel packs them itself): X/X2 are null and these describe
     // the [N][K] source; with two planes the ternary planes of sign(x) are formed
@@ -269,6 +284,8 @@ int pack_sign_pair(const void* srcA, int64_t rowsA, void* dstA, const void* srcB
 
 // Kernel families (each in its own translation unit).
 int launch_gemm_mfma(const GemmArgs& a, hipStream_t st, bool fp4);
+int gemm_mfma_kernel_id(int64_t batch, int64_t M, int64_t N, int64_t KT, int planes);     // BGEMM_KERNEL_MFMA_* by shape
+int gemm_skinny_kernel_id(const GemmArgs& a, bool fp4);                                   // BGEMM_KERNEL_SKINNY_* by shape
 int launch_gemm_valu(const GemmArgs& a, hipStream_t st);
 // Skinny shapes (few activation rows): K is split inside the block, no workspace.
 bool gemm_skinny_shape(int planes, int64_t batch, int64_t M, int64_t N, int64_t K);

@@ -198,13 +198,14 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
 #pragma unroll
         for (int i = 0; i < WN; i++) pb[p][i] += __shfl_xor(pb[p][i], 32);
 
-    // All factors stay below 2^24 (K < 2^24, small coefficients), so the full-rate 24-bit
-    // multiply is exact; v_mul_lo_u32 would cost four times as much per element.
+    // Per-element terms go through the full-rate unsigned 24-bit multiply (dot_term: the dots stay below
+    // 2^24); v_mul_lo_u32 would cost four times as much per element, and is used for the few row and
+    // column terms only.
     const ModeCoef mc = a.mc;
     const int col = lane & 31, half = lane >> 5;
     int capa[WM];
 #pragma unroll
-    for (int j = 0; j < WM; j++) capa[j] = __mul24(mc.c0, bits) + __mul24(mc.ca, pa[j]);
+    for (int j = 0; j < WM; j++) capa[j] = mc.c0 * bits + mc.ca * pa[j];
     // Row terms go through a small LDS table of the wave's own, so that a strip fetches its 16 with four
     // vector reads issued together (sixteen dependent lane permutes cost a strip two thousand cycles).
     // All LDS traffic of the epilogue is private to the wave: LDS executes one wave's accesses in
@@ -220,8 +221,8 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
     if (half == 0) {
 #pragma unroll
         for (int i = 0; i < WN; i++) {
-            int rowterm = __mul24(mc.cb, pb[0][i]);
-            if (PL == 2) rowterm += __mul24(mc.cb2, pb[PL - 1][i]);
+            int rowterm = mc.cb * pb[0][i];
+            if (PL == 2) rowterm += mc.cb2 * pb[PL - 1][i];
             rp[i * 32 + col] = rowterm;
         }
     }
@@ -237,9 +238,8 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
             const int rowterm = (v & 3) == 0 ? q.x : (v & 3) == 1 ? q.y : (v & 3) == 2 ? q.z : q.w;
 #pragma unroll
             for (int j = 0; j < WM; j++) {
-                int t = capa[j] + rowterm + __mul24(mc.cd, Eng::to_int(acc[0][i][j], v));
-                if (PL == 2) t += __mul24(mc.cd2, Eng::to_int(acc[PL - 1][i][j], v));
-                val[j][v] = t;
+                val[j][v] = capa[j] + rowterm + (PL == 2 ? dot_terms2(mc, Eng::to_int(acc[0][i][j], v), Eng::to_int(acc[PL - 1][i][j], v))
+                                                          : dot_term(mc, Eng::to_int(acc[0][i][j], v)));
             }
         }
     };
@@ -457,12 +457,12 @@ struct MfmaCfg { int id, bn, bm; };
 static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int planes)
 {
     auto blocks = [&](int bn, int bm) { return batch * cdiv(N, bn) * cdiv(M, bm); };
-    if (M <= 64) return blocks(128, 64) >= 512 ? MfmaCfg{7, 128, 64} : MfmaCfg{6, 64, 64};   // narrow outputs
-    if (planes == 1 && blocks(256, 256) >= 512 && KT >= 32) return {0, 256, 256};
-    if (planes == 1 && blocks(256, 128) >= (KT >= 64 ? 256 : 512) && (KT >= 4 || blocks(128, 128) < 512)) return {4, 256, 128};
-    if (blocks(128, 128) >= 512) return {1, 128, 128};
-    if (blocks(64, 128) >= 512) return {2, 64, 128};      // below two blocks a unit, twice as many 32-row tiles are faster
-    return {3, 32, 128};
+    if (M <= 64) return blocks(128, 64) >= 512 ? MfmaCfg{BGEMM_KERNEL_MFMA_128x64, 128, 64} : MfmaCfg{BGEMM_KERNEL_MFMA_64x64, 64, 64};   // narrow outputs
+    if (planes == 1 && blocks(256, 256) >= 512 && KT >= 32) return {BGEMM_KERNEL_MFMA_256x256, 256, 256};
+    if (planes == 1 && blocks(256, 128) >= (KT >= 64 ? 256 : 512) && (KT >= 4 || blocks(128, 128) < 512)) return {BGEMM_KERNEL_MFMA_256x128, 256, 128};
+    if (blocks(128, 128) >= 512) return {BGEMM_KERNEL_MFMA_128x128, 128, 128};
+    if (blocks(64, 128) >= 512) return {BGEMM_KERNEL_MFMA_64x128, 64, 128};      // below two blocks a unit, twice as many 32-row tiles are faster
+    return {BGEMM_KERNEL_MFMA_32x128, 32, 128};
 }
 
 template <typename Eng, int WGN, int WGM, int WN, int WM>
@@ -485,18 +485,24 @@ static int launch_cfg(const GemmArgs& a, hipStream_t st)
     return check_launch("gemm_mfma");
 }
 
+int gemm_mfma_kernel_id(int64_t batch, int64_t M, int64_t N, int64_t KT, int planes)
+{
+    return pick_cfg(batch, M, N, KT, planes).id;
+}
+
 template <typename Eng>
 static int launch_eng(const GemmArgs& a, hipStream_t st)
 {
-    const MfmaCfg cfg = pick_cfg(a.batch, a.M, a.N, a.KT, a.mc.planes);
-    switch (cfg.id) {
-    case 0: return launch_cfg<Eng, 2, 2, 4, 4>(a, st);    // 256 x 256
-    case 4: return launch_cfg<Eng, 2, 2, 4, 2>(a, st);    // 256 x 128, two blocks per CU
-    case 6: return launch_cfg<Eng, 2, 2, 1, 1>(a, st);    // 64 x 64
-    case 7: return launch_cfg<Eng, 2, 2, 2, 1>(a, st);    // 128 x 64
-    case 1: return launch_cfg<Eng, 2, 2, 2, 2>(a, st);    // 128 x 128
-    case 2: return launch_cfg<Eng, 1, 4, 2, 1>(a, st);    // 64 x 128
-    default: return launch_cfg<Eng, 1, 4, 1, 1>(a, st);   // 32 x 128
+    const int id = a.force >= 0 ? a.force : pick_cfg(a.batch, a.M, a.N, a.KT, a.mc.planes).id;
+    switch (id) {
+    case BGEMM_KERNEL_MFMA_256x256: return launch_cfg<Eng, 2, 2, 4, 4>(a, st);
+    case BGEMM_KERNEL_MFMA_256x128: return launch_cfg<Eng, 2, 2, 4, 2>(a, st);    // two blocks per CU
+    case BGEMM_KERNEL_MFMA_64x64: return launch_cfg<Eng, 2, 2, 1, 1>(a, st);
+    case BGEMM_KERNEL_MFMA_128x64: return launch_cfg<Eng, 2, 2, 2, 1>(a, st);
+    case BGEMM_KERNEL_MFMA_128x128: return launch_cfg<Eng, 2, 2, 2, 2>(a, st);
+    case BGEMM_KERNEL_MFMA_64x128: return launch_cfg<Eng, 1, 4, 2, 1>(a, st);
+    case BGEMM_KERNEL_MFMA_32x128: return launch_cfg<Eng, 1, 4, 1, 1>(a, st);
+    default: return fail(BGEMM_EINVAL, "gemm_mfma: no kernel %d", id);
     }
 }
 

@@ -46,9 +46,8 @@ __device__ __forceinline__ const uint4* skinny_x_ptr(const GemmArgs& a, const in
 __device__ __forceinline__ int skinny_value(const ModeCoef& mc, const bool two, const int kbits, const int pa,
                                             const int pb, const int pb2, const int d, const int d2)
 {
-    int val = __mul24(mc.c0, kbits) + __mul24(mc.ca, pa) + __mul24(mc.cb, pb) + __mul24(mc.cd, d);
-    if (two) val += __mul24(mc.cb2, pb2) + __mul24(mc.cd2, d2);
-    return val;
+    const int val = mc.c0 * kbits + mc.ca * pa + mc.cb * pb;
+    return two ? val + mc.cb2 * pb2 + dot_terms2(mc, d, d2) : val + dot_term(mc, d);
 }
 
 // ---- streaming kernel --------------------------------------------------------------------------
@@ -130,25 +129,24 @@ __global__ __launch_bounds__(256) void gemm_skinny_stream_kernel(const GemmArgs 
     bool col_ok[RT];
 #pragma unroll
     for (int t = 0; t < RT; t++) {
-        colterm[t] = __mul24(mc.c0, (int)a.K) + __mul24(mc.ca, pa[t]);
+        colterm[t] = mc.c0 * (int)a.K + mc.ca * pa[t];
         col_ok[t] = ((int64_t)grp * RT + t) * 32 + r < a.M;
     }
     const int64_t m0 = (int64_t)grp * RT * 32 + r;                        // column of tile 0
     const int64_t out_row0 = (int64_t)b * a.strideC;
     auto row_of = [&](const int v) { return 8 * (v >> 2) + 4 * h + (v & 3); };
     auto value = [&](const int v, const int t, const int rowterm) {
-        int val = colterm[t] + rowterm + __mul24(mc.cd, Eng::to_int(acc[t], v));
-        if (two) val += __mul24(mc.cd2, Eng::to_int(acc[t], (v + 8) & 15));
-        return val;
+        const int base = colterm[t] + rowterm;
+        return two ? base + dot_terms2(mc, Eng::to_int(acc[t], v), Eng::to_int(acc[t], (v + 8) & 15)) : base + dot_term(mc, Eng::to_int(acc[t], v));
     };
     // row terms: the popcounts sit in lanes 0..31; both candidates (lane half 0 / 1) are read as
     // scalars and selected, which costs no LDS round trip
     auto row_term = [&](const int v) {
         const int n0 = 8 * (v >> 2) + (v & 3), n1 = n0 + 4;
-        int t0 = __mul24(mc.cb, __builtin_amdgcn_readlane(pb, n0)), t1 = __mul24(mc.cb, __builtin_amdgcn_readlane(pb, n1));
+        int t0 = mc.cb * __builtin_amdgcn_readlane(pb, n0), t1 = mc.cb * __builtin_amdgcn_readlane(pb, n1);
         if (two) {
-            t0 += __mul24(mc.cb2, __builtin_amdgcn_readlane(pb, (n0 + 16) & 31));
-            t1 += __mul24(mc.cb2, __builtin_amdgcn_readlane(pb, (n1 + 16) & 31));
+            t0 += mc.cb2 * __builtin_amdgcn_readlane(pb, (n0 + 16) & 31);
+            t1 += mc.cb2 * __builtin_amdgcn_readlane(pb, (n1 + 16) & 31);
         }
         return h ? t1 : t0;
     };
@@ -757,6 +755,7 @@ static bool skinny_quad_shape(int planes, int64_t batch, int64_t MT, int64_t NT,
 // full memory latency per step.  Beyond, the four-pieces kernel where that pays (see above), else the general one.
 bool gemm_skinny_shape(int planes, int64_t batch, int64_t M, int64_t N, int64_t K)
 {
+    if (batch > 65535) return false;             // these kernels walk the batch in the grid's third dimension
     if (N <= (planes == 2 ? 16 : 32)) return true;
     const int64_t pieces = batch * row_tiles(M) * row_tiles(N), KT = k_tiles(K);
     if (skinny_quad_shape(planes, batch, row_tiles(M), row_tiles(N), KT)) return true;
@@ -809,7 +808,6 @@ static int launch_splitk_quad(const GemmArgs& a, hipStream_t st)
 template <typename Eng>
 static int launch_splitk(const GemmArgs& a, hipStream_t st)
 {
-    if (skinny_quad(a)) return a.mc.planes == 2 ? launch_splitk_quad<Eng, true>(a, st) : launch_splitk_quad<Eng, false>(a, st);
     const int64_t blocks = (int64_t)a.batch * a.MT;
     const bool pl2 = a.mc.planes == 2 && a.N > 32;      // two operands a block
     const int64_t groups = a.mc.planes == 2 && !pl2 ? cdiv(a.N, 16) : a.NT;      // 16 rows of two planes a block, else 32 rows
@@ -882,24 +880,44 @@ bool gemm_skinny_fusex_shape(int planes, int64_t M, int64_t N)
     return N >= 1 && N <= 4 && row_tiles(M) < 4096;
 }
 
-int launch_gemm_skinny(const GemmArgs& a, hipStream_t st, bool fp4)
+// Which of the kernels above a shape gets (BGEMM_KERNEL_* ids).
+int gemm_skinny_kernel_id(const GemmArgs& a, bool fp4)
 {
     // a few vectors: the vector ALU does it with less work than the expansion costs (the int8-engine variant
     // keeps the matrix-core kernels for every row count)
-    int rc;
-    const int64_t row_tiles = (int64_t)a.batch * a.MT;
-    if (a.xsrc) {
-        if (fp4 && launch_popc_for<true>(a, st, &rc)) return rc;
-        return fp4 ? launch_splitk_fusex<EngF4>(a, st) : launch_splitk_fusex<EngI8>(a, st);
-    }
-    if (fp4 && row_tiles < 4096 && launch_popc_for<false>(a, st, &rc)) return rc;
+    const int64_t row_tiles = (int64_t)a.batch * a.MT, nvec = a.N * a.mc.planes;
+    if (a.xsrc) return fp4 && nvec <= 2 ? BGEMM_KERNEL_SKINNY_POPC : BGEMM_KERNEL_SKINNY_SPLITK;
+    if (fp4 && row_tiles < 4096 && nvec <= 2) return BGEMM_KERNEL_SKINNY_POPC;
     // Enough row tiles for about four waves on every SIMD: no K split needed (the result does not
-    // depend on it).  Two row tiles per wave share one expansion of the activation tiles.
-    if (a.mc.planes == 2 ? a.N <= 16 : a.NT <= 1) {
-        if (row_tiles >= 8192) return fp4 ? launch_stream<EngF4, 2>(a, st) : launch_stream<EngI8, 2>(a, st);
-        if (row_tiles >= 4096) return fp4 ? launch_stream<EngF4, 1>(a, st) : launch_stream<EngI8, 1>(a, st);
+    // depend on it).
+    if ((a.mc.planes == 2 ? a.N <= 16 : a.NT <= 1) && row_tiles >= 4096) return BGEMM_KERNEL_SKINNY_STREAM;
+    return skinny_quad(a) ? BGEMM_KERNEL_SKINNY_QUAD : BGEMM_KERNEL_SKINNY_SPLITK;
+}
+
+int launch_gemm_skinny(const GemmArgs& a, hipStream_t st, bool fp4)
+{
+    int rc;
+    const int id = a.force >= 0 ? a.force : gemm_skinny_kernel_id(a, fp4);
+    switch (id) {
+    case BGEMM_KERNEL_SKINNY_POPC:
+        if (a.xsrc ? launch_popc_for<true>(a, st, &rc) : launch_popc_for<false>(a, st, &rc)) return rc;
+        return fail(BGEMM_EINVAL, "gemm_skinny: the vector-ALU decode kernel takes one or two vectors");
+    case BGEMM_KERNEL_SKINNY_STREAM:
+        if (a.xsrc || !(a.mc.planes == 2 ? a.N <= 16 : a.NT <= 1))
+            return fail(BGEMM_EINVAL, "gemm_skinny: the streaming kernel takes one group of packed activation rows");
+        // two row tiles per wave share one expansion of the activation tiles
+        if ((int64_t)a.batch * a.MT >= 8192) return fp4 ? launch_stream<EngF4, 2>(a, st) : launch_stream<EngI8, 2>(a, st);
+        return fp4 ? launch_stream<EngF4, 1>(a, st) : launch_stream<EngI8, 1>(a, st);
+    case BGEMM_KERNEL_SKINNY_QUAD:
+        if (a.xsrc) return fail(BGEMM_EINVAL, "gemm_skinny: the four-pieces kernel takes packed activations");
+        if (a.mc.planes == 2) return fp4 ? launch_splitk_quad<EngF4, true>(a, st) : launch_splitk_quad<EngI8, true>(a, st);
+        return fp4 ? launch_splitk_quad<EngF4, false>(a, st) : launch_splitk_quad<EngI8, false>(a, st);
+    case BGEMM_KERNEL_SKINNY_SPLITK:
+        if (a.xsrc) return fp4 ? launch_splitk_fusex<EngF4>(a, st) : launch_splitk_fusex<EngI8>(a, st);
+        return fp4 ? launch_splitk<EngF4>(a, st) : launch_splitk<EngI8>(a, st);
+    default:
+        return fail(BGEMM_EINVAL, "gemm_skinny: no kernel %d", id);
     }
-    return fp4 ? launch_splitk<EngF4>(a, st) : launch_splitk<EngI8>(a, st);
 }
 
 }  // namespace bgemm

@@ -24,7 +24,7 @@ AND_POP, XOR_POP, ATTN_MM = 0, 1, 2   # lowbit_kernel/csrc/include/configs.h:70-
 
 __all__ = ["bgemm_linear_forward_cuda", "binary_weight_prepacking", "pack_sign", "pack_ternary",
            "pack_sign_transposed", "bgemm_packed_forward", "bgemm_packed_weight_forward", "PackedBits", "zeros_packed", "save_packed", "load_packed",
-           "set_weight_cache", "AND_POP", "XOR_POP", "ATTN_MM"]
+           "set_weight_cache", "packed_kernel_id", "AND_POP", "XOR_POP", "ATTN_MM"]
 
 
 _NULL_CTX = contextlib.nullcontext()
@@ -108,6 +108,26 @@ class PackedBits:
 
     def nbytes(self):
         return self.data.numel() * 4 * (2 if self.ternary else 1)
+
+
+def _check_packed(p, name):
+    """A PackedBits is a public constructor: its buffers must be what the kernels will index."""
+    words = _b.lib().bgemm_tiled_words(p.rows, p.K)
+    for plane in ((p.data, p.data2) if p.ternary else (p.data,)):
+        _need_cuda(plane, name)
+        if plane.dtype != torch.int32 or tuple(plane.shape) != (p.batch, words) or not plane.is_contiguous():
+            raise ValueError("%s: every plane must be a contiguous int32 tensor of shape (%d, %d) for %d rows x %d bits, "
+                             "got %s %s" % (name, p.batch, words, p.rows, p.K, plane.dtype, tuple(plane.shape)))
+        if plane.device != p.data.device:
+            raise ValueError("%s: both planes must live on one device" % name)
+
+
+def packed_kernel_id(w, x, mode=MODE_XOR, splitK=1, variant=VARIANT_AUTO):
+    """The kernel (``_lib.KERNEL_*``) that ``bgemm_packed_forward(w, x, mode, ..., splitK, variant)`` runs."""
+    rc = _b.lib().bgemm_packed_kernel_id(mode, max(w.batch, x.batch), w.rows, x.rows, w.K, splitK, variant)
+    if rc < 0:
+        _b.check(rc)
+    return rc
 
 
 def zeros_packed(rows, K, batch=1, device="cuda"):
@@ -254,6 +274,8 @@ def bgemm_packed_forward(w, x, mode=MODE_XOR, out_dtype=torch.int32, splitK=1, v
         raise ValueError("batch mismatch: %d vs %d" % (w.batch, x.batch))
     M, N, K = w.rows, x.rows, w.K
     dev = w.data.device
+    _check_packed(w, "w")
+    _check_packed(x, "x")
     if scale is not None:
         sw, sa, bias = scale
         out_dtype = sw.dtype
@@ -269,6 +291,7 @@ def bgemm_packed_forward(w, x, mode=MODE_XOR, out_dtype=torch.int32, splitK=1, v
         if bits_out is not None:
             if bits_out.ternary or bits_out.rows != N or bits_out.K != M or bits_out.batch != batch:
                 raise ValueError("bits_out must be a binary PackedBits of %d x %d rows x bits, batch %d" % (N, M, batch))
+            _check_packed(bits_out, "bits_out")
             if next_zero_point is not None:
                 _need_cuda(next_zero_point, "next_zero_point")
                 if next_zero_point.dtype != out_dtype or next_zero_point.numel() != 1:
@@ -282,6 +305,12 @@ def bgemm_packed_forward(w, x, mode=MODE_XOR, out_dtype=torch.int32, splitK=1, v
         kind = OUT_F16 if out_dtype == torch.half else OUT_I32
     if out is None and bits_out is None:
         out = torch.empty((batch, N, M), dtype=out_dtype, device=dev)
+    elif bits_out is None:
+        # the kernel writes batch * N * M elements from out's first byte on
+        _need_cuda(out, "out")
+        if out.device != dev or out.dtype != out_dtype or not out.is_contiguous() or out.numel() != batch * N * M:
+            raise ValueError("out must be a contiguous %s tensor of %d x %d x %d elements on %s"
+                             % (out_dtype, batch, N, M, dev))
     L = _b.lib()
     with _on(dev):
         ws = cnt = None

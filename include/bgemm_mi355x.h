@@ -50,6 +50,20 @@ enum { BGEMM_SRC_F16 = 0, BGEMM_SRC_F32 = 1 };
  * (products are 0/1 and the fp32 accumulator stays below 2^24, so it is exact too). */
 enum { BGEMM_VARIANT_AUTO = 0, BGEMM_VARIANT_VALU = 1, BGEMM_VARIANT_MFMA = 2, BGEMM_VARIANT_MFMA_F4 = 3 };
 
+/* The kernels behind bgemm_packed_forward*, as bgemm_packed_kernel_id() names them: the general matrix-core
+ * kernel by its block tile (activation rows x weight rows), the decode-shaped kernels, the VALU kernel. */
+enum { BGEMM_KERNEL_MFMA_256x256 = 0, BGEMM_KERNEL_MFMA_128x128 = 1, BGEMM_KERNEL_MFMA_64x128 = 2,
+       BGEMM_KERNEL_MFMA_32x128 = 3, BGEMM_KERNEL_MFMA_256x128 = 4, BGEMM_KERNEL_MFMA_64x64 = 6,
+       BGEMM_KERNEL_MFMA_128x64 = 7,
+       BGEMM_KERNEL_SKINNY_STREAM = 16, BGEMM_KERNEL_SKINNY_SPLITK = 17, BGEMM_KERNEL_SKINNY_QUAD = 18,
+       BGEMM_KERNEL_SKINNY_POPC = 19,
+       BGEMM_KERNEL_VALU = 32 };
+/* Test and benchmark aid, OR-ed into a `variant` argument whose family is one of the matrix-core ones (or AUTO):
+ * the call runs kernel `id` instead of the one chosen by shape, or returns BGEMM_EINVAL where that kernel
+ * cannot take the shape (two bit planes on a tile built for one; the decode kernels beyond their row counts).
+ * Results never depend on it. */
+#define BGEMM_FORCE_KERNEL(id) (((id) + 1) << 8)
+
 enum {
     BGEMM_OK = 0,
     BGEMM_EINVAL = -1,      /* bad shape, mode, dtype, variant or splitK            */
@@ -158,6 +172,11 @@ int bgemm_packed_forward(int mode, const void* W_tiled, const void* X_tiled, con
                          int64_t strideW, int64_t strideX, int64_t strideC,
                          int splitK, int variant, void* ws, size_t ws_bytes,
                          void* counters, size_t counter_bytes, void* stream);
+/* The kernel (BGEMM_KERNEL_*) the three bgemm_packed_forward* entry points run for these arguments, or a
+ * negative BGEMM_E* code for arguments they would reject.  The reference's dispatch is the N-bucket switch
+ * of bin_pack_linear_kernel (fp6_linear.cu:292-330), which lands on one tile for every shape; here the
+ * choice depends on the shape, and tests and benchmarks ask which kernel they are looking at. */
+int bgemm_packed_kernel_id(int mode, int64_t batch, int64_t M, int64_t N, int64_t K, int splitK, int variant);
 
 /* The same GEMM with the binary Linear's output scaling fused into the store, replacing the
  * separate elementwise kernels of `bgemm(...) * sw * sa (+ bias)`

@@ -29,7 +29,7 @@ def test_header_symbols_exported():
 
 def test_layout_sizes():
     L = _lib.lib()
-    assert L.bgemm_abi_version() == _lib.ABI_VERSION == 6
+    assert L.bgemm_abi_version() == _lib.ABI_VERSION == 7
     assert L.bgemm_tiled_words(1, 1) == 256
     assert L.bgemm_tiled_words(32, 256) == 256
     assert L.bgemm_tiled_words(33, 257) == 4 * 256
@@ -56,6 +56,9 @@ def test_layout_sizes():
     (dict(mode=7), _lib.EINVAL),
     (dict(out_dtype=5), _lib.EINVAL),
     (dict(variant=4), _lib.EINVAL),
+    (dict(variant=_lib.force_kernel(5)), _lib.EINVAL),                                   # no such kernel
+    (dict(variant=_lib.force_kernel(_lib.KERNEL_MFMA_64x64, _lib.VARIANT_VALU)), _lib.EINVAL),   # the VALU design has one kernel
+    (dict(variant=_lib.force_kernel(_lib.KERNEL_SKINNY_STREAM), batch=70000, strideC=64 * 256), _lib.EINVAL),
     (dict(M=-1), _lib.EINVAL),
     (dict(splitK=0), _lib.EINVAL),
     (dict(K=1 << 24), _lib.EINVAL),
@@ -86,6 +89,32 @@ def test_packed_forward_rejects(kwargs, code):
     assert L.bgemm_last_error()            # a message was recorded
     with pytest.raises(ValueError):
         _lib.check(rc)
+
+
+def test_dispatch_of_the_benchmark_configurations():
+    """Which kernel each benchmark configuration runs (what the profiles and the bench lines are about):
+    the query is host code and needs no GPU."""
+    B = _lib
+    kid = B.lib().bgemm_packed_kernel_id
+    MODE_XOR, MODE_BWTA, MODE_ATTN_X, VARIANT_AUTO, VARIANT_VALU, force_kernel = (
+        B.MODE_XOR, B.MODE_BWTA, B.MODE_ATTN_X, B.VARIANT_AUTO, B.VARIANT_VALU, B.force_kernel)
+    TILES = (0, 1, 2, 3, 4, 6, 7)
+    A = VARIANT_AUTO
+    assert kid(MODE_XOR, 1, 8192, 8192, 8192, 1, A) == B.KERNEL_MFMA_256x256
+    assert kid(MODE_XOR, 1, 8192, 2048, 4096, 1, A) == B.KERNEL_MFMA_256x128
+    assert kid(MODE_XOR, 1, 8192, 2048, 16384, 4, A) == B.KERNEL_MFMA_256x128
+    assert kid(MODE_XOR, 1, 8192, 256, 16384, 1, A) == B.KERNEL_SKINNY_QUAD
+    assert kid(MODE_ATTN_X, 192, 64, 512, 512, 1, A) == B.KERNEL_MFMA_128x64
+    assert kid(MODE_ATTN_X, 24, 64, 512, 512, 1, A) == B.KERNEL_MFMA_64x64
+    assert kid(MODE_BWTA, 1, 11008, 1, 4096, 8, A) == B.KERNEL_SKINNY_POPC
+    assert kid(MODE_BWTA, 1, 11008, 16, 4096, 8, A) == B.KERNEL_SKINNY_SPLITK
+    assert kid(MODE_BWTA, 64, 11008, 16, 4096, 1, A) == B.KERNEL_SKINNY_STREAM
+    assert kid(MODE_XOR, 1, 4096, 128, 4096, 1, VARIANT_VALU) == B.KERNEL_VALU
+    assert kid(MODE_XOR, 70000, 40, 8, 300, 1, A) in TILES        # a batch beyond the decode kernels' grid
+    assert kid(MODE_XOR, 1, 64, 64, 64, 1, force_kernel(B.KERNEL_MFMA_256x256)) == B.KERNEL_MFMA_256x256
+    assert kid(MODE_XOR, 1, 64, 64, 64, 1, force_kernel(5)) == B.EINVAL    # no such kernel
+    assert kid(MODE_XOR, 1, 64, 64, 64, 1, force_kernel(B.KERNEL_MFMA_64x64, VARIANT_VALU)) == B.EINVAL
+    assert kid(9, 1, 64, 64, 64, 1, A) == B.EINVAL and kid(MODE_XOR, 1, 64, 0, 64, 1, A) == B.EINVAL
 
 
 def test_decode_entry_states_its_shapes_and_rejects_others():
@@ -206,3 +235,26 @@ def test_packed_file_format_round_trip_and_rejects(tmp_path):
     open(path, "wb").write(raw[:-4])          # truncated payload
     with pytest.raises(ValueError):
         lk.load_packed(path, device="cpu")
+
+
+def test_shim_checks_buffers_before_the_kernel_sees_them(monkeypatch):
+    """A wrong output tensor or a hand-built PackedBits is a ValueError, not an out-of-bounds access on the GPU."""
+    import torch
+    import lowbit_kernel as lk
+    monkeypatch.setattr(lk, "_need_cuda", lambda t, name: None)       # the checks themselves are host code
+    words = _lib.lib().bgemm_tiled_words(40, 300)
+    good = lambda rows: lk.PackedBits(torch.zeros((1, _lib.lib().bgemm_tiled_words(rows, 300)), dtype=torch.int32), None, 1, rows, 300)
+    w, x = good(40), good(7)
+    for bad_out in (torch.zeros((1, 7, 39), dtype=torch.int32),                 # too small
+                    torch.zeros((1, 7, 40), dtype=torch.int16),                 # wrong element type
+                    torch.zeros((1, 40, 7), dtype=torch.int32).transpose(1, 2)):    # not contiguous
+        with pytest.raises(ValueError):
+            lk.bgemm_packed_forward(w, x, out=bad_out)
+    for bad in (lk.PackedBits(torch.zeros((1, words - 256), dtype=torch.int32), None, 1, 40, 300),     # a tile short
+                lk.PackedBits(torch.zeros((1, words), dtype=torch.int64), None, 1, 40, 300),
+                lk.PackedBits(torch.zeros((2, words), dtype=torch.int32), None, 1, 40, 300),
+                lk.PackedBits(torch.zeros((1, 2 * words), dtype=torch.int32)[:, ::2], None, 1, 40, 300)):
+        with pytest.raises(ValueError):
+            lk.bgemm_packed_forward(bad, x)
+    with pytest.raises(ValueError):
+        lk.bgemm_packed_forward(w, lk.PackedBits(x.data, torch.zeros((1, 256), dtype=torch.int32), 1, 7, 300), _lib.MODE_BWTA)

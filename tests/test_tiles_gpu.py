@@ -1,0 +1,273 @@
+"""Parity of every kernel behind bgemm_packed_forward*, kernel by kernel.
+
+The library picks a kernel per shape, so a test only covers the kernel its shape lands on.  Here every
+case either asserts the kernel the library reports for the call (``packed_kernel_id``) or insists on one
+(``force_kernel``), so that each tile of the general matrix-core kernel, and each decode-shaped kernel, runs
+ragged M / N / K, odd K-tile counts and every output kind against the dense closed forms on de-binarised
+operands (the reference drivers' own method, csrc/benchmark.cu:146-204), the epilogue and prologue models of
+the oracle, bit for bit.  Output order and fp16 rounding follow kernel_matmul.cuh:529-546.
+"""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+import lowbit_kernel as lk
+import _lib as B
+from _lib import (MODE_AND, MODE_XOR, MODE_ATTN, MODE_BWTA, MODE_ATTN_X, VARIANT_AUTO, VARIANT_VALU, VARIANT_MFMA,
+                  VARIANT_MFMA_F4, force_kernel)
+
+DEV = "cuda:0"
+TILES = {"256x256": B.KERNEL_MFMA_256x256, "256x128": B.KERNEL_MFMA_256x128, "128x128": B.KERNEL_MFMA_128x128,
+         "64x128": B.KERNEL_MFMA_64x128, "32x128": B.KERNEL_MFMA_32x128, "128x64": B.KERNEL_MFMA_128x64,
+         "64x64": B.KERNEL_MFMA_64x64}
+ENGINES = {"fp4": VARIANT_MFMA_F4, "int8": VARIANT_MFMA}
+
+
+def to_dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+def pm1(rng, *shape):
+    """+-1 fp16 with both zeros mixed in: -0.0 counts as negative, +0.0 as positive."""
+    bits = rng.integers(0, 2, shape, dtype=np.int8)
+    v = np.where(bits == 1, np.float16(-1), np.float16(1)).astype(np.float16)
+    z = rng.random(shape) < 0.01
+    return np.where(z, np.where(bits == 1, np.float16(-0.0), np.float16(0.0)), v).astype(np.float16)
+
+
+def sgn(a):
+    return 1.0 - 2.0 * (a.view(np.uint16) >> 15).astype(np.float32)
+
+
+def dense(mode, w, x):
+    """fp32 closed forms (exact below 2^24) on operands de-binarised by sign bit; x [.., N, K], w [.., M, K]."""
+    a, b = (1 - sgn(w)) / 2, (1 - sgn(x)) / 2
+    wt = np.swapaxes
+    if mode == MODE_XOR:
+        r = sgn(x) @ wt(sgn(w), -1, -2)
+    elif mode == MODE_AND:
+        r = b @ wt(a, -1, -2)
+    elif mode == MODE_ATTN:
+        r = sgn(x) @ wt(1 - a, -1, -2)
+    elif mode == MODE_ATTN_X:
+        r = (1 - b) @ wt(sgn(w), -1, -2)
+    else:
+        xs = x.view(np.uint16)
+        t = np.where((xs & 0x7FFF) == 0, 0.0, sgn(x)).astype(np.float32)
+        r = t @ wt(sgn(w), -1, -2)
+    return r.astype(np.int32)
+
+
+def f16_of(i32):
+    with np.errstate(over="ignore"):
+        return i32.astype(np.float32).astype(np.float16)
+
+
+def bits_of(a):
+    return a.view(np.uint16 if a.dtype == np.float16 else np.uint32)
+
+
+def check_all_kinds(oracle, wp, xp, acc, M, N, variant, rng, rows=None, cols=None):
+    """Every output kind of one GEMM against `acc` (the exact int32 result, or its [rows][:, cols] sample)."""
+    def sample(t):
+        t = t[0]
+        if rows is not None:
+            t = t[torch.from_numpy(rows).to(DEV)][:, torch.from_numpy(cols).to(DEV)]
+        return t.cpu().numpy()
+
+    got = sample(lk.bgemm_packed_forward(wp, xp, MODE_XOR, torch.int32, 1, variant))
+    assert (got == acc).all(), "int32"
+    got = sample(lk.bgemm_packed_forward(wp, xp, MODE_XOR, torch.half, 1, variant))
+    assert (bits_of(got) == bits_of(f16_of(acc))).all(), "fp16"
+    for dtype in (np.float32, np.float16):
+        sw = rng.uniform(1e-4, 3e-3, M).astype(dtype)
+        sa = np.asarray(1.7371, dtype=dtype)
+        bias = (0.05 * rng.standard_normal(M)).astype(dtype)
+        swc, bc = (sw, bias) if cols is None else (sw[cols], bias[cols])
+        for with_bias in (True, False):
+            want = oracle.np_scale_epilogue(acc, swc, sa, bc if with_bias else None)
+            got = sample(lk.bgemm_packed_forward(wp, xp, MODE_XOR, variant=variant,
+                                                 scale=(to_dev(sw), to_dev(sa.reshape(1)), to_dev(bias) if with_bias else None)))
+            assert got.dtype == want.dtype and (bits_of(got) == bits_of(want)).all(), ("scaled", dtype, with_bias)
+        # bits kinds: the next layer's operand, the zero point at a value that splits the outputs
+        zp = np.asarray(0.011, dtype=dtype)
+        out = lk.zeros_packed(N, M, 1, DEV)
+        lk.bgemm_packed_forward(wp, xp, MODE_XOR, variant=variant, bits_out=out,
+                                scale=(to_dev(sw), to_dev(sa.reshape(1)), to_dev(bias)), next_zero_point=to_dev(zp.reshape(1)))
+        logical = lk.logical_from_tiled(out).cpu().numpy().view(np.uint32)               # [N][ceil(M/32)]
+        y = oracle.np_scale_epilogue(acc, swc, sa, bc)
+        want_bits = oracle.np_center_to_f16(y, zp).view(np.uint16) >> 15                  # 1 = negative
+        got_bits = np.unpackbits(logical.byteswap().view(np.uint8), axis=1)[:, :M]        # MSB-first words
+        if rows is not None:
+            got_bits = got_bits[rows][:, cols]
+        assert (got_bits == want_bits).all(), ("bits", dtype)
+        assert 0.2 < want_bits.mean() < 0.8                                               # the zero point does split them
+        # nothing but real bits was written
+        assert int(np.unpackbits(out.data.cpu().numpy().view(np.uint8)).sum()) == int(np.unpackbits(logical.view(np.uint8)).sum())
+
+
+# M picks the store path of the general kernel: 520 = 16-byte stores of eight halves / four ints, 516 = four elements a lane,
+# 517 = one element a lane; N = 515 leaves a ragged last strip; K = 1275 is five K-tiles (odd: the pipelined
+# loops run a zero tile to fill their last pair), the last one ragged
+@pytest.mark.parametrize("M", [520, 516, 517])
+@pytest.mark.parametrize("engine", list(ENGINES))
+@pytest.mark.parametrize("tile", list(TILES))
+def test_each_tile_every_output_kind(oracle, tile, engine, M):
+    N, K = 515, 1275
+    rng = np.random.default_rng(M * 31 + TILES[tile])
+    w, x = pm1(rng, M, K), pm1(rng, N, K)
+    wp, xp = lk.pack_sign(to_dev(w)), lk.pack_sign(to_dev(x))
+    variant = force_kernel(TILES[tile], ENGINES[engine])
+    assert lk.packed_kernel_id(wp, xp, MODE_XOR, 1, variant) == TILES[tile]
+    check_all_kinds(oracle, wp, xp, dense(MODE_XOR, w, x), M, N, variant, rng)
+
+
+@pytest.mark.parametrize("engine", list(ENGINES))
+@pytest.mark.parametrize("tile", list(TILES))
+def test_each_tile_every_mode_batched(tile, engine):
+    """All five modes on a batch of ragged matrices, one K-tile and an even number of them; tiles built for one bit
+    plane refuse the ternary operand."""
+    rng = np.random.default_rng(TILES[tile])
+    variant = force_kernel(TILES[tile], ENGINES[engine])
+    for Bn, M, N, K in ((3, 70, 300, 200), (2, 300, 70, 1000)):
+        w, x = pm1(rng, Bn, M, K), pm1(rng, Bn, N, K)
+        x[rng.random(x.shape) < 0.3] = 0                          # ternary zeros (+0.0: positive for the sign modes)
+        wp, xp, xt = lk.pack_sign(to_dev(w)), lk.pack_sign(to_dev(x)), lk.pack_ternary(to_dev(x))
+        for mode in (MODE_AND, MODE_XOR, MODE_ATTN, MODE_ATTN_X):
+            got = lk.bgemm_packed_forward(wp, xp, mode, torch.int32, 2, variant).cpu().numpy()
+            assert (got == dense(mode, w, x)).all(), mode
+        if tile in ("256x256", "256x128"):
+            with pytest.raises(ValueError):
+                lk.bgemm_packed_forward(wp, xt, MODE_BWTA, torch.int32, 1, variant)
+        else:
+            got = lk.bgemm_packed_forward(wp, xt, MODE_BWTA, torch.half, 1, variant).cpu().numpy()
+            assert (bits_of(got) == bits_of(f16_of(dense(MODE_BWTA, w, x)))).all()
+
+
+@pytest.mark.parametrize("engine", list(ENGINES))
+@pytest.mark.parametrize("M,N,K,want_kernel", [
+    (5907, 5903, 33 * 256 - 5, B.KERNEL_MFMA_256x256),       # the 8192^3 kernel: ragged edges, 33 K-tiles
+    (8195, 2053, 17 * 256 - 7, B.KERNEL_MFMA_256x128),       # the 8192 x 2048 x 4096 kernel likewise
+])
+def test_headline_tiles_where_the_library_picks_them(oracle, engine, M, N, K, want_kernel):
+    """No forcing: shapes that the library itself sends to the two large tiles, ragged in M, N and K with an odd
+    K-tile count, every output kind, on sampled rows and columns (the edges included)."""
+    rng = np.random.default_rng(M + N)
+    g = torch.Generator(device=DEV).manual_seed(M * 7 + N)
+    w16 = (1 - 2 * torch.randint(0, 2, (M, K), generator=g, device=DEV, dtype=torch.int8)).to(torch.half)
+    x16 = (1 - 2 * torch.randint(0, 2, (N, K), generator=g, device=DEV, dtype=torch.int8)).to(torch.half)
+    wp, xp = lk.pack_sign(w16), lk.pack_sign(x16)
+    variant = ENGINES[engine]
+    assert lk.packed_kernel_id(wp, xp, MODE_XOR, 1, variant) == want_kernel
+    rows = np.unique(np.concatenate([rng.choice(N, 90, replace=False), [0, N - 1, N - 2, (N // 32) * 32, (N // 256) * 256]]))
+    cols = np.unique(np.concatenate([rng.choice(M, 120, replace=False), [0, M - 1, M - 2, (M // 32) * 32, (M // 128) * 128]]))
+    wsub = w16[torch.from_numpy(cols).to(DEV)].float().cpu()
+    xsub = x16[torch.from_numpy(rows).to(DEV)].float().cpu()
+    acc = (xsub @ wsub.T).to(torch.int32).numpy()
+    check_all_kinds(oracle, wp, xp, acc, M, N, variant, rng, rows, cols)
+    # the whole output: parity, range, the checksum of checksums
+    out = lk.bgemm_packed_forward(wp, xp, MODE_XOR, torch.int32, 1, variant)[0]
+    assert int(((out - K) % 2).abs().max()) == 0 and int(out.abs().max()) <= K
+    assert int(out.to(torch.int64).sum()) == int((w16.double().sum(0) * x16.double().sum(0)).sum().item())
+
+
+def test_config3_attention_av_all_192_heads():
+    """BASELINE configuration 3 at its full size, every element: 16 x 12 heads, attn {0,1} [512,512] x value +-1 [512,64]."""
+    rng = np.random.default_rng(3192)
+    Bn, S, D = 192, 512, 64
+    attn_bits = rng.integers(0, 2, (Bn, S, S), dtype=np.int8)
+    v = np.where(rng.integers(0, 2, (Bn, S, D), dtype=np.int8) == 1, np.float16(-1), np.float16(1)).astype(np.float16)
+    want = np.matmul(attn_bits.astype(np.float32), v.astype(np.float32)).astype(np.int32)
+    attn16 = to_dev((2 * attn_bits - 1).astype(np.float16))          # "1" must have its sign bit clear
+    ap, vp = lk.pack_sign(attn16), lk.pack_sign_transposed(to_dev(v))
+    assert lk.packed_kernel_id(vp, ap, MODE_ATTN_X) == B.KERNEL_MFMA_128x64
+    for variant in (VARIANT_AUTO, VARIANT_MFMA):
+        got = lk.bgemm_packed_forward(vp, ap, MODE_ATTN_X, torch.int32, 1, variant).cpu().numpy()
+        assert (got == want).all(), variant
+        # the reference's orientation (attn as the weight side, INSTR = 2) gives the transpose
+        got_t = lk.bgemm_packed_forward(ap, vp, MODE_ATTN, torch.int32, 1, variant).cpu().numpy()
+        assert (got_t.transpose(0, 2, 1) == want).all(), variant
+    goth = lk.bgemm_packed_forward(vp, ap, MODE_ATTN_X, torch.half).cpu().numpy()
+    assert (bits_of(goth) == bits_of(f16_of(want))).all()
+
+
+def test_narrow_outputs_ragged_batch():
+    """The 128 x 64 tile where the library picks it, ragged in every dimension."""
+    rng = np.random.default_rng(77)
+    Bn, M, N, K = 200, 50, 300, 700
+    w, x = pm1(rng, Bn, M, K), pm1(rng, Bn, N, K)
+    wp, xp = lk.pack_sign(to_dev(w)), lk.pack_sign(to_dev(x))
+    assert lk.packed_kernel_id(wp, xp, MODE_XOR) == B.KERNEL_MFMA_128x64
+    for mode in (MODE_XOR, MODE_ATTN_X):
+        assert (lk.bgemm_packed_forward(wp, xp, mode).cpu().numpy() == dense(mode, w, x)).all()
+    got = lk.bgemm_packed_forward(wp, xp, MODE_AND, torch.half, 1, VARIANT_MFMA).cpu().numpy()
+    assert (bits_of(got) == bits_of(f16_of(dense(MODE_AND, w, x)))).all()
+
+
+@pytest.mark.parametrize("N,want_kernel", [(256, B.KERNEL_SKINNY_QUAD), (2048, B.KERNEL_MFMA_256x128)])
+def test_config5_sweep_long_k(N, want_kernel):
+    """The K = 16384 points of configuration 5's sweep, split-K 1 / 2 / 4: sampled rows and columns against the
+    closed form, identities over the whole output, and agreement between the split-K values and the designs."""
+    M, K = 8192, 16384
+    g = torch.Generator(device=DEV).manual_seed(N)
+    w16 = (1 - 2 * torch.randint(0, 2, (M, K), generator=g, device=DEV, dtype=torch.int8)).to(torch.half)
+    x16 = (1 - 2 * torch.randint(0, 2, (N, K), generator=g, device=DEV, dtype=torch.int8)).to(torch.half)
+    wp, xp = lk.pack_sign(w16), lk.pack_sign(x16)
+    assert lk.packed_kernel_id(wp, xp, MODE_XOR) == want_kernel
+    out = lk.bgemm_packed_forward(wp, xp, MODE_XOR, torch.int32, 1)[0]
+    rng = np.random.default_rng(N)
+    rows, cols = rng.choice(N, 64, replace=False), rng.choice(M, 96, replace=False)
+    want = (x16[torch.from_numpy(rows).to(DEV)].float().cpu() @ w16[torch.from_numpy(cols).to(DEV)].float().cpu().T).to(torch.int32)
+    assert torch.equal(out[torch.from_numpy(rows).to(DEV)][:, torch.from_numpy(cols).to(DEV)].cpu(), want)
+    assert int(((out - K) % 2).abs().max()) == 0 and int(out.abs().max()) <= K
+    assert int(out.to(torch.int64).sum()) == int((w16.double().sum(0) * x16.double().sum(0)).sum().item())
+    for splitK in (2, 4):
+        assert torch.equal(lk.bgemm_packed_forward(wp, xp, MODE_XOR, torch.int32, splitK)[0], out), splitK
+    for variant in (VARIANT_MFMA, VARIANT_VALU):
+        assert torch.equal(lk.bgemm_packed_forward(wp, xp, MODE_XOR, torch.int32, 4, variant)[0], out), variant
+
+
+KERNELS_FOR_LONG_K = {
+    "mfma 32x128": (B.KERNEL_MFMA_32x128, 32), "mfma 256x256": (B.KERNEL_MFMA_256x256, 32),
+    "mfma 128x64": (B.KERNEL_MFMA_128x64, 32), "split-K in the block": (B.KERNEL_SKINNY_SPLITK, 32),
+    "four pieces": (B.KERNEL_SKINNY_QUAD, 32), "stream": (B.KERNEL_SKINNY_STREAM, 16), "popcount": (B.KERNEL_SKINNY_POPC, 1),
+}
+
+
+@pytest.mark.parametrize("kernel", list(KERNELS_FOR_LONG_K))
+def test_k_just_under_2_to_24_every_term_at_its_maximum(kernel):
+    """K = 2^24 - 32 with every bit set: the range term, both popcount terms and the AND-dot all lie between 2^23 and
+    2^24, where a signed 24-bit multiply would misread them.  Closed forms for all-ones / all-zero / half-set
+    operands in every mode; every kernel with an epilogue of its own, both engines, and the VALU design."""
+    kid, N = KERNELS_FOR_LONG_K[kernel]
+    K = (1 << 24) - 32
+    W = K // 32
+    ones = torch.full((32, W), -1, dtype=torch.int32, device=DEV)              # every sign bit set: all -1
+    half = ones[:N].clone()
+    half[:, ::2] = 0                                                            # every other word clear
+    pb = (W // 2) * 32                                                          # W is odd: one more word clear than set
+    zeros = torch.zeros((32, W), dtype=torch.int32, device=DEV)                 # all +1
+    w1, w0 = lk.tile_from_logical(ones, K), lk.tile_from_logical(zeros, K)
+    x1, xh = lk.tile_from_logical(ones[:N].contiguous(), K), lk.tile_from_logical(half, K)
+    tern = lambda p: lk.PackedBits(p.data, p.data.clone(), 1, p.rows, p.K)     # nonzero = sign plane: every set bit is a -1
+    variants = [force_kernel(kid, VARIANT_MFMA_F4)] + ([force_kernel(kid, VARIANT_MFMA)] if kid != B.KERNEL_SKINNY_POPC else [])
+    if kernel == "mfma 32x128":
+        variants.append(VARIANT_VALU)
+    two_planes = kid not in (B.KERNEL_MFMA_256x256,)
+    for variant in variants:
+        def run(w, x, mode):
+            out = lk.bgemm_packed_forward(w, x, mode, torch.int32, 1, variant)
+            lo, hi = int(out.min()), int(out.max())
+            assert lo == hi, (mode, lo, hi)
+            return lo
+        assert run(w1, x1, MODE_AND) == K and run(w1, x1, MODE_XOR) == K
+        assert run(w1, x1, MODE_ATTN) == 0 and run(w1, x1, MODE_ATTN_X) == 0
+        assert run(w0, x1, MODE_AND) == 0 and run(w0, x1, MODE_XOR) == -K
+        assert run(w0, x1, MODE_ATTN) == -K and run(w0, x1, MODE_ATTN_X) == 0
+        assert run(w1, xh, MODE_AND) == pb and run(w1, xh, MODE_XOR) == 2 * pb - K
+        assert run(w1, xh, MODE_ATTN_X) == -(K - pb) and run(w0, xh, MODE_ATTN) == K - 2 * pb
+        if two_planes:
+            assert run(w1, tern(x1), MODE_BWTA) == K and run(w0, tern(x1), MODE_BWTA) == -K
+            assert run(w1, tern(xh), MODE_BWTA) == pb
