@@ -14,6 +14,7 @@ MODE_AND, MODE_XOR, MODE_ATTN, MODE_BWTA, MODE_ATTN_X = 0, 1, 2, 3, 4
 OUT_I32, OUT_F16, OUT_F32_SCALED, OUT_F16_SCALED, OUT_BITS_F32, OUT_BITS_F16 = 0, 1, 2, 3, 4, 5
 SRC_F16, SRC_F32 = 0, 1
 ABI_VERSION = 7
+STATIC_SCRATCH_BYTES = 32 << 20      # BGEMM_STATIC_SCRATCH_BYTES
 VARIANT_AUTO, VARIANT_VALU, VARIANT_MFMA, VARIANT_MFMA_F4 = 0, 1, 2, 3
 # BGEMM_KERNEL_*: what bgemm_packed_kernel_id() returns and force_kernel() takes
 KERNEL_MFMA_256x256, KERNEL_MFMA_128x128, KERNEL_MFMA_64x128, KERNEL_MFMA_32x128, KERNEL_MFMA_256x128 = 0, 1, 2, 3, 4
@@ -55,6 +56,7 @@ SIGNATURES = {
     "bgemm_packed_weight_forward": (_int, [_int, _p, _p, _int, _i64, _p, _p, _int, _i64, _i64, _i64, _int, _p, _p, _p, _p, _p]),
     "bgemm_f16_workspace_bytes": (_sz, [_i64, _i64, _i64, _int]),
     "bgemm_f16_forward": (_int, [_p, _p, _p, _i64, _i64, _i64, _p, _sz, _int, _int, _p]),
+    "bgemm_f16_forward_static": (_int, [_p, _p, _p, _i64, _i64, _i64, _int, _int, _p]),
 }
 
 _lib = None

@@ -1,6 +1,7 @@
 // C ABI: argument checking, workspace carving, variant dispatch.
 #include "common.h"
 #include <string.h>
+#include <mutex>
 
 namespace bgemm {
 
@@ -360,4 +361,53 @@ extern "C" int bgemm_f16_forward(const void* W, const void* X, void* C, int64_t 
     if (rc) return rc;
     return bgemm_packed_forward(INSTR, wt, xt, nullptr, C, BGEMM_OUT_F16, 1, M, N, K, 0, 0, 0, splitK,
                                 BGEMM_VARIANT_AUTO, part, pb, cnt, cb, stream);
+}
+
+// ---- the same call for callers that cannot allocate -------------------------------------------
+// The workspace of bgemm_f16_forward (the two packed operands, split-K state) lives in a device array of the
+// library's own instead of a buffer the caller brings.  Every GPU holds its own copy of the array at its own
+// address; the array's name is only a host-side handle for hipGetSymbolAddress, never an address itself.
+static __device__ __align__(256) unsigned char scratch[BGEMM_STATIC_SCRATCH_BYTES];
+
+static int static_scratch(void** ptr)
+{
+    constexpr int MAX_DEVICES = 64;
+    static std::mutex mu;
+    static void* per_device[MAX_DEVICES] = {};
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(BGEMM_ELAUNCH, "bgemm_f16_forward_static: hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= MAX_DEVICES) return fail(BGEMM_EINVAL, "bgemm_f16_forward_static: device %d out of range", dev);
+    std::lock_guard<std::mutex> lock(mu);
+    if (!per_device[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));       // the address of THIS device's copy
+        if (e != hipSuccess || !p)
+            return fail(BGEMM_ELAUNCH, "bgemm_f16_forward_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+        per_device[dev] = p;
+    }
+    *ptr = per_device[dev];
+    return BGEMM_OK;
+}
+
+extern "C" int bgemm_f16_forward_static(const void* W, const void* X, void* C, int64_t M, int64_t N, int64_t K,
+                                        int splitK, int INSTR, void* stream)
+{
+    g_err[0] = 0;
+    if (M < 0 || N < 0 || K < 0 || splitK < 1)
+        return fail(BGEMM_EINVAL, "bgemm_f16_forward_static: bad shape M=%lld N=%lld K=%lld splitK=%d", (long long)M,
+                    (long long)N, (long long)K, splitK);
+    const size_t need = bgemm_f16_workspace_bytes(M, N, K, splitK);
+    if (need > (size_t)BGEMM_STATIC_SCRATCH_BYTES)
+        return fail(BGEMM_EWORKSPACE, "bgemm_f16_forward_static: M=%lld N=%lld K=%lld needs %zu bytes of scratch, the "
+                                      "library's own array holds %zu: use bgemm_f16_forward with a workspace",
+                    (long long)M, (long long)N, (long long)K, need, (size_t)BGEMM_STATIC_SCRATCH_BYTES);
+    void* ws = nullptr;
+    if (need) {     // (an empty problem touches no scratch and needs no device)
+        const int rc = static_scratch(&ws);
+        if (rc) return rc;
+    }
+    // Nothing in the scratch has to start at zero: the pack kernels write whole tiles, padding included, and
+    // the call clears the split-K counters it uses (with a kernel, not a memset node) before the GEMM.
+    return bgemm_f16_forward(W, X, C, M, N, K, ws, need ? (size_t)BGEMM_STATIC_SCRATCH_BYTES : 0, splitK, INSTR, stream);
 }

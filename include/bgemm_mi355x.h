@@ -238,6 +238,20 @@ size_t bgemm_f16_workspace_bytes(int64_t M, int64_t N, int64_t K, int splitK);
 int bgemm_f16_forward(const void* W, const void* X, void* C, int64_t M, int64_t N, int64_t K,
                       void* ws, size_t ws_bytes, int splitK, int INSTR, void* stream);
 
+/* bgemm_f16_forward for callers that cannot allocate device memory or bring a workspace: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference (whose
+ * wrapper allocates its output and workspace with torch::empty on every call, fp6_linear.cu:580-586).
+ * The scratch is a device array of BGEMM_STATIC_SCRATCH_BYTES inside the library, one copy per GPU, held
+ * until the process ends; the call allocates and frees nothing.  Shapes whose
+ * bgemm_f16_workspace_bytes(M, N, K, splitK) exceeds that size return BGEMM_EWORKSPACE (32 MiB covers
+ * (M + N) * K up to about 2^28 bits, e.g. 8192 x 8192 against 8192 x 8192).  All calls on one GPU share the
+ * one array: calls that overlap in time on the same GPU (two streams, two threads) race; serialise them, or
+ * use bgemm_f16_forward with a workspace each.  The first call on a GPU looks the array's address up
+ * (hipGetSymbolAddress): make it outside stream capture.  Same results as bgemm_f16_forward. */
+#define BGEMM_STATIC_SCRATCH_BYTES (32u << 20)
+int bgemm_f16_forward_static(const void* W, const void* X, void* C, int64_t M, int64_t N, int64_t K,
+                             int splitK, int INSTR, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
