@@ -1,19 +1,27 @@
 #!/usr/bin/env python3
 """Benchmark of the BGEMM / BWTA hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--all]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--headline-only] [--only SECTION]
 
 A step is one pass of the hot path over one batch of synthetic input: one 8192^3
 {-1,1}x{-1,1} BGEMM on prepacked operands (benchmark configuration 5, the compute-bound case the
 metric's target is quoted on), int32 output, operands resident in HBM before the timed
 region.  One JSON line goes to stdout; `value` is effective binary TOPS = 2*M*N*K / t
-(the reference drivers' own op count, lowbit_kernel/csrc/benchmark.cu:291).  With --all the
-line also carries the other benchmark configurations (MLP forward, batched attention A x V,
-decode-shape BWTA) under "all_configs".
+(the reference drivers' own op count, lowbit_kernel/csrc/benchmark.cu:291).
+
+Beside the headline the line carries, under "all_configs", one compact row per other benchmark
+configuration (MLP forward, batched attention A x V, decode-shape BWTA: one launch, 64 matrices in one
+launch, and the GEMMs a Llama-7B decode step issues; the sweep around 8192^3), each with its kernel, its time,
+TOPS, GB/s, bit-exactness and the roofline that bounds it; under "floor" what the hardware allows a
+decode-size launch (empty launch, cold read); under "mfma_peak_measured" the rate of the two MFMA
+instructions the library issues with nothing else going on (the reference's protocol: warm-up launches,
+then timed launches between two events, lowbit_kernel/csrc/kernel_test.h:10-11, csrc/benchmark.cu:275-291).
 """
 import argparse
+import ctypes
 import json
 import os
+import re
 import sys
 import time
 
@@ -25,11 +33,26 @@ for _p in (ROOT, os.path.join(ROOT, "bgemm-cuda_amd")):
 INT8_MFMA_PEAK_TOPS = 5000.0      # MI355X dense int8 MFMA, published
 FP4_MFMA_PEAK_TOPS = 10100.0      # MI355X dense fp4 MFMA, published
 HBM_PEAK_GBS = 8000.0             # MI355X HBM3E, published
-MEASURED_TRAFFIC_BYTES_C5_FP4 = int((96.5 + 257.0) * 2 ** 20)   # fetched + written, rocprofv3 --pmc
+C5_PROFILE = os.path.join(ROOT, "profiles", "gemm_mfma_f4_bgemm_8192x8192x8192.txt")
+PROBES_SO = os.path.join(ROOT, "libbench_probes.so")
+
+KERNEL_NAMES = {0: "mfma 256x256", 1: "mfma 128x128", 2: "mfma 64x128", 3: "mfma 32x128", 4: "mfma 256x128",
+                6: "mfma 64x64", 7: "mfma 128x64", 16: "decode stream", 17: "decode split-K in the block",
+                18: "decode four pieces a block", 19: "decode AND-popcount (vector ALU)", 32: "VALU popcount GEMM"}
 
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
+
+
+def measured_traffic_bytes():
+    """HBM bytes per launch of the headline kernel as the tracked profile summary states them (a line
+    `traffic_bytes_per_launch = N` under the FETCH_SIZE / WRITE_SIZE counter runs), or None."""
+    try:
+        m = re.search(r"^traffic_bytes_per_launch\s*=\s*(\d+)", open(C5_PROFILE).read(), re.M)
+        return int(m.group(1)) if m else None
+    except OSError:
+        return None
 
 
 def time_gpu(fn, warmup, steps):
@@ -83,6 +106,35 @@ def pm1_f16(shape, seed, device):
     return (1 - 2 * bits).to(torch.half)
 
 
+def ternary_f16(shape, seed, device):
+    """{-1, 0, +1} with p(0) = 0.5."""
+    import torch
+    g = torch.Generator(device=device).manual_seed(seed)
+    t = torch.randint(0, 4, shape, generator=g, device=device)
+    return torch.where(t == 0, -1.0, torch.where(t == 3, 1.0, 0.0)).to(torch.half)
+
+
+def random_packed(rows, K, batch, seed, device):
+    """A packed operand of random bits (rows a multiple of 32, K of 256: no padding to keep zero)."""
+    import torch
+    import lowbit_kernel as lk
+    assert rows % 32 == 0 and K % 256 == 0
+    g = torch.Generator(device=device).manual_seed(seed)
+    data = torch.randint(-2 ** 31, 2 ** 31 - 1, (batch, rows * K // 32), generator=g, device=device, dtype=torch.int32)
+    return lk.PackedBits(data, None, batch, rows, K)
+
+
+def unpacked_pm1(packed, b=0):
+    """The +-1 fp32 matrix [rows, K] behind matrix b of a packed operand."""
+    import torch
+    import lowbit_kernel as lk
+    one = lk.PackedBits(packed.data[b:b + 1], None, 1, packed.rows, packed.K)
+    logical = lk.logical_from_tiled(one)
+    shifts = torch.arange(31, -1, -1, device=logical.device, dtype=torch.int32)
+    bits = ((logical.unsqueeze(-1) >> shifts) & 1).reshape(packed.rows, -1)[:, :packed.K]
+    return (1 - 2 * bits).float()
+
+
 def check_sampled(out, w16, x16, n_rows=64, n_cols=64):
     """Spot parity check of an [N,M] XOR result against the fp32 closed form on sampled rows."""
     import torch
@@ -94,6 +146,25 @@ def check_sampled(out, w16, x16, n_rows=64, n_cols=64):
     return bool(torch.equal(out[cs][:, rs].cpu(), want))
 
 
+def kernel_of(w, x, mode, splitK=1, variant=0):
+    import lowbit_kernel as lk
+    return KERNEL_NAMES.get(lk.packed_kernel_id(w, x, mode, splitK, variant), "?")
+
+
+def row(name, ms, ops, bytes_alg, ok, kernel, bound, **more):
+    """One compact all_configs row; `bound` names the roofline ('mfma' against the fp4 peak the kernels issue, or 'hbm')."""
+    r = {"name": name, "kernel": kernel, "us": round(ms * 1e3, 3), "tops": round(ops / ms / 1e9, 1),
+         "gbs": round(bytes_alg / ms / 1e6, 1), "bit_exact": ok}
+    if bound == "mfma":
+        r["roofline"] = {"bound": "mfma", "frac": round(r["tops"] / FP4_MFMA_PEAK_TOPS, 4),
+                         "frac_of_int8_peak": round(r["tops"] / INT8_MFMA_PEAK_TOPS, 4)}
+    else:
+        r["roofline"] = {"bound": "hbm", "frac": round(r["gbs"] / HBM_PEAK_GBS, 4)}
+    r.update(more)
+    return r
+
+
+# ---------------------------------------------------------------- configuration 5: 8192^3 and its sweep
 def bench_c5(steps, warmup, M=8192, N=8192, K=8192, splitK=1, variant=0):
     import torch
     import lowbit_kernel as lk
@@ -109,7 +180,21 @@ def bench_c5(steps, warmup, M=8192, N=8192, K=8192, splitK=1, variant=0):
     pack_ms = time_gpu(lambda i: lk.pack_sign(x16), 2, 10)
     return {"name": "C5 BGEMM %dx%dx%d xor int32 splitK=%d" % (M, N, K, splitK), "ms": ms,
             "tops": ops / ms / 1e9, "gbs": bytes_alg / ms / 1e6, "ops": ops, "bytes": bytes_alg,
-            "bit_exact": ok, "act_pack_ms": pack_ms}, (w16, x16)
+            "bit_exact": ok, "act_pack_ms": pack_ms, "kernel": kernel_of(wp, xp, lk.MODE_XOR, splitK, variant)}, (w16, x16)
+
+
+def bench_sweep(steps=40, warmup=5):
+    """The sweep of configuration 5: K in {4096, 16384} x N in {256, 2048}, M = 8192.  One row per point: the
+    library does not split these shapes across blocks, so split-K 1, 2 and 4 run the same kernel (timed at 1 and 4)."""
+    rows = []
+    for (K, N) in [(4096, 256), (4096, 2048), (16384, 256), (16384, 2048)]:
+        r1, _ = bench_c5(steps, warmup, 8192, N, K, 1)
+        r4, _ = bench_c5(steps, warmup, 8192, N, K, 4)
+        rows.append(row("C5 sweep 8192x%dx%d xor int32" % (N, K), r1["ms"], r1["ops"], r1["bytes"],
+                        r1["bit_exact"] and r4["bit_exact"], r1["kernel"], "mfma", us_splitK_4=round(r4["ms"] * 1e3, 3),
+                        split_k_note="splitK 1 / 2 / 4 run one kernel: the value is an upper bound and these outputs fill the GPU without a K split"))
+        log(json.dumps(rows[-1]))
+    return rows
 
 
 def bench_c5_dropin(steps, warmup, M=8192, N=8192, K=8192):
@@ -128,9 +213,8 @@ def bench_c5_dropin(steps, warmup, M=8192, N=8192, K=8192):
     rs, cs = torch.randperm(M, generator=g)[:64].to(dev), torch.randperm(N, generator=g)[:64].to(dev)
     want = (x16[cs].float() @ w16[rs].float().T).half()
     ok = bool(torch.equal(out[0][cs][:, rs], want))
-    ops = 2.0 * M * N * K
-    return {"name": "C5 through the fp16 drop-in call %dx%dx%d (packs both operands per call, fp16 out)" % (M, N, K),
-            "ms": ms, "tops": ops / ms / 1e9, "ops": ops, "bit_exact": ok}
+    return row("C5 through the fp16 drop-in call %dx%dx%d (packs both operands per call, fp16 out)" % (M, N, K),
+               ms, 2.0 * M * N * K, 2.0 * (M * K + N * K + M * N), ok, "pack + mfma 256x256", "mfma")
 
 
 def cpu_baseline_c5(w16, x16, budget_s=12.0):
@@ -159,33 +243,119 @@ def cpu_baseline_c5(w16, x16, budget_s=12.0):
                       % (M, K, n, K, n, x16.shape[0], reps)}
 
 
-def bench_c4(steps, warmup, N, splitK, variant=0, copies=64):
-    """Decode-shape BWTA linear: W[11008,4096] prepacked, ternary activations, weights rotated
-    over `copies` buffers (> 256 MB in total) so no launch finds its weights in cache."""
+# ---------------------------------------------------------------- hardware floors and measured peaks
+def probes():
+    if not os.path.exists(PROBES_SO):
+        raise ImportError("%s is missing: build it with `python __graft_entry__.py`" % PROBES_SO)
+    L = ctypes.CDLL(PROBES_SO)
+    p, i64, ci = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+    L.bench_probe_empty.argtypes = [ci, ci, p, p]
+    L.bench_probe_read.argtypes = [p, i64, ci, ci, p, p]
+    L.bench_probe_mfma.argtypes = [ci, ci, ci, ci, p, p]
+    return L
+
+
+class ColdRead:
+    """Time of a plain read (no compute, no store) of `nbytes` that no cache holds: the probe walks a pool larger
+    than the 256 MB Infinity Cache, one piece per launch."""
+
+    def __init__(self):
+        import torch
+        self.L = probes()
+        self.pool = torch.ones((384 << 20) // 4, dtype=torch.int32, device="cuda:0")
+        self.scratch = torch.zeros(64, dtype=torch.int32, device="cuda:0")
+        self.cache = {}
+
+    def us(self, nbytes):
+        import torch
+        nbytes = int(nbytes) // 16 * 16
+        if nbytes not in self.cache:
+            copies = max(1, min(64, self.pool.numel() * 4 // nbytes))
+            st = lambda: torch.cuda.current_stream().cuda_stream
+            best = None
+            for blocks, threads in ((512, 512), (1024, 256), (1024, 512), (2048, 256)):
+                t = 1e3 * time_gpu_graph(lambda i: self.L.bench_probe_read(self.pool.data_ptr() + (i % copies) * nbytes, nbytes,
+                                                                           blocks, threads, self.scratch.data_ptr(), st()),
+                                         copies, 2, max(4, 256 // copies))
+                best = t if best is None else min(best, t)
+            self.cache[nbytes] = best
+        return self.cache[nbytes]
+
+
+def bench_floor(cold):
+    """What the hardware allows a kernel of the decode path's shape: the cost of launching an empty kernel,
+    of reading one cold 5.6 MB buffer (the packed W[11008,4096]), and the bandwidth a plain read sustains."""
+    import torch
+    L = cold.L
+    st = lambda: torch.cuda.current_stream().cuda_stream
+    nbytes = 11008 * 4096 // 8
+    res = {"empty_kernel_us": round(1e3 * time_gpu_graph(lambda i: L.bench_probe_empty(344, 512, cold.scratch.data_ptr(), st()), 64, 2, 20), 3)}
+    res["cold_read_5p6MB_us"] = round(cold.us(nbytes), 3)
+    res["cold_read_5p6MB_gbs"] = round(nbytes / cold.us(nbytes) / 1e3, 1)
+    total = 64 * nbytes
+    best = None
+    for blocks, threads in ((2048, 512), (4096, 512), (8192, 512)):
+        us = 1e3 * time_gpu_graph(lambda i: L.bench_probe_read(cold.pool.data_ptr(), total, blocks, threads, cold.scratch.data_ptr(), st()), 4, 2, 10)
+        best = us if best is None else min(best, us)
+    res["sustained_read_361MB_us"] = round(best, 2)
+    res["sustained_read_gbs"] = round(total / best / 1e3, 1)
+    res["sustained_read_frac_of_8TBs"] = round(res["sustained_read_gbs"] / HBM_PEAK_GBS, 4)
+    return res
+
+
+def bench_mfma_peak(cold):
+    """The matrix cores alone: v_mfma_f32_32x32x64_f8f6f4 (E2M1 operands) and v_mfma_i32_32x32x32_i8 from two waves
+    per SIMD with eight independent accumulators each, no memory traffic; then with two and four independent vector-ALU
+    instructions after every MFMA (what the bit expansion adds to the issue stream).  20 warm-up + 100 timed launches."""
+    import torch
+    L = cold.L
+    out = torch.empty(512 * 256, dtype=torch.int32, device="cuda:0")
+    st = lambda: torch.cuda.current_stream().cuda_stream
+    iters, blocks = 2000, 512
+    res = {}
+    for fp4 in (1, 0):
+        for valu in (0, 2, 4):
+            ms = time_gpu(lambda i: L.bench_probe_mfma(fp4, valu, blocks, iters, out.data_ptr(), st()), 20, 100)
+            ops = 2.0 * 32 * 32 * (64 if fp4 else 32) * 8 * iters * 4 * blocks
+            key = ("fp4" if fp4 else "int8") + ("_tops" if valu == 0 else "_tops_with_%d_valu_per_mfma" % valu)
+            res[key] = round(ops / ms / 1e9, 1)
+    res["fp4_frac_of_datasheet"] = round(res["fp4_tops"] / FP4_MFMA_PEAK_TOPS, 4)
+    res["int8_frac_of_datasheet"] = round(res["int8_tops"] / INT8_MFMA_PEAK_TOPS, 4)
+    return res
+
+
+# ---------------------------------------------------------------- configuration 4: decode-shape BWTA
+def bench_decode(cold, name, M, K, Ns, steps=640, total_mb=361):
+    """One launch per matrix: prepacked W[M,K] x ternary activations [N,K] -> int32, weights rotated over enough
+    copies (> 256 MB in total) that no launch finds them in a cache; launches replayed from a HIP graph.  Every row
+    states its fraction of 8 TB/s and its ratio to a plain cold read of the same number of bytes."""
     import torch
     import lowbit_kernel as lk
     dev = torch.device("cuda:0")
-    M, K = 11008, 4096
-    g = torch.Generator(device=dev).manual_seed(4000 + N)
-    t = torch.randint(0, 4, (N, K), generator=g, device=dev)
-    x16 = torch.where(t == 0, -1.0, torch.where(t == 3, 1.0, 0.0)).to(torch.half)      # p(0) = 0.5
-    xt = lk.pack_ternary(x16)
-    w16 = pm1_f16((M, K), 4001, dev)
-    base = lk.pack_sign(w16)
-    wps = [lk.PackedBits(base.data.clone(), None, 1, M, K) for _ in range(copies)]
-    out = torch.empty((1, N, M), dtype=torch.int32, device=dev)
-    fn = lambda i: lk.bgemm_packed_forward(wps[i % copies], xt, lk.MODE_BWTA, torch.int32, splitK, variant, out=out)
-    ms_eager = time_gpu(fn, warmup, steps)
-    ms = time_gpu_graph(fn, copies, 4, max(2, steps // copies))
-    want = (torch.sign(x16.float()).cpu() @ w16.float().cpu().T).to(torch.int32)
-    ok = bool(torch.equal(out[0].cpu(), want))
-    ops = 2.0 * M * N * K
-    bytes_alg = M * K / 8 + 2 * N * K / 8 + 4.0 * M * N
-    return {"name": "C4 BWTA W[11008,4096] N=%d splitK=%d" % (N, splitK), "ms": ms, "tops": ops / ms / 1e9,
-            "ms_eager_launch": ms_eager, "gbs": bytes_alg / ms / 1e6, "ops": ops, "bytes": bytes_alg, "bit_exact": ok}
+    wbytes = M * K // 8
+    copies = max(8, min(64, int(total_mb * 1e6 // wbytes)))
+    pool = random_packed(M, K, copies, 4001, dev)
+    wps = [lk.PackedBits(pool.data[c:c + 1], None, 1, M, K) for c in range(copies)]
+    w_pm1 = unpacked_pm1(pool, 0)
+    rows = []
+    for N in Ns:
+        x16 = ternary_f16((N, K), 4000 + N, dev)
+        xt = lk.pack_ternary(x16)
+        out = torch.empty((1, N, M), dtype=torch.int32, device=dev)
+        fn = lambda i: lk.bgemm_packed_forward(wps[i % copies], xt, lk.MODE_BWTA, torch.int32, 8, 0, out=out)
+        fn(0)
+        ok = bool(torch.equal(out[0], (torch.sign(x16.float()) @ w_pm1.T).to(torch.int32)))
+        ms = time_gpu_graph(fn, copies, 4, max(2, steps // copies))
+        bytes_alg = wbytes + 2 * N * K / 8 + 4.0 * M * N
+        floor_us = cold.us(bytes_alg)
+        rows.append(row("%s W[%d,%d] N=%d, one launch (splitK<=8), cold weights" % (name, M, K, N), ms, 2.0 * M * N * K, bytes_alg, ok,
+                        kernel_of(wps[0], xt, lk.MODE_BWTA, 8), "hbm", cold_read_same_bytes_us=round(floor_us, 3),
+                        ratio_to_cold_read=round(ms * 1e3 / floor_us, 3)))
+        log(json.dumps(rows[-1]))
+    return rows
 
 
-def bench_c4_batched(steps, N, B=64):
+def bench_decode_batched(N, B=64, replays=10):
     """The same decode-shape BWTA linear over B weight matrices in ONE launch (the layers of a model,
     a set of experts): 361 MB of weights stream through once, so the launch is long enough to show the
     bandwidth the kernel sustains rather than the latency of one 5.6 MB launch."""
@@ -193,93 +363,44 @@ def bench_c4_batched(steps, N, B=64):
     import lowbit_kernel as lk
     dev = torch.device("cuda:0")
     M, K = 11008, 4096
-    g = torch.Generator(device=dev).manual_seed(4100 + N)
-    t = torch.randint(0, 4, (N, K), generator=g, device=dev)
-    x16 = torch.where(t == 0, -1.0, torch.where(t == 3, 1.0, 0.0)).to(torch.half)
+    x16 = ternary_f16((N, K), 4100 + N, dev)
     xt = lk.pack_ternary(x16)
-    words = M * K // 32
-    wdata = torch.randint(-2 ** 31, 2 ** 31 - 1, (B, words), generator=g, device=dev, dtype=torch.int32)
-    wb = lk.PackedBits(wdata, None, B, M, K)
+    wb = random_packed(M, K, B, 4101, dev)
     out = torch.empty((B, N, M), dtype=torch.int32, device=dev)
     fn = lambda i: lk.bgemm_packed_forward(wb, xt, lk.MODE_BWTA, torch.int32, 1, 0, out=out)
-    ms = time_gpu_graph(fn, 4, 2, max(5, steps // 40))
-    # parity of three of the matrices against the fp32 closed form on unpacked bits
+    ms = time_gpu_graph(fn, 4, 2, replays)
     ok = True
-    for b in (0, B // 2, B - 1):
-        w_logical = lk.logical_from_tiled(lk.PackedBits(wdata[b:b + 1], None, 1, M, K))
-        shifts = torch.arange(31, -1, -1, device=dev, dtype=torch.int32)
-        bits = ((w_logical.unsqueeze(-1) >> shifts) & 1).reshape(M, K)
-        want = (torch.sign(x16.float()) @ (1 - 2 * bits).float().T).to(torch.int32)
-        ok = ok and bool(torch.equal(out[b], want))
-    ops = 2.0 * B * M * N * K
+    for b in (0, B // 2, B - 1):       # parity of three of the matrices against the fp32 closed form on unpacked bits
+        ok = ok and bool(torch.equal(out[b], (torch.sign(x16.float()) @ unpacked_pm1(wb, b).T).to(torch.int32)))
     bytes_alg = B * (M * K / 8 + 4.0 * M * N) + 2 * N * K / 8
-    return {"name": "C4 batched: %d x BWTA W[11008,4096] N=%d in one launch" % (B, N), "ms": ms, "tops": ops / ms / 1e9,
-            "gbs": bytes_alg / ms / 1e6, "ops": ops, "bytes": bytes_alg, "bit_exact": ok}
+    return row("C4 %d x BWTA W[11008,4096] N=%d in one launch" % (B, N), ms, 2.0 * B * M * N * K, bytes_alg, ok,
+               kernel_of(wb, xt, lk.MODE_BWTA), "hbm")
 
 
-def bench_c4_from_fp16(steps, N, copies=64):
+def bench_decode_from_fp16(N, steps=640, copies=64):
     """A decode step as a model runs it: fp16 activations in, prepacked W[11008,4096], int32 out.  Timed as two
-    launches (ternary pack, then the packed GEMM) and as the one launch that packs its activations itself; weights
-    rotate over `copies` buffers as in bench_c4."""
+    launches (ternary pack, then the packed GEMM) and as the one launch that packs its activations itself."""
     import torch
     import lowbit_kernel as lk
     dev = torch.device("cuda:0")
     M, K = 11008, 4096
-    g = torch.Generator(device=dev).manual_seed(4200 + N)
-    t = torch.randint(0, 4, (N, K), generator=g, device=dev)
-    x16 = torch.where(t == 0, -1.0, torch.where(t == 3, 1.0, 0.0)).to(torch.half)
-    base = lk.pack_sign(pm1_f16((M, K), 4001, dev))
-    wps = [lk.PackedBits(base.data.clone(), None, 1, M, K) for _ in range(copies)]
+    x16 = ternary_f16((N, K), 4200 + N, dev)
+    pool = random_packed(M, K, copies, 4001, dev)
+    wps = [lk.PackedBits(pool.data[c:c + 1], None, 1, M, K) for c in range(copies)]
     two = lambda i: lk.bgemm_packed_forward(wps[i % copies], lk.pack_ternary(x16), lk.MODE_BWTA, torch.int32)
     one = lambda i: lk.bgemm_packed_weight_forward(wps[i % copies], x16, lk.MODE_BWTA, torch.int32)
     ok = bool(torch.equal(two(0)[0], one(0)))
     ms_two = time_gpu_graph(two, copies, 2, max(2, steps // copies))
     ms_one = time_gpu_graph(one, copies, 2, max(2, steps // copies))
-    ms_one_eager, ms_two_eager = time_gpu(one, 20, steps), time_gpu(two, 20, steps)
-    ops = 2.0 * M * N * K
+    ms_one_eager = time_gpu(one, 20, steps)
     bytes_alg = M * K / 8 + 2.0 * N * K + 4.0 * M * N
-    return {"name": "C4 decode step from fp16 activations, W[11008,4096] N=%d (one launch: the kernel packs x itself)" % N,
-            "ms": ms_one, "ms_pack_then_gemm": ms_two, "ms_eager_launch": ms_one_eager, "ms_pack_then_gemm_eager": ms_two_eager,
-            "tops": ops / ms_one / 1e9, "gbs": bytes_alg / ms_one / 1e6, "ops": ops, "bytes": bytes_alg, "bit_exact": ok}
+    return row("C4 decode step from fp16 activations W[11008,4096] N=%d, one launch (the kernel packs x itself)" % N, ms_one,
+               2.0 * M * N * K, bytes_alg, ok, "decode kernels, activations packed in the launch", "hbm",
+               us_pack_launch_then_gemm=round(ms_two * 1e3, 3), us_launched_from_python=round(ms_one_eager * 1e3, 3))
 
 
-def bench_floor():
-    """What the hardware allows a kernel of the decode path's shape: the cost of launching an empty kernel,
-    of reading one cold 5.6 MB buffer (the packed W[11008,4096]), and the bandwidth a plain read sustains."""
-    import ctypes
-    import torch
-    so = os.path.join(ROOT, "bgemm-cuda_amd", "libbgemm_membench.so")
-    L = ctypes.CDLL(so)
-    p, i64, ci = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
-    L.bgemm_membench_empty.argtypes = [ci, ci, p, p]
-    L.bgemm_membench_read.argtypes = [p, i64, ci, ci, p, p]
-    dev = torch.device("cuda:0")
-    nbytes, copies = 11008 * 4096 // 8, 64
-    buf = torch.ones(copies * nbytes // 4, dtype=torch.int32, device=dev)
-    scratch = torch.zeros(64, dtype=torch.int32, device=dev)
-    st = lambda: torch.cuda.current_stream().cuda_stream
-    res = {}
-    res["empty_kernel_us"] = 1e3 * time_gpu_graph(
-        lambda i: L.bgemm_membench_empty(344, 512, scratch.data_ptr(), st()), 64, 2, 20)
-    best = None
-    for blocks, threads in ((512, 512), (1024, 256), (1024, 512), (2048, 256)):
-        us = 1e3 * time_gpu_graph(lambda i: L.bgemm_membench_read(buf.data_ptr() + (i % copies) * nbytes, nbytes, blocks,
-                                                                  threads, scratch.data_ptr(), st()), copies, 2, 20)
-        best = us if best is None else min(best, us)
-    res["cold_read_5p6MB_us"] = best
-    res["cold_read_5p6MB_gbs"] = nbytes / best / 1e3
-    best = None
-    for blocks, threads in ((2048, 512), (4096, 512), (8192, 512)):
-        us = 1e3 * time_gpu_graph(lambda i: L.bgemm_membench_read(buf.data_ptr(), copies * nbytes, blocks, threads,
-                                                                  scratch.data_ptr(), st()), 4, 2, 10)
-        best = us if best is None else min(best, us)
-    res["sustained_read_361MB_us"] = best
-    res["sustained_read_gbs"] = copies * nbytes / best / 1e3
-    res["sustained_read_frac_of_8TBs"] = res["sustained_read_gbs"] / HBM_PEAK_GBS
-    return res
-
-
-def bench_c3(steps, warmup, variant=0):
+# ---------------------------------------------------------------- configurations 3 and 2
+def bench_c3(steps=200, warmup=20, variant=0):
     """192 x ([512,512] {0,1} x [512,64] {-1,1}) -> int32 [192,512,64]."""
     import torch
     import lowbit_kernel as lk
@@ -287,25 +408,39 @@ def bench_c3(steps, warmup, variant=0):
     B, S, D = 192, 512, 64
     attn16 = pm1_f16((B, S, S), 3001, dev)                 # sign bit clear = 1
     v16 = pm1_f16((B, S, D), 3002, dev)
-    ap, vp = lk.pack_sign(attn16), lk.pack_sign(v16.transpose(1, 2).contiguous())
+    ap, vp = lk.pack_sign(attn16), lk.pack_sign_transposed(v16)
     out = torch.empty((B, S, D), dtype=torch.int32, device=dev)
     fn = lambda i: lk.bgemm_packed_forward(vp, ap, lk.MODE_ATTN_X, torch.int32, 1, variant, out=out)
     ms_eager = time_gpu(fn, warmup, steps)
     ms = time_gpu_graph(fn, 20, 4, max(2, steps // 20))
-    want = torch.bmm((attn16[:4] > 0).float(), v16[:4].float()).to(torch.int32)
-    ok = bool(torch.equal(out[:4], want))
+    ok = bool(torch.equal(out, torch.bmm((attn16 > 0).float(), v16.float()).to(torch.int32)))      # every head
     ops = 2.0 * B * S * S * D
     bytes_alg = B * (S * S / 8 + S * D / 8 + 4.0 * S * D)
-    return {"name": "C3 attention AxV 192x[512,512]x[512,64]", "ms": ms, "ms_eager_launch": ms_eager,
-            "tops": ops / ms / 1e9,
-            "gbs": bytes_alg / ms / 1e6, "ops": ops, "bytes": bytes_alg, "bit_exact": ok}
+    return row("C3 attention AxV 192x[512,512]x[512,64] int32", ms, ops, bytes_alg, ok, kernel_of(vp, ap, lk.MODE_ATTN_X), "hbm",
+               us_launched_from_python=round(ms_eager * 1e3, 3))
 
 
-def bench_c2(steps, warmup):
+def bench_qk(steps=100):
+    """The other half of the attention pair: Q.K^T, 192 x ([512,64] x [64,512]) -> fp16 scores [192,512,512]."""
+    import torch
+    import lowbit_kernel as lk
+    dev = torch.device("cuda:0")
+    B, S, D = 192, 512, 64
+    q16, k16 = pm1_f16((B, S, D), 3003, dev), pm1_f16((B, S, D), 3004, dev)
+    qp, kp = lk.pack_sign(q16), lk.pack_sign(k16)
+    out = torch.empty((B, S, S), dtype=torch.half, device=dev)
+    fn = lambda i: lk.bgemm_packed_forward(kp, qp, lk.MODE_XOR, torch.half, 1, 0, out=out)
+    ms = time_gpu_graph(fn, 10, 2, max(2, steps // 10))
+    ok = bool(torch.equal(out, torch.bmm(q16.float(), k16.float().transpose(1, 2)).half()))
+    bytes_alg = B * (2 * S * D / 8 + 2.0 * S * S)
+    return row("attention Q.K^T 192x[512,64]x[64,512] fp16", ms, 2.0 * B * S * S * D, bytes_alg, ok, kernel_of(kp, qp, lk.MODE_XOR), "hbm")
+
+
+def bench_c2(steps=200, warmup=20):
     """3-layer binarised MLP forward 784->4096->4096->10, batch 128, fp16 activations and per-output-channel
-    fp16 scales.  Timed twice: op by op through the fp16 drop-in call (weights packed on every call, scaling as
-    separate torch kernels, as the reference layer does), and fused (weights prepacked once, activations
-    sign-packed in one pass, scaling applied in the GEMM's store)."""
+    fp16 scales.  Timed op by op through the fp16 drop-in call (weights packed on every call, scaling as
+    separate torch kernels, as the reference layer does), fused (weights prepacked once, activations
+    sign-packed in one pass, scaling applied in the GEMM's store), and with nothing but bits between the layers."""
     import torch
     import lowbit_kernel as lk
     dev = torch.device("cuda:0")
@@ -336,61 +471,117 @@ def bench_c2(steps, warmup):
         for l in range(2):
             hp = lk.bgemm_packed_forward(Wps[l], hp, lk.MODE_XOR, splitK=8, scale=(sws[l], sa, None), bits_out=hidden[l])
         return lk.bgemm_packed_forward(Wps[2], hp, lk.MODE_XOR, splitK=8, scale=(sws[2], sa, None))[0]
-    same = bool(torch.equal(fwd_ops(0), fwd_fused(0))) and bool(torch.equal(fwd_ops(0), fwd_bits(0)))
+    # the fp16 reference: torch matmul on the de-binarised tensors, scaled op by op
+    h = x
+    for W, sw in zip(Ws, sws):
+        sx = torch.where(h.view(torch.int16) < 0, -1.0, 1.0)
+        sw_ = torch.where(W.view(torch.int16) < 0, -1.0, 1.0)
+        h = (sx @ sw_.T).half() * sw * sa
+    same = bool(torch.equal(fwd_ops(0), h)) and bool(torch.equal(fwd_fused(0), h)) and bool(torch.equal(fwd_bits(0), h))
     ms_ops = time_gpu(fwd_ops, warmup, steps)
     ms_fused = time_gpu(fwd_fused, warmup, steps)
     ms_graph = time_gpu_graph(fwd_fused, 4, 2, max(2, steps // 4))
     ms_bits = time_gpu_graph(fwd_bits, 4, 2, max(2, steps // 4))
-    # what a Python caller sees per forward when the four launches are replayed as one captured graph
-    import bgemm_linear as bl
-    fast = bl.GraphedInference(lambda t: fwd_bits(0, t), x)
-    same = same and bool(torch.equal(fast(x), fwd_bits(0)))
-    ms_call = time_gpu(lambda i: fast(x), warmup, steps)
     ops = 2.0 * 128 * (784 * 4096 + 4096 * 4096 + 4096 * 10)
-    return {"name": "C2 MLP 784-4096-4096-10 batch 128, fp16 in/out, bits between layers (4 launches, graph replay)",
-            "ms": ms_bits, "ms_fused_6_launches": ms_graph, "ms_graph_call_from_python": ms_call,
-            "ms_eager_launch": ms_fused, "ms_op_by_op": ms_ops,
-            "tops": ops / ms_bits / 1e9, "ops": ops, "bit_exact": same}
+    bytes_alg = sum(W.numel() for W in Ws) / 8 + 2.0 * 128 * (784 + 10)
+    return row("C2 MLP 784-4096-4096-10 batch 128, fp16 in/out, bits between layers (4 launches, graph replay)", ms_bits, ops,
+               bytes_alg, same, "pack + three GEMM launches", "mfma", us_fused_6_launches=round(ms_graph * 1e3, 2),
+               us_fused_launched_from_python=round(ms_fused * 1e3, 2), us_op_by_op_drop_in=round(ms_ops * 1e3, 2))
 
 
-def run_extra(which, quick=False, variant=0):
-    """The non-headline benchmark configurations: 'c4' decode BWTA, 'c3' attention, 'c2' MLP, 'sweep'.
-    quick: a tenth of the launches (for counter collection, where every dispatch is serialised)."""
-    extra = []
-    div = 10 if quick else 1
-    if which in ("c4", "all"):
-        for N in (1, 4, 16):
-            for sk in (1, 8):
-                extra.append(bench_c4(2000 // div, 200 // div, N, sk, variant))
-                log(json.dumps(extra[-1]))
-        for N in (32, 64, 128):             # a batch of decode steps, beyond the configuration's row counts
-            extra.append(bench_c4(1000 // div, 100 // div, N, 1, variant))
-            log(json.dumps(extra[-1]))
-        for N in (1, 4, 16):
-            extra.append(bench_c4_batched(400 // div, N))
-            log(json.dumps(extra[-1]))
-        for N in (1, 4):
-            extra.append(bench_c4_from_fp16(2000 // div, N))
-            log(json.dumps(extra[-1]))
-    if which in ("c3", "all"):
-        extra.append(bench_c3(200 // div, 20 // div + 1, variant))
-        log(json.dumps(extra[-1]))
-    if which in ("c2", "all"):
-        extra.append(bench_c2(200 // div, 20 // div + 1))
-        log(json.dumps(extra[-1]))
-    if which in ("sweep", "all"):
-        extra.append(bench_c5_dropin(50 // div + 2, 5))
-        log(json.dumps(extra[-1]))
-        for (K, N) in [(4096, 256), (4096, 2048), (16384, 256), (16384, 2048)]:
-            for sk in (1, 2, 4):
-                r, _ = bench_c5(20, 3, 8192, N, K, sk)
-                extra.append(r)
-                log(json.dumps(r))
-    for r in extra:
-        r["frac_int8_mfma"] = r["tops"] / INT8_MFMA_PEAK_TOPS
-        if "gbs" in r:
-            r["frac_hbm"] = r["gbs"] / HBM_PEAK_GBS
-    return extra
+# ---------------------------------------------------------------- thresholds behind the dispatch
+THRESHOLD_SHAPES = [
+    # (planes, batch, M, N, K): around the choices of pick_cfg (general kernel tiles) and of the decode kernels' ranges
+    (1, 1, 8192, 8192, 2048), (1, 1, 8192, 8192, 4096), (1, 1, 8192, 8192, 8192), (1, 1, 8192, 8192, 16384),
+    (1, 1, 8192, 2048, 4096), (1, 1, 8192, 2048, 16384), (1, 1, 11008, 768, 4096), (1, 1, 4096, 2048, 4096),
+    (1, 1, 8192, 256, 4096), (1, 1, 8192, 256, 8192), (1, 1, 8192, 256, 16384), (1, 1, 8192, 512, 8192),
+    (1, 1, 8192, 768, 16384), (1, 1, 8192, 1024, 16384), (1, 1, 1024, 1024, 16384), (1, 1, 4096, 256, 11008),
+    (1, 1, 4096, 256, 4096), (1, 1, 11008, 128, 4096), (1, 1, 4096, 384, 4096), (1, 1, 2048, 256, 16384),
+    (1, 1, 256, 256, 16384), (1, 1, 4096, 128, 4096), (1, 192, 512, 512, 64), (1, 192, 64, 512, 512),
+    (2, 1, 11008, 32, 4096), (2, 1, 11008, 64, 4096), (2, 1, 11008, 128, 4096), (2, 1, 4096, 128, 11008),
+    (2, 1, 4096, 256, 11008), (2, 1, 4096, 512, 11008), (2, 1, 8192, 128, 8192), (2, 1, 8192, 256, 8192),
+]
+
+
+def bench_thresholds(steps=60):
+    """Every shape above under every kernel that can take it (BGEMM_FORCE_KERNEL), weights from HBM (rotating copies
+    beyond the Infinity Cache) and from a warm cache: the timings the dispatch thresholds of the library rest on."""
+    import torch
+    import lowbit_kernel as lk
+    import _lib as B
+    dev = torch.device("cuda:0")
+    general = [B.KERNEL_MFMA_256x256, B.KERNEL_MFMA_256x128, B.KERNEL_MFMA_128x128, B.KERNEL_MFMA_64x128, B.KERNEL_MFMA_32x128,
+               B.KERNEL_MFMA_128x64, B.KERNEL_MFMA_64x64]
+    rows = []
+    for planes, batch, M, N, K in THRESHOLD_SHAPES:
+        mode = lk.MODE_BWTA if planes == 2 else lk.MODE_XOR
+        wbytes = batch * M * K // 8
+        copies = max(2, min(40, int(300e6 // wbytes)))
+        pool = lk.pack_sign(pm1_f16((copies * batch, M, K), 11, dev))
+        wps = [lk.PackedBits(pool.data[c * batch:(c + 1) * batch], None, batch, M, K) for c in range(copies)]
+        if planes == 2:
+            xp = lk.pack_ternary(ternary_f16((batch, N, K) if batch > 1 else (N, K), 12, dev))
+        else:
+            xp = lk.pack_sign(pm1_f16((batch, N, K) if batch > 1 else (N, K), 12, dev))
+        out = torch.empty((batch, N, M), dtype=torch.int32, device=dev)
+        auto = lk.packed_kernel_id(wps[0], xp, mode, 8)
+        res = {"shape": "%d planes, batch %d, M=%d N=%d K=%d" % (planes, batch, M, N, K), "auto": KERNEL_NAMES[auto], "us_cold": {}, "us_warm": {}}
+        ref = None
+        for kid in general + [B.KERNEL_SKINNY_SPLITK, B.KERNEL_SKINNY_QUAD]:
+            if planes == 2 and kid in (B.KERNEL_MFMA_256x256, B.KERNEL_MFMA_256x128):
+                continue
+            if kid in (B.KERNEL_MFMA_128x64, B.KERNEL_MFMA_64x64) and M > 64:
+                continue
+            if kid >= B.KERNEL_SKINNY_STREAM and -(-M // 32) * -(-N // 32) * batch > 8192:
+                continue
+            v = B.force_kernel(kid)
+            fn = lambda i: lk.bgemm_packed_forward(wps[i % copies], xp, mode, torch.int32, 8, v, out=out)
+            try:
+                fn(0)
+            except ValueError:
+                continue
+            if ref is None:
+                ref = out.clone()
+            elif not torch.equal(out, ref):
+                res["mismatch"] = KERNEL_NAMES[kid]
+            res["us_cold"][KERNEL_NAMES[kid]] = round(1e3 * time_gpu_graph(fn, copies, 2, max(2, steps // copies)), 2)
+            res["us_warm"][KERNEL_NAMES[kid]] = round(1e3 * time_gpu_graph(lambda i: fn(0), 8, 2, max(2, steps // 8)), 2)
+        res["fastest_cold"] = min(res["us_cold"], key=res["us_cold"].get)
+        res["auto_vs_fastest_cold"] = round(res["us_cold"][res["auto"]] / res["us_cold"][res["fastest_cold"]], 3) if res["auto"] in res["us_cold"] else None
+        rows.append(res)
+        log(json.dumps(res))
+        del pool, wps, xp, out
+    return rows
+
+
+# ---------------------------------------------------------------- sections
+def section_decode(cold):
+    rows = bench_decode(cold, "C4 BWTA", 11008, 4096, (1, 4, 16))
+    for N in (1, 4, 16):
+        rows.append(bench_decode_batched(N))
+        log(json.dumps(rows[-1]))
+    # the GEMMs a Llama-7B decode step issues against one set of activations: QKV fused, gate + up fused, down
+    rows += bench_decode(cold, "Llama-7B QKV fused, BWTA", 12288, 4096, (1, 4, 16))
+    rows += bench_decode(cold, "Llama-7B gate+up fused, BWTA", 22016, 4096, (1, 4, 16))
+    rows += bench_decode(cold, "Llama-7B down, BWTA", 4096, 11008, (1, 4, 16))
+    for N in (1, 4):
+        rows.append(bench_decode_from_fp16(N))
+        log(json.dumps(rows[-1]))
+    return rows
+
+
+def all_configs(cold):
+    rows = [bench_c2()]
+    log(json.dumps(rows[-1]))
+    rows.append(bench_c3())
+    log(json.dumps(rows[-1]))
+    rows.append(bench_qk())
+    log(json.dumps(rows[-1]))
+    rows += section_decode(cold)
+    rows += bench_sweep()
+    rows.append(bench_c5_dropin(20, 3))
+    log(json.dumps(rows[-1]))
+    return rows
 
 
 def main():
@@ -398,15 +589,13 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--all", action="store_true", help="also time the other benchmark configurations")
-    ap.add_argument("--only", choices=["c2", "c3", "c4", "sweep"], help="time just that configuration (for profiling)")
+    ap.add_argument("--headline-only", action="store_true", help="time the 8192^3 launch only (profiling runs)")
+    ap.add_argument("--only", choices=["c2", "c3", "c4", "sweep", "floor", "peak", "thresholds"],
+                    help="time just that section and print it (for profiling and for re-deriving the dispatch thresholds)")
     ap.add_argument("--variant", type=int, default=0, help="0 auto, 1 VALU, 2 MFMA int8, 3 MFMA fp4")
     ap.add_argument("--split-k", type=int, default=1,
                     help="splitK of the headline launch: the most K ranges a tile may be computed in (same bits for any value)")
-    ap.add_argument("--quick", action="store_true", help="with --only: a tenth of the launches (counter collection)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--floor", action="store_true",
-                    help="print the hardware floors for the decode shape (empty launch, cold 5.6 MB read, sustained read)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run a 256 MiB device-to-device copy (known traffic, for scaling rocprof counters)")
     args = ap.parse_args()
@@ -424,32 +613,51 @@ def main():
         dst = torch.empty_like(src)
         ms = time_gpu(lambda i: dst.copy_(src), 2, 5)
         log("calibration copy: 256 MiB read + 256 MiB written per launch, %.4f ms" % ms)
-    if args.floor:
-        print(json.dumps({"floor": bench_floor()}), flush=True)
-        return
+        del src, dst
     if args.only:
-        print(json.dumps({"configs": run_extra(args.only, args.quick, args.variant)}), flush=True)
+        cold = ColdRead() if args.only in ("c4", "floor", "peak") else None
+        res = {"c2": lambda: [bench_c2()], "c3": lambda: [bench_c3(), bench_qk()], "c4": lambda: section_decode(cold),
+               "sweep": bench_sweep, "floor": lambda: bench_floor(cold), "peak": lambda: bench_mfma_peak(cold),
+               "thresholds": bench_thresholds}[args.only]()
+        print(json.dumps({args.only: res}), flush=True)
         return
+
+    extra = floor = peak_measured = None
+    if not args.headline_only:
+        cold = ColdRead()
+        floor = bench_floor(cold)
+        log("floor:", json.dumps(floor))
+        peak_measured = bench_mfma_peak(cold)
+        log("mfma peak:", json.dumps(peak_measured))
+        extra = all_configs(cold)
+        del cold
+        torch.cuda.empty_cache()
 
     c5, (w16, x16) = bench_c5(args.steps, args.warmup, splitK=args.split_k, variant=args.variant)
     log("C5:", json.dumps(c5))
     cpu = None if args.no_cpu else cpu_baseline_c5(w16, x16)
     del w16, x16
-    extra = run_extra("all") if args.all else []
     fp4 = args.variant in (0, 3)
     peak = FP4_MFMA_PEAK_TOPS if fp4 else INT8_MFMA_PEAK_TOPS
-    # HBM bytes per launch of the dominant kernel, from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
-    # profiles/gemm_mfma_f4_bgemm_8192x8192x8192.txt (scaled by the same counters on a 256 MiB device copy)
-    traffic = MEASURED_TRAFFIC_BYTES_C5_FP4 if fp4 else None
+    ok = bool(c5["bit_exact"]) and all(r["bit_exact"] for r in (extra or []))
 
+    roofline = {"bound": "mfma", "achieved": c5["tops"], "peak": peak, "unit": "TFLOP/s", "frac": c5["tops"] / peak,
+                # HBM bytes per launch of this kernel from the FETCH_SIZE / WRITE_SIZE counter runs, as the tracked
+                # profile summary of the same command states them (null when it holds no such line)
+                "traffic": measured_traffic_bytes() if fp4 else None}
+    if peak_measured:
+        mp = peak_measured["fp4_tops" if fp4 else "int8_tops"]
+        roofline["peak_measured"] = mp
+        roofline["frac_of_measured_peak"] = round(c5["tops"] / mp, 4)
     line = {
         "metric": "effective binary TOPS (2*M*N*K/t), bit-exact int32",
-        "value": c5["tops"], "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "value": c5["tops"] if c5["bit_exact"] else None, "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": c5["ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "fp4" if fp4 else "int8",
         "data": "synthetic",
         "config": {"workload": "BASELINE.json config 5: BGEMM M=N=K=8192, {-1,+1}x{-1,+1}, weights and activations "
                                "prepacked (tiled bit layout), int32 output, splitK=%d" % args.split_k,
+                   "kernel": c5["kernel"],
                    "arithmetic": ("1-bit operands expanded in registers to E2M1 (fp4) MFMA operands, fp32 accumulation "
                                   "of exact integers" if fp4 else
                                   "1-bit operands expanded in registers to int8 MFMA operands, int32 accumulation"),
@@ -458,13 +666,16 @@ def main():
                    "bit_exact_sampled": c5["bit_exact"], "hbm_gbs_algorithmic": c5["gbs"],
                    "activation_pack_ms": c5["act_pack_ms"],
                    "frac_of_int8_mfma_peak": c5["tops"] / INT8_MFMA_PEAK_TOPS},
-        "roofline": {"bound": "mfma", "achieved": c5["tops"], "peak": peak, "unit": "TFLOP/s",
-                     "frac": c5["tops"] / peak, "traffic": traffic},
+        "roofline": roofline,
         "cpu_baseline": cpu,
     }
-    if extra:
+    if extra is not None:
         line["all_configs"] = extra
+        line["floor"] = floor
+        line["mfma_peak_measured"] = peak_measured
     print(json.dumps(line), flush=True)
+    if not ok:
+        sys.exit("bench.py: a timed configuration did NOT match its closed form bit for bit (see bit_exact in the line above)")
 
 
 if __name__ == "__main__":

@@ -1,0 +1,123 @@
+// Measurement probes for bench.py (not part of the GEMM library): what the hardware allows the
+// kernels of the library, measured on the GPU the benchmark runs on.
+//   * the cost of launching a kernel that does nothing, and of reading a buffer once (the floor under a
+//     decode-size launch, whose weights are one 5.6 MB read);
+//   * the rate the matrix cores reach on the two MFMA instructions the library issues when nothing else
+//     happens (no memory traffic, no bit expansion): the measured peak beside the datasheet one, following
+//     the protocol of the reference's drivers (lowbit_kernel/csrc/kernel_test.h:10-11: warm-up launches, then
+//     timed launches between two events, which bench.py does around these entry points);
+//   * the same with a number of independent vector-ALU instructions after every MFMA, which is what the
+//     in-register bit expansion costs the matrix-core kernels.
+// Built into libbench_probes.so beside bench.py.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+__global__ void probe_empty_kernel(unsigned* out)
+{
+    if (out == reinterpret_cast<unsigned*>(1)) out[0] = 0;      // never true: nothing is done
+}
+
+// Grid-stride read of n_u4 16-byte words, four loads in flight per thread; the xor of everything
+// read is compared with a value it never takes, so the loads stay and nothing is written.
+__global__ __launch_bounds__(512) void probe_read_kernel(const uint4* __restrict__ src, int64_t n_u4, unsigned* out)
+{
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    unsigned acc = 0;
+    for (; i + 3 * stride < n_u4; i += 4 * stride) {
+        uint4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) v[u] = src[i + u * stride];
+#pragma unroll
+        for (int u = 0; u < 4; u++) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+    }
+    for (; i < n_u4; i += stride) { const uint4 v = src[i]; acc ^= v.x ^ v.y ^ v.z ^ v.w; }
+    if (acc == 0x12345678u && out == reinterpret_cast<unsigned*>(1)) out[0] = acc;
+}
+
+// NACC independent accumulators per wave keep the matrix pipe full; VALU masks of live registers after
+// every MFMA stand in for the bit expansion (their results feed the next round's operands, so they stay).
+template <bool FP4, int NACC, int VALU>
+__global__ __launch_bounds__(256) void probe_mfma_kernel(unsigned* out, const int iters)
+{
+    unsigned m[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) m[i] = threadIdx.x * 2654435761u + i;
+    typename std::conditional<FP4, v16f, v16i>::type acc[NACC];
+#pragma unroll
+    for (int i = 0; i < NACC; i++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) acc[i][v] = 0;
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int i = 0; i < NACC; i++) {
+            if constexpr (FP4) {
+                const v8i a = {(int)(m[0] & 0x22222222u), (int)(m[1] & 0x22222222u), (int)(m[2] & 0x22222222u), (int)(m[3] & 0x22222222u), 0, 0, 0, 0};
+                const v8i b = {(int)(m[4] & 0x22222222u), (int)(m[5] & 0x22222222u), (int)(m[6] & 0x22222222u), (int)(m[7] & 0x22222222u), 0, 0, 0, 0};
+                acc[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[i], 4, 4, 0, 0, 0, 0);
+            } else {
+                const v4i a = {(int)(m[0] & 0x01010101u), (int)(m[1] & 0x01010101u), (int)(m[2] & 0x01010101u), (int)(m[3] & 0x01010101u)};
+                const v4i b = {(int)(m[4] & 0x01010101u), (int)(m[5] & 0x01010101u), (int)(m[6] & 0x01010101u), (int)(m[7] & 0x01010101u)};
+                acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc[i], 0, 0, 0);
+            }
+#pragma unroll
+            for (int u = 0; u < VALU; u++) m[(i * VALU + u) & 7] = (m[(i * VALU + u) & 7] >> 1) ^ (it + u);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    unsigned s = 0;
+#pragma unroll
+    for (int i = 0; i < NACC; i++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) s += (unsigned)acc[i][v];
+    out[(size_t)blockIdx.x * 256 + threadIdx.x] = s;
+}
+
+}  // namespace
+
+// All return 0, -1 for bad arguments, or the hipError_t of the launch.
+extern "C" int bench_probe_empty(int blocks, int threads, void* scratch, void* stream)
+{
+    if (blocks <= 0 || threads <= 0 || threads > 1024) return -1;
+    hipLaunchKernelGGL(probe_empty_kernel, dim3(blocks), dim3(threads), 0, (hipStream_t)stream, (unsigned*)scratch);
+    return (int)hipGetLastError();
+}
+
+extern "C" int bench_probe_read(const void* src, int64_t bytes, int blocks, int threads, void* scratch, void* stream)
+{
+    if (!src || bytes < 16 || blocks <= 0 || threads <= 0 || threads > 512 || ((uintptr_t)src & 15)) return -1;
+    hipLaunchKernelGGL(probe_read_kernel, dim3(blocks), dim3(threads), 0, (hipStream_t)stream, (const uint4*)src,
+                       bytes / 16, (unsigned*)scratch);
+    return (int)hipGetLastError();
+}
+
+// One launch of `blocks` blocks of four waves, each wave issuing iters * 8 MFMAs (fp4 != 0:
+// v_mfma_f32_32x32x64_f8f6f4 with E2M1 operands, 2 * 32 * 32 * 64 ops each; else v_mfma_i32_32x32x32_i8,
+// 2 * 32 * 32 * 32 ops each) with `valu` in {0, 2, 4} vector-ALU instructions after every one.
+// out: blocks * 256 words.
+extern "C" int bench_probe_mfma(int fp4, int valu, int blocks, int iters, void* out, void* stream)
+{
+    if (blocks <= 0 || iters <= 0 || !out) return -1;
+    const dim3 g(blocks), b(256);
+    hipStream_t st = (hipStream_t)stream;
+    unsigned* o = (unsigned*)out;
+    if (fp4) {
+        if (valu == 0) hipLaunchKernelGGL((probe_mfma_kernel<true, 8, 0>), g, b, 0, st, o, iters);
+        else if (valu == 2) hipLaunchKernelGGL((probe_mfma_kernel<true, 8, 2>), g, b, 0, st, o, iters);
+        else if (valu == 4) hipLaunchKernelGGL((probe_mfma_kernel<true, 8, 4>), g, b, 0, st, o, iters);
+        else return -1;
+    } else {
+        if (valu == 0) hipLaunchKernelGGL((probe_mfma_kernel<false, 8, 0>), g, b, 0, st, o, iters);
+        else if (valu == 2) hipLaunchKernelGGL((probe_mfma_kernel<false, 8, 2>), g, b, 0, st, o, iters);
+        else if (valu == 4) hipLaunchKernelGGL((probe_mfma_kernel<false, 8, 4>), g, b, 0, st, o, iters);
+        else return -1;
+    }
+    return (int)hipGetLastError();
+}

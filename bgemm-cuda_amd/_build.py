@@ -7,9 +7,6 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 SO = os.path.join(HERE, "libbgemm_mi355x.so")
 SOURCES = ["api.hip", "pack.hip", "gemm_mfma.hip", "gemm_valu.hip", "gemm_skinny.hip"]
-# measurement probes for bench.py --floor, kept out of the library proper
-MEMBENCH_SO = os.path.join(HERE, "libbgemm_membench.so")
-MEMBENCH_SOURCE = "membench.hip"
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
          # keep the compiler from forming packed-fp32 VALU ops
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
@@ -20,10 +17,9 @@ def build(verbose=True):
     objs = []
     procs = []
     os.makedirs(os.path.join(HERE, "build"), exist_ok=True)
-    for s in SOURCES + [MEMBENCH_SOURCE]:
+    for s in SOURCES:
         o = os.path.join(HERE, "build", s.replace(".hip", ".o"))
-        if s != MEMBENCH_SOURCE:
-            objs.append(o)
+        objs.append(o)
         cmd = [hipcc] + FLAGS + ["-c", os.path.join(CSRC, s), "-o", o]
         if verbose:
             print(" ".join(cmd), flush=True)
@@ -35,12 +31,18 @@ def build(verbose=True):
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)
-    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", MEMBENCH_SO,
-           os.path.join(HERE, "build", MEMBENCH_SOURCE.replace(".hip", ".o"))]
+    return SO
+
+
+def build_probes(root, verbose=True):
+    """bench.py's measurement probes (bench_probes.hip beside it) -> libbench_probes.so, not part of the library."""
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    so = os.path.join(root, "libbench_probes.so")
+    cmd = [hipcc] + FLAGS + ["-shared", "-o", so, os.path.join(root, "bench_probes.hip")]
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)
-    return SO
+    return so
 
 
 if __name__ == "__main__":

@@ -13,15 +13,13 @@
 
 namespace bgemm {
 
-// One all-zero operand tile (never written): K-tiles past a range are read from here.
-__device__ const uint4 g_zero_tile[TILE_U4] = {};
-
 // Block = WGN x WGM waves, each wave owns WN x WM tiles of 32x32 outputs, PL activation planes.
 template <typename Eng, int WGN, int WGM, int WN, int WM, int PL, bool PIPE>
 __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mfma_kernel(const GemmArgs a, const int tiles_n,
                                                                    const int tiles_m)
 {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // the wave index as a scalar: tile coordinates and operand bases stay on the scalar unit
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wn = wave / WGM, wm = wave % WGM;
 
     // logical block id: XCD-contiguous (see xcd_contiguous_id)
@@ -86,21 +84,25 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
         constexpr int NF = WN + WM, ND = NF * 4, NM = WN * WM, STEPS = Eng::STEPS;
         static_assert(ND % NM == 0 && NF <= NM && STEPS % 2 == 0, "tile shape does not pipeline");
         constexpr int DPG = ND / NM;                       // expanded registers produced per MFMA
-        const uint4* fp[NF];
+        // Every fragment's row of K-tiles is a buffer of its own (a wave-uniform base in scalar registers, KT KiB
+        // long), so all loads of a K-tile share ONE per-lane offset, lane * 16 + kt * 1024: no address arithmetic
+        // per load, and K-tiles past the range read as zero bits (a buffer load out of range returns 0; zero bits
+        // add nothing to the dot or the popcounts), so the loop can always run whole pairs of K-tiles.  Buffer
+        // loads also return in order, which lets the compiler wait for the K-tile it needs and no more (flat
+        // loads, as a pointer that may point at a zero tile made them, are waited for down to the last one).
+        __amdgpu_buffer_rsrc_t rs[NF];
 #pragma unroll
-        for (int i = 0; i < WN; i++) fp[i] = xp[0][i];
-#pragma unroll
-        for (int j = 0; j < WM; j++) fp[WN + j] = wp[j];
+        for (int f = 0; f < NF; f++) {
+            const int64_t rt = f < WN ? min(nt0 + f, a.NT - 1) : min(mt0 + (f - WN), a.MT - 1);
+            const uint4* base = (f < WN ? Xb : Wb) + rt * a.KT * TILE_U4;
+            rs[f] = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint4*>(base), 0, a.KT * (TILE_U4 * 16), 0x00020000);
+        }
         unsigned rawA[NF][4], rawB[NF][4], buf[2][NF][4];
         int pop[NF];
 #pragma unroll
         for (int f = 0; f < NF; f++) pop[f] = 0;
-        const int kt_last = kt1 - 1;
-        // K-tiles past the range read as zero bits (which add nothing to the dot or the popcounts),
-        // so the loop can always run whole pairs of K-tiles
         auto load_frag = [&](unsigned (&r)[4], const int f, const int kt) {
-            const uint4* src = kt <= kt_last ? fp[f] + (int64_t)kt * TILE_U4 : g_zero_tile + lane;
-            const uint4 v = *src;
+            const v4i v = __builtin_amdgcn_raw_buffer_load_b128(rs[f], lane * 16 + kt * (TILE_U4 * 16), 0, 0);
             r[0] = v.x; r[1] = v.y; r[2] = v.z; r[3] = v.w;
         };
         auto k_tile = [&](unsigned (&A)[NF][4], unsigned (&B)[NF][4], const int kt) {
@@ -117,7 +119,10 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
                         nxt[d / 4][d % 4] = d / 4 < WN      // fragments 0 .. WN-1 are the activation side
                             ? (s + 1 < STEPS ? Eng::expand1_x(A[d / 4][d % 4], s + 1) : Eng::expand1_x(B[d / 4][d % 4], 0))
                             : (s + 1 < STEPS ? Eng::expand1_w(A[d / 4][d % 4], s + 1) : Eng::expand1_w(B[d / 4][d % 4], 0));
-                    if (s == 0 && q < NF) pop[q] += __popc(A[q][0]) + __popc(A[q][1]) + __popc(A[q][2]) + __popc(A[q][3]);
+                    if (s == 0 && q < NF) {     // v_bcnt adds into its accumulator: four instructions a fragment, written out
+#pragma unroll                                  // because the compiler prefers four counts and two three-way adds
+                        for (int c = 0; c < 4; c++) asm("v_bcnt_u32_b32 %0, %1, %0" : "+v"(pop[q]) : "v"(A[q][c]));
+                    }
                     if (s == STEPS - 1 && q < NF) load_frag(A[q], q, kt + 2);   // A is dead after step STEPS-2
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -272,11 +277,13 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
         // Stores past the caches (non-temporal) where timing favours them: always for the 2-byte kinds, for the
         // 4-byte kinds on outputs of up to 32 MiB (a.nt_store); larger int32 outputs are faster with ordinary stores.
         // (The non-temporal store is written as an instruction: as a builtin next to an ordinary store of the same
-        // value the optimiser merges the two into one ordinary store.)
+        // value the optimiser merges the two into one ordinary store.  The s_nop belongs to it: a store of more
+        // than 64 bits must not be followed at once by a vector-ALU write to its data registers, and the compiler,
+        // which pads that hazard for its own stores, does not look inside an asm statement.)
         auto store16 = [&](char* const to, const int4 v, const bool past_cache) {
             if (past_cache) {
                 const v4i x = {v.x, v.y, v.z, v.w};
-                asm volatile("global_store_dwordx4 %0, %1, off nt" : : "v"(to), "v"(x) : "memory");
+                asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 1" : : "v"(to), "v"(x) : "memory");
             } else
                 *reinterpret_cast<int4*>(to) = v;
         };
