@@ -10,6 +10,7 @@
 // popcounts for the rank-one terms come from the same registers (4 v_bcnt per fragment).
 #include "common.h"
 #include "mfma_engines.h"
+#include <type_traits>
 
 namespace bgemm {
 
@@ -249,6 +250,55 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
         }
     };
 
+    // ---- int32 output: straight from the accumulators ---------------------------------------------
+    // In the accumulator layout of the 32 x 32 MFMA a lane holds one output column (weight row m) of sixteen
+    // output rows, and the lanes of a half-wave hold 32 consecutive columns: one 4-byte store instruction
+    // writes two whole 128-byte lines, one per half-wave, and needs no transposition.  The address is a
+    // wave-uniform base (strip row, weight tile: scalar registers) plus one fixed 32-bit offset per lane.
+    if (a.out_kind == BGEMM_OUT_I32 && a.M < (1 << 28)) {
+        const int64_t row_b = a.M * 4;
+        char* const out_b = reinterpret_cast<char*>(a.out) + (int64_t)b * a.strideC * 4;
+        const uint32_t voff = (uint32_t)(half * 4 * row_b + col * 4);
+        auto rows_out = [&](auto past_cache) {
+#pragma unroll
+            for (int i = 0; i < WN; i++) {
+                const int64_t nrow0 = (int64_t)(nt0 + i) * 32;
+                if (nrow0 >= a.N) break;                          // the whole strip lies past the last row
+                int val[WM][16];
+                tile_row_vals(i, val);
+                auto put = [&](int* const to, const int v) {
+                    if constexpr (decltype(past_cache)::value) __builtin_nontemporal_store(v, to);
+                    else *to = v;
+                };
+                char* const ub = out_b + nrow0 * row_b + (int64_t)mt0 * 128;      // uniform: scalar registers
+                if (nrow0 + 32 <= a.N && (int64_t)(mt0 + WM) * 32 <= a.M) {
+                    // the strip exists as a whole: no test per store, one scalar base per row, the weight tile in
+                    // the instruction's immediate offset (a lone wave on its SIMD issues an instruction every
+                    // 2.3 ns at best, so the epilogue costs what it counts in instructions, scalar ones included)
+#pragma unroll
+                    for (int v = 0; v < 16; v++) {
+                        int* const row = reinterpret_cast<int*>(ub + (8 * (v >> 2) + (v & 3)) * row_b + voff);
+#pragma unroll
+                        for (int j = 0; j < WM; j++) put(row + j * 32, val[j][v]);
+                    }
+                } else {
+#pragma unroll
+                    for (int j = 0; j < WM; j++) {
+                        if ((int64_t)(mt0 + j) * 32 + col >= a.M) continue;
+#pragma unroll
+                        for (int v = 0; v < 16; v++) {
+                            const int r = 8 * (v >> 2) + (v & 3);      // the lane's row is r + 4 * half
+                            if (nrow0 + r + 4 * half < a.N) put(reinterpret_cast<int*>(ub + r * row_b + voff) + j * 32, val[j][v]);
+                        }
+                    }
+                }
+            }
+        };
+        if (a.nt_store) rows_out(std::true_type{});
+        else rows_out(std::false_type{});
+        return;
+    }
+
     // ---- store ------------------------------------------------------------------------------
     // Every 32-row strip of the wave's tile is transposed through the wave's own LDS area, so that
     // lanes own consecutive outputs of one row.  Only the plain int32 case with 16-byte-aligned rows
@@ -452,21 +502,21 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
 // ---- host side ---------------------------------------------------------------------------
 struct MfmaCfg { int id, bn, bm; };
 
-// Tile choice, from timings of each configuration over a sweep of shapes: the 256 x 256 tile (one
-// block per CU, hand-pipelined loop) needs at least two rounds of blocks and a long K (from 32
-// K-tiles) to pay for its long epilogue, during which its CU computes nothing; 256 x 128 (two
-// resident blocks per CU, so one block's stores overlap the other's main loop) wins once both of
-// those blocks exist, from two blocks per CU upwards (from one on a K of 64 K-tiles or more),
-// except on very short K (under 4 K-tiles), where 128 x 128 keeps more waves in flight for what
-// is then all prologue and epilogue; between one and two such blocks per CU 128 x 128 is 5 to 15 %
-// faster (11008 x 768 x 4096: 24.4 against 27.9 us); below that the smaller tiles, down to
-// 32 x 128, are chosen so that every CU gets a block.
+// Tile choice, from timings of every tile over a sweep of shapes (bench.py --only thresholds prints them): the
+// 256 x 256 tile (one block per CU, hand-pipelined loop, the fastest main loop) needs at least two rounds of
+// blocks and a long K (from 32 K-tiles) to pay for its epilogue, during which its CU computes nothing;
+// 256 x 128 (two resident blocks per CU that run half a tile apart, so one block's stores overlap the other's
+// main loop) from one block per CU upwards on 16 K-tiles or more (4096 x 2048 x 4096: 17.2 against 18.5 us on
+// 128 x 128), from two below that, except on very short K (under 4 K-tiles), where 128 x 128 keeps more waves
+// in flight for what is then all prologue and epilogue; below that the smaller tiles, down to 32 x 128, are
+// chosen so that every CU gets a block.  Narrow outputs (M <= 64) take 64-wide tiles: 128 rows from four
+// blocks per CU on, else 64 (192 x [512 x 512] x [512 x 64]: 7.0 against 7.3 us).
 static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int planes)
 {
     auto blocks = [&](int bn, int bm) { return batch * cdiv(N, bn) * cdiv(M, bm); };
-    if (M <= 64) return blocks(128, 64) >= 512 ? MfmaCfg{BGEMM_KERNEL_MFMA_128x64, 128, 64} : MfmaCfg{BGEMM_KERNEL_MFMA_64x64, 64, 64};   // narrow outputs
+    if (M <= 64) return blocks(128, 64) >= 1024 ? MfmaCfg{BGEMM_KERNEL_MFMA_128x64, 128, 64} : MfmaCfg{BGEMM_KERNEL_MFMA_64x64, 64, 64};   // narrow outputs
     if (planes == 1 && blocks(256, 256) >= 512 && KT >= 32) return {BGEMM_KERNEL_MFMA_256x256, 256, 256};
-    if (planes == 1 && blocks(256, 128) >= (KT >= 64 ? 256 : 512) && (KT >= 4 || blocks(128, 128) < 512)) return {BGEMM_KERNEL_MFMA_256x128, 256, 128};
+    if (planes == 1 && blocks(256, 128) >= (KT >= 16 ? 256 : 512) && (KT >= 4 || blocks(128, 128) < 512)) return {BGEMM_KERNEL_MFMA_256x128, 256, 128};
     if (blocks(128, 128) >= 512) return {BGEMM_KERNEL_MFMA_128x128, 128, 128};
     if (blocks(64, 128) >= 512) return {BGEMM_KERNEL_MFMA_64x128, 64, 128};      // below two blocks a unit, twice as many 32-row tiles are faster
     return {BGEMM_KERNEL_MFMA_32x128, 32, 128};

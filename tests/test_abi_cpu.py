@@ -104,7 +104,9 @@ def test_dispatch_of_the_benchmark_configurations():
     assert kid(MODE_XOR, 1, 8192, 2048, 4096, 1, A) == B.KERNEL_MFMA_256x128
     assert kid(MODE_XOR, 1, 8192, 2048, 16384, 4, A) == B.KERNEL_MFMA_256x128
     assert kid(MODE_XOR, 1, 8192, 256, 16384, 1, A) == B.KERNEL_SKINNY_QUAD
-    assert kid(MODE_ATTN_X, 192, 64, 512, 512, 1, A) == B.KERNEL_MFMA_128x64
+    assert kid(MODE_ATTN_X, 192, 64, 512, 512, 1, A) == B.KERNEL_MFMA_64x64
+    assert kid(MODE_ATTN_X, 384, 64, 512, 512, 1, A) == B.KERNEL_MFMA_128x64
+    assert kid(MODE_XOR, 1, 4096, 2048, 4096, 1, A) == B.KERNEL_MFMA_256x128
     assert kid(MODE_ATTN_X, 24, 64, 512, 512, 1, A) == B.KERNEL_MFMA_64x64
     assert kid(MODE_BWTA, 1, 11008, 1, 4096, 8, A) == B.KERNEL_SKINNY_POPC
     assert kid(MODE_BWTA, 1, 11008, 16, 4096, 8, A) == B.KERNEL_SKINNY_SPLITK

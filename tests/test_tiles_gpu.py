@@ -182,8 +182,8 @@ def test_config3_attention_av_all_192_heads():
     want = np.matmul(attn_bits.astype(np.float32), v.astype(np.float32)).astype(np.int32)
     attn16 = to_dev((2 * attn_bits - 1).astype(np.float16))          # "1" must have its sign bit clear
     ap, vp = lk.pack_sign(attn16), lk.pack_sign_transposed(to_dev(v))
-    assert lk.packed_kernel_id(vp, ap, MODE_ATTN_X) == B.KERNEL_MFMA_128x64
-    for variant in (VARIANT_AUTO, VARIANT_MFMA):
+    assert lk.packed_kernel_id(vp, ap, MODE_ATTN_X) == B.KERNEL_MFMA_64x64
+    for variant in (VARIANT_AUTO, VARIANT_MFMA, force_kernel(B.KERNEL_MFMA_128x64)):
         got = lk.bgemm_packed_forward(vp, ap, MODE_ATTN_X, torch.int32, 1, variant).cpu().numpy()
         assert (got == want).all(), variant
         # the reference's orientation (attn as the weight side, INSTR = 2) gives the transpose
@@ -196,7 +196,7 @@ def test_config3_attention_av_all_192_heads():
 def test_narrow_outputs_ragged_batch():
     """The 128 x 64 tile where the library picks it, ragged in every dimension."""
     rng = np.random.default_rng(77)
-    Bn, M, N, K = 200, 50, 300, 700
+    Bn, M, N, K = 350, 50, 300, 700
     w, x = pm1(rng, Bn, M, K), pm1(rng, Bn, N, K)
     wp, xp = lk.pack_sign(to_dev(w)), lk.pack_sign(to_dev(x))
     assert lk.packed_kernel_id(wp, xp, MODE_XOR) == B.KERNEL_MFMA_128x64
