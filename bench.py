@@ -36,7 +36,7 @@ HBM_PEAK_GBS = 8000.0             # MI355X HBM3E, published
 C5_PROFILE = os.path.join(ROOT, "profiles", "gemm_mfma_f4_bgemm_8192x8192x8192.txt")
 PROBES_SO = os.path.join(ROOT, "libbench_probes.so")
 
-KERNEL_NAMES = {0: "mfma 256x256", 1: "mfma 128x128", 2: "mfma 64x128", 3: "mfma 32x128", 4: "mfma 256x128",
+KERNEL_NAMES = {0: "mfma 256x256", 1: "mfma 128x128", 2: "mfma 64x128", 3: "mfma 32x128", 4: "mfma 256x128", 5: "mfma 32x256",
                 6: "mfma 64x64", 7: "mfma 128x64", 16: "decode stream", 17: "decode split-K in the block",
                 18: "decode four pieces a block", 19: "decode AND-popcount (vector ALU)", 32: "VALU popcount GEMM"}
 
@@ -511,7 +511,7 @@ def bench_thresholds(steps=60):
     import _lib as B
     dev = torch.device("cuda:0")
     general = [B.KERNEL_MFMA_256x256, B.KERNEL_MFMA_256x128, B.KERNEL_MFMA_128x128, B.KERNEL_MFMA_64x128, B.KERNEL_MFMA_32x128,
-               B.KERNEL_MFMA_128x64, B.KERNEL_MFMA_64x64]
+               B.KERNEL_MFMA_32x256, B.KERNEL_MFMA_128x64, B.KERNEL_MFMA_64x64]
     rows = []
     for planes, batch, M, N, K in THRESHOLD_SHAPES:
         mode = lk.MODE_BWTA if planes == 2 else lk.MODE_XOR

@@ -284,7 +284,7 @@ int pack_sign_pair(const void* srcA, int64_t rowsA, void* dstA, const void* srcB
 
 // Kernel families (each in its own translation unit).
 int launch_gemm_mfma(const GemmArgs& a, hipStream_t st, bool fp4);
-int gemm_mfma_kernel_id(int64_t batch, int64_t M, int64_t N, int64_t KT, int planes);     // BGEMM_KERNEL_MFMA_* by shape
+int gemm_mfma_kernel_id(int64_t batch, int64_t M, int64_t N, int64_t KT, int planes, int out_shift);     // BGEMM_KERNEL_MFMA_* by shape
 int gemm_skinny_kernel_id(const GemmArgs& a, bool fp4);                                   // BGEMM_KERNEL_SKINNY_* by shape
 int launch_gemm_valu(const GemmArgs& a, hipStream_t st);
 // Skinny shapes (few activation rows): K is split inside the block, no workspace.

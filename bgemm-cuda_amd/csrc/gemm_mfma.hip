@@ -32,16 +32,24 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
     const int band_id = tile_id / (band * tiles_m), in_band = tile_id % (band * tiles_m);
     const int band_n0 = band_id * band;
     const int band_h = min(band, tiles_n - band_n0);
-    const int tn = band_n0 + in_band % band_h, tm = in_band / band_h;
+    const int tn_block = band_n0 + in_band % band_h, tm = in_band / band_h;
 
     // K is never split across blocks here: outputs of so few tiles that a K split would pay go to the kernel
     // that splits K among the waves of a block (gemm_skinny_shape)
     const int kt0 = 0, kt1 = a.KT;
 
-    const int nt0 = (tn * WGN + wn) * WN, mt0 = (tm * WGM + wm) * WM;
+    const int mt0 = (tm * WGM + wm) * WM;
     const uint4* Wb = a.W + (int64_t)b * a.strideW;
     const uint4* Xb = a.X + (int64_t)b * a.strideX;
     const uint4* X2b = PL == 2 ? a.X2 + (int64_t)b * a.strideX : nullptr;
+    constexpr int ROW_I = WM * 32 + 8;       // staged row stride in ints (+8 keeps the two lane halves on
+                                             // different LDS banks)
+    __shared__ __align__(16) int rowp[WGN * WGM * WN * 32];
+    __shared__ __align__(16) int stage[WGN * WGM * 32 * ROW_I];
+    // The tile's work is a function object of its own: written straight into the kernel body the same code came
+    // out with 10 to 25 % more registers (113 against 89 for the 64 x 128 tile: three waves a SIMD instead of four).
+  auto do_tile = [&](const int tn) {
+    const int nt0 = (tn * WGN + wn) * WN;
 
     // per-fragment base pointers (row tile clamped so ragged edges re-read a valid tile)
     const uint4* xp[PL][WN];
@@ -217,7 +225,6 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
     // All LDS traffic of the epilogue is private to the wave: LDS executes one wave's accesses in
     // order, so compiler-level wave fences are all the synchronisation it needs, and the waves of a
     // block drift apart freely (one computes a strip while another's stores drain).
-    __shared__ __align__(16) int rowp[WGN * WGM * WN * 32];
     int* const rp = rowp + wave * (WN * 32);
     auto wave_sync = [] {
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -304,14 +311,56 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
     // lanes own consecutive outputs of one row.  Only the plain int32 case with 16-byte-aligned rows
     // is unrolled; the conversions of the other output kinds sit in rolled loops after the staging,
     // which keeps them out of the fully unrolled part of the kernel.
-    constexpr int ROW_I = WM * 32 + 8;       // staged row stride in ints (+8 keeps the two lane halves on
-                                             // different LDS banks)
-    __shared__ __align__(16) int stage[WGN * WGM * 32 * ROW_I];
     const int esz_shift = out_elem_shift(a.out_kind);
     const int64_t out_off = (int64_t)b * a.strideC;
     char* const out_base = reinterpret_cast<char*>(a.out) + (out_off << esz_shift);
     const int64_t row_bytes = a.M << esz_shift;
     int* const st = stage + wave * (32 * ROW_I);
+    // Stores past the caches (non-temporal) where timing favours them: always for the 2-byte kinds, for the
+    // 4-byte kinds on outputs of up to 32 MiB (a.nt_store); larger int32 outputs are faster with ordinary stores.
+    // (The non-temporal store is written as an instruction: as a builtin next to an ordinary store of the same
+    // value the optimiser merges the two into one ordinary store.  The s_nop belongs to it: a store of more
+    // than 64 bits must not be followed at once by a vector-ALU write to its data registers, and the compiler,
+    // which pads that hazard for its own stores, does not look inside an asm statement.)
+    auto store16 = [&](char* const to, const int4 v, const bool past_cache) {
+        if (past_cache) {
+            const v4i x = {v.x, v.y, v.z, v.w};
+            asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 1" : : "v"(to), "v"(x) : "memory");
+        } else
+            *reinterpret_cast<int4*>(to) = v;
+    };
+    // Plain fp16 with rows a multiple of eight long: the integers are rounded once, staged as halves, and a
+    // lane reads back the eight it stores with one 16-byte LDS read (no conversion behind the staging).
+    if (a.out_kind == BGEMM_OUT_F16 && a.vec_store == 8) {
+        constexpr int ROW_H = WM * 32 + 8;       // staged row stride in halves (+8: rows four apart, the two
+                                                 // lane halves, fall on different LDS banks)
+        constexpr int C8 = WM * 4, RSTEP = 64 / C8;              // lanes per staged row, rows per store instruction
+        __half* const sh = reinterpret_cast<__half*>(st);
+        const int c8 = lane % C8, row0 = lane / C8;
+        const int64_t m = (int64_t)mt0 * 32 + c8 * 8;
+#pragma unroll
+        for (int i = 0; i < WN; i++) {
+            const int64_t nrow0 = (int64_t)(nt0 + i) * 32;
+            if (nrow0 >= a.N) break;                              // the whole strip lies past the last row
+            int val[WM][16];
+            tile_row_vals(i, val);
+#pragma unroll
+            for (int v = 0; v < 16; v++)
+#pragma unroll
+                for (int j = 0; j < WM; j++)
+                    sh[(8 * (v >> 2) + 4 * half + (v & 3)) * ROW_H + j * 32 + col] = __float2half_rn((float)val[j][v]);
+            wave_sync();
+            if (m < a.M) {
+                char* dst = out_base + (nrow0 + row0) * row_bytes + (m << 1);
+                const __half* sp = sh + row0 * ROW_H + c8 * 8;
+#pragma unroll
+                for (int row = row0; row < 32; row += RSTEP, sp += RSTEP * ROW_H, dst += RSTEP * row_bytes)
+                    if (nrow0 + row < a.N) store16(dst, *reinterpret_cast<const int4*>(sp), true);
+            }
+            wave_sync();                                 // the next strip overwrites the staging area
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < WN; i++) {
         int val[WM][16];
@@ -324,19 +373,6 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
         const int64_t nrow0 = (int64_t)(nt0 + i) * 32, mcol0 = (int64_t)mt0 * 32;
         constexpr int C4 = WM * 8;               // int4 per staged row
         constexpr int NP = 32 * C4 / 64;
-        // Stores past the caches (non-temporal) where timing favours them: always for the 2-byte kinds, for the
-        // 4-byte kinds on outputs of up to 32 MiB (a.nt_store); larger int32 outputs are faster with ordinary stores.
-        // (The non-temporal store is written as an instruction: as a builtin next to an ordinary store of the same
-        // value the optimiser merges the two into one ordinary store.  The s_nop belongs to it: a store of more
-        // than 64 bits must not be followed at once by a vector-ALU write to its data registers, and the compiler,
-        // which pads that hazard for its own stores, does not look inside an asm statement.)
-        auto store16 = [&](char* const to, const int4 v, const bool past_cache) {
-            if (past_cache) {
-                const v4i x = {v.x, v.y, v.z, v.w};
-                asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 1" : : "v"(to), "v"(x) : "memory");
-            } else
-                *reinterpret_cast<int4*>(to) = v;
-        };
         if (a.vec_store && a.out_kind == BGEMM_OUT_I32) {
             // 16-byte stores: one instruction covers 64 * 4 consecutive elements of the strip.  Eight
             // LDS reads are issued together, then their stores; the address advances by whole rows.
@@ -497,6 +533,8 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
         }
         wave_sync();                                 // the next strip overwrites the staging area
     }
+  };
+    do_tile(tn_block);
 }
 
 // ---- host side ---------------------------------------------------------------------------
@@ -511,10 +549,13 @@ struct MfmaCfg { int id, bn, bm; };
 // in flight for what is then all prologue and epilogue; below that the smaller tiles, down to 32 x 128, are
 // chosen so that every CU gets a block.  Narrow outputs (M <= 64) take 64-wide tiles: 128 rows from four
 // blocks per CU on, else 64 (192 x [512 x 512] x [512 x 64]: 7.0 against 7.3 us).
-static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int planes)
+static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int planes, int out_shift)
 {
     auto blocks = [&](int bn, int bm) { return batch * cdiv(N, bn) * cdiv(M, bm); };
     if (M <= 64) return blocks(128, 64) >= 1024 ? MfmaCfg{BGEMM_KERNEL_MFMA_128x64, 128, 64} : MfmaCfg{BGEMM_KERNEL_MFMA_64x64, 64, 64};   // narrow outputs
+    // a short K with a 2-byte output is all store path: rows of 512 bytes per block, many blocks in flight
+    // (192 x [512 x 512] x 64 -> fp16: 23.3 us against 25.0 to 28 on the other tiles; int32 output shows no preference)
+    if (KT < 4 && out_shift == 1 && M >= 256 && blocks(32, 256) >= 512) return {BGEMM_KERNEL_MFMA_32x256, 32, 256};
     if (planes == 1 && blocks(256, 256) >= 512 && KT >= 32) return {BGEMM_KERNEL_MFMA_256x256, 256, 256};
     if (planes == 1 && blocks(256, 128) >= (KT >= 16 ? 256 : 512) && (KT >= 4 || blocks(128, 128) < 512)) return {BGEMM_KERNEL_MFMA_256x128, 256, 128};
     if (blocks(128, 128) >= 512) return {BGEMM_KERNEL_MFMA_128x128, 128, 128};
@@ -542,15 +583,15 @@ static int launch_cfg(const GemmArgs& a, hipStream_t st)
     return check_launch("gemm_mfma");
 }
 
-int gemm_mfma_kernel_id(int64_t batch, int64_t M, int64_t N, int64_t KT, int planes)
+int gemm_mfma_kernel_id(int64_t batch, int64_t M, int64_t N, int64_t KT, int planes, int out_shift)
 {
-    return pick_cfg(batch, M, N, KT, planes).id;
+    return pick_cfg(batch, M, N, KT, planes, out_shift).id;
 }
 
 template <typename Eng>
 static int launch_eng(const GemmArgs& a, hipStream_t st)
 {
-    const int id = a.force >= 0 ? a.force : pick_cfg(a.batch, a.M, a.N, a.KT, a.mc.planes).id;
+    const int id = a.force >= 0 ? a.force : pick_cfg(a.batch, a.M, a.N, a.KT, a.mc.planes, out_elem_shift(a.out_kind)).id;
     switch (id) {
     case BGEMM_KERNEL_MFMA_256x256: return launch_cfg<Eng, 2, 2, 4, 4>(a, st);
     case BGEMM_KERNEL_MFMA_256x128: return launch_cfg<Eng, 2, 2, 4, 2>(a, st);    // two blocks per CU
@@ -559,6 +600,7 @@ static int launch_eng(const GemmArgs& a, hipStream_t st)
     case BGEMM_KERNEL_MFMA_128x128: return launch_cfg<Eng, 2, 2, 2, 2>(a, st);
     case BGEMM_KERNEL_MFMA_64x128: return launch_cfg<Eng, 1, 4, 2, 1>(a, st);
     case BGEMM_KERNEL_MFMA_32x128: return launch_cfg<Eng, 1, 4, 1, 1>(a, st);
+    case BGEMM_KERNEL_MFMA_32x256: return launch_cfg<Eng, 1, 4, 1, 2>(a, st);
     default: return fail(BGEMM_EINVAL, "gemm_mfma: no kernel %d", id);
     }
 }

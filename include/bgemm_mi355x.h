@@ -53,7 +53,8 @@ enum { BGEMM_VARIANT_AUTO = 0, BGEMM_VARIANT_VALU = 1, BGEMM_VARIANT_MFMA = 2, B
 /* The kernels behind bgemm_packed_forward*, as bgemm_packed_kernel_id() names them: the general matrix-core
  * kernel by its block tile (activation rows x weight rows), the decode-shaped kernels, the VALU kernel. */
 enum { BGEMM_KERNEL_MFMA_256x256 = 0, BGEMM_KERNEL_MFMA_128x128 = 1, BGEMM_KERNEL_MFMA_64x128 = 2,
-       BGEMM_KERNEL_MFMA_32x128 = 3, BGEMM_KERNEL_MFMA_256x128 = 4, BGEMM_KERNEL_MFMA_64x64 = 6,
+       BGEMM_KERNEL_MFMA_32x128 = 3, BGEMM_KERNEL_MFMA_256x128 = 4, BGEMM_KERNEL_MFMA_32x256 = 5,
+       BGEMM_KERNEL_MFMA_64x64 = 6,
        BGEMM_KERNEL_MFMA_128x64 = 7,
        BGEMM_KERNEL_SKINNY_STREAM = 16, BGEMM_KERNEL_SKINNY_SPLITK = 17, BGEMM_KERNEL_SKINNY_QUAD = 18,
        BGEMM_KERNEL_SKINNY_POPC = 19,

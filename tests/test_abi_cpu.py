@@ -56,7 +56,7 @@ def test_layout_sizes():
     (dict(mode=7), _lib.EINVAL),
     (dict(out_dtype=5), _lib.EINVAL),
     (dict(variant=4), _lib.EINVAL),
-    (dict(variant=_lib.force_kernel(5)), _lib.EINVAL),                                   # no such kernel
+    (dict(variant=_lib.force_kernel(8)), _lib.EINVAL),                                   # no such kernel
     (dict(variant=_lib.force_kernel(_lib.KERNEL_MFMA_64x64, _lib.VARIANT_VALU)), _lib.EINVAL),   # the VALU design has one kernel
     (dict(variant=_lib.force_kernel(_lib.KERNEL_SKINNY_STREAM), batch=70000, strideC=64 * 256), _lib.EINVAL),
     (dict(M=-1), _lib.EINVAL),
@@ -98,7 +98,7 @@ def test_dispatch_of_the_benchmark_configurations():
     kid = B.lib().bgemm_packed_kernel_id
     MODE_XOR, MODE_BWTA, MODE_ATTN_X, VARIANT_AUTO, VARIANT_VALU, force_kernel = (
         B.MODE_XOR, B.MODE_BWTA, B.MODE_ATTN_X, B.VARIANT_AUTO, B.VARIANT_VALU, B.force_kernel)
-    TILES = (0, 1, 2, 3, 4, 6, 7)
+    TILES = (0, 1, 2, 3, 4, 5, 6, 7)
     A = VARIANT_AUTO
     assert kid(MODE_XOR, 1, 8192, 8192, 8192, 1, A) == B.KERNEL_MFMA_256x256
     assert kid(MODE_XOR, 1, 8192, 2048, 4096, 1, A) == B.KERNEL_MFMA_256x128
@@ -114,7 +114,7 @@ def test_dispatch_of_the_benchmark_configurations():
     assert kid(MODE_XOR, 1, 4096, 128, 4096, 1, VARIANT_VALU) == B.KERNEL_VALU
     assert kid(MODE_XOR, 70000, 40, 8, 300, 1, A) in TILES        # a batch beyond the decode kernels' grid
     assert kid(MODE_XOR, 1, 64, 64, 64, 1, force_kernel(B.KERNEL_MFMA_256x256)) == B.KERNEL_MFMA_256x256
-    assert kid(MODE_XOR, 1, 64, 64, 64, 1, force_kernel(5)) == B.EINVAL    # no such kernel
+    assert kid(MODE_XOR, 1, 64, 64, 64, 1, force_kernel(8)) == B.EINVAL    # no such kernel
     assert kid(MODE_XOR, 1, 64, 64, 64, 1, force_kernel(B.KERNEL_MFMA_64x64, VARIANT_VALU)) == B.EINVAL
     assert kid(9, 1, 64, 64, 64, 1, A) == B.EINVAL and kid(MODE_XOR, 1, 64, 0, 64, 1, A) == B.EINVAL
 

@@ -20,7 +20,7 @@ from _lib import (MODE_AND, MODE_XOR, MODE_ATTN, MODE_BWTA, MODE_ATTN_X, VARIANT
 
 DEV = "cuda:0"
 TILES = {"256x256": B.KERNEL_MFMA_256x256, "256x128": B.KERNEL_MFMA_256x128, "128x128": B.KERNEL_MFMA_128x128,
-         "64x128": B.KERNEL_MFMA_64x128, "32x128": B.KERNEL_MFMA_32x128, "128x64": B.KERNEL_MFMA_128x64,
+         "64x128": B.KERNEL_MFMA_64x128, "32x128": B.KERNEL_MFMA_32x128, "32x256": B.KERNEL_MFMA_32x256, "128x64": B.KERNEL_MFMA_128x64,
          "64x64": B.KERNEL_MFMA_64x64}
 ENGINES = {"fp4": VARIANT_MFMA_F4, "int8": VARIANT_MFMA}
 
