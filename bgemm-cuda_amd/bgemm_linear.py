@@ -255,9 +255,32 @@ class _ScaledBinaryLinear(nn.Linear):
             out += self.bias.view(1, -1).expand_as(out)
         return out
 
+    # The inference paths keep the weight's packed bits, keyed on the weight tensor's version counter, storage and
+    # type.  The counter only sees writes made through the tensor itself: an update through ``weight.data``
+    # (``p.data.copy_(...)``, ``p.data.clamp_()``, as some BNN training loops do) leaves it unchanged.  The cache is
+    # therefore also dropped whenever the module changes mode (train() / eval()) or loads a state dict, and
+    # invalidate_packed_weight() drops it by hand after such a write.
+    def invalidate_packed_weight(self):
+        """Forget the cached packed weight: the next inference forward packs the float weight again."""
+        self.__dict__.pop("_wp", None)
+        self.__dict__.pop("_wp_key", None)
+
+    def train(self, mode=True):
+        self.invalidate_packed_weight()
+        return super().train(mode)
+
+    def _load_from_state_dict(self, *args, **kwargs):
+        self.invalidate_packed_weight()
+        return super()._load_from_state_dict(*args, **kwargs)
+
 
 class BGEMMLinear(_ScaledBinaryLinear):
-    """out = bgemm(x - zpa, w - zpw) * sw * sa (+ bias)  (bgemm_linear.py:460-486)."""
+    """out = bgemm(x - zpa, w - zpw) * sw * sa (+ bias)  (bgemm_linear.py:460-486).
+
+    Under ``torch.no_grad()`` the forward is fused (``fuse_inference``) and multiplies with a cached packed copy of
+    the weight.  The cache follows every update made through the parameter (optimizer steps, ``copy_``, ``+=``) and is
+    dropped by ``train()`` / ``eval()`` and ``load_state_dict``; after a write through ``weight.data`` call
+    ``invalidate_packed_weight()``."""
     _fn = bgemm_linear
     fuse_inference = True
 

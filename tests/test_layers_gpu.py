@@ -326,3 +326,31 @@ def test_config2_mlp_forward_bitwise(oracle):
         assert torch.equal(acc_gpu.cpu(), acc_cpu)
         assert torch.equal(h_gpu.cpu(), h_cpu)
     assert tuple(h_gpu.shape) == (128, 10)
+
+
+@pytest.mark.parametrize("cls", [bl.BGEMMLinear, bl.BGEMMLinear_elastic_signed])
+def test_packed_weight_cache_follows_the_parameter_and_can_be_dropped(cls):
+    """Updates through the parameter are seen (version counter); a write through ``.data`` is not, and train() /
+    eval(), load_state_dict and invalidate_packed_weight() drop the cached bits."""
+    torch.manual_seed(11)
+    lin = cls(256, 64).to(DEV)
+    x = torch.randn(8, 256, device=DEV)
+    lin(x)                                           # initialises the scales
+    with torch.no_grad():
+        y0 = lin(x).clone()
+        lin.weight.neg_()                            # through the parameter: the cache follows
+        y1 = lin(x).clone()
+        lin.weight.data.neg_()                       # behind the version counter: stale bits until told
+        stale = lin(x).clone()
+        lin.invalidate_packed_weight()
+        y2 = lin(x).clone()
+    assert not torch.equal(y0, y1) and torch.equal(stale, y1) and torch.equal(y2, y0)
+    with torch.no_grad():
+        lin.weight.data.neg_()
+        lin.eval()                                   # a change of mode drops the cache as well
+        assert torch.equal(lin(x), y1)
+        sd = {k: v.clone() for k, v in lin.state_dict().items()}
+        sd["weight"] = -sd["weight"]
+        lin.weight.data.mul_(3.0)                    # (same signs: the bits would not change)
+        lin.load_state_dict(sd)
+        assert torch.equal(lin(x), y0)
