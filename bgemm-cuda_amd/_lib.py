@@ -13,7 +13,8 @@ OK, EINVAL, ENULL, EWORKSPACE, ELAUNCH, EALIGN = 0, -1, -2, -3, -4, -5
 MODE_AND, MODE_XOR, MODE_ATTN, MODE_BWTA, MODE_ATTN_X = 0, 1, 2, 3, 4
 OUT_I32, OUT_F16, OUT_F32_SCALED, OUT_F16_SCALED, OUT_BITS_F32, OUT_BITS_F16 = 0, 1, 2, 3, 4, 5
 SRC_F16, SRC_F32 = 0, 1
-ABI_VERSION = 7
+ABI_VERSION = 8
+LAYOUT_VERSION = 6     # of the tiled operand layout, written into packed files; changes only when the layout does
 STATIC_SCRATCH_BYTES = 32 << 20      # BGEMM_STATIC_SCRATCH_BYTES
 VARIANT_AUTO, VARIANT_VALU, VARIANT_MFMA, VARIANT_MFMA_F4 = 0, 1, 2, 3
 # BGEMM_KERNEL_*: what bgemm_packed_kernel_id() returns and force_kernel() takes
@@ -44,7 +45,7 @@ SIGNATURES = {
     "bgemm_packed_counter_bytes": (_sz, [_int, _i64, _i64, _i64, _i64, _int, _int]),
     "bgemm_packed_forward": (_int, [_int, _p, _p, _p, _p, _int, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
                                     _int, _int, _p, _sz, _p, _sz, _p]),
-    "bgemm_packed_kernel_id": (_int, [_int, _i64, _i64, _i64, _i64, _int, _int]),
+    "bgemm_packed_kernel_id": (_int, [_int, _int, _i64, _i64, _i64, _i64, _int, _int]),
     "bgemm_packed_forward_scaled": (_int, [_int, _p, _p, _p, _p, _int, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
                                            _int, _int, _p, _sz, _p, _sz, _p, _p, _p, _p]),
     "bgemm_packed_forward_bits": (_int, [_int, _p, _p, _p, _p, _int, _i64, _i64, _i64, _i64, _i64, _i64, _i64,

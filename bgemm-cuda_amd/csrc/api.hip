@@ -71,7 +71,7 @@ __global__ void clear_counters_kernel(uint32_t* c, int64_t n)
 using namespace bgemm;
 
 extern "C" const char* bgemm_last_error(void) { return g_err; }
-extern "C" int bgemm_abi_version(void) { return 7; }
+extern "C" int bgemm_abi_version(void) { return 8; }
 
 static bool ws_query(int mode, int64_t batch, int64_t M, int64_t N, int64_t K, int splitK, int variant,
                      size_t* part, size_t* counters)
@@ -241,13 +241,14 @@ static int packed_forward(int mode, const void* W_tiled, const void* X_tiled, co
     return launch_gemm_mfma(a, (hipStream_t)stream, fp4);
 }
 
-extern "C" int bgemm_packed_kernel_id(int mode, int64_t batch, int64_t M, int64_t N, int64_t K, int splitK, int variant)
+extern "C" int bgemm_packed_kernel_id(int mode, int out_dtype, int64_t batch, int64_t M, int64_t N, int64_t K, int splitK,
+                                      int variant)
 {
     // the same checks and the same choice as a call, with stand-in pointers that are never dereferenced
     // and a workspace that is never too small
     alignas(16) static char stand_in[16];
-    return packed_forward(mode, stand_in, stand_in, stand_in, stand_in, BGEMM_OUT_I32, batch, M, N, K, 0, 0, M * N,
-                          splitK, variant, stand_in, (size_t)-1, stand_in, (size_t)-1, nullptr, nullptr, nullptr, nullptr,
+    return packed_forward(mode, stand_in, stand_in, stand_in, stand_in, out_dtype, batch, M, N, K, 0, 0, M * N,
+                          splitK, variant, stand_in, (size_t)-1, stand_in, (size_t)-1, stand_in, stand_in, nullptr, nullptr,
                           nullptr, nullptr, true);
 }
 

@@ -122,9 +122,11 @@ def _check_packed(p, name):
             raise ValueError("%s: both planes must live on one device" % name)
 
 
-def packed_kernel_id(w, x, mode=MODE_XOR, splitK=1, variant=VARIANT_AUTO):
-    """The kernel (``_lib.KERNEL_*``) that ``bgemm_packed_forward(w, x, mode, ..., splitK, variant)`` runs."""
-    rc = _b.lib().bgemm_packed_kernel_id(mode, max(w.batch, x.batch), w.rows, x.rows, w.K, splitK, variant)
+def packed_kernel_id(w, x, mode=MODE_XOR, splitK=1, variant=VARIANT_AUTO, out_dtype=torch.int32):
+    """The kernel (``_lib.KERNEL_*``) that ``bgemm_packed_forward(w, x, mode, out_dtype, splitK, variant)`` runs
+    (2-byte and 4-byte outputs can take different tiles)."""
+    kind = OUT_F16 if out_dtype == torch.half else OUT_I32
+    rc = _b.lib().bgemm_packed_kernel_id(mode, kind, max(w.batch, x.batch), w.rows, x.rows, w.K, splitK, variant)
     if rc < 0:
         _b.check(rc)
     return rc
@@ -492,15 +494,15 @@ def bgemm_linear_forward_cuda(in_feats, weights, splitK=1, INSTR=1):
 # ---- prepacked operands on disk -----------------------------------------------------------------
 # The reference has no binary prepack format (its TODO list asks for one, README.md:25-33).  A file is
 # a 64-byte little-endian header followed by the tiled words of plane 0 and, for ternary operands,
-# plane 1: magic "BGEMMPK1", layout version (= the library's ABI version, which changes with the tiled
-# layout), planes, batch, rows, K, words per matrix.
+# plane 1: magic "BGEMMPK1", version of the tiled layout (_lib.LAYOUT_VERSION, which changes only when the
+# layout does, not with the C ABI), planes, batch, rows, K, words per matrix.
 _PK_MAGIC = b"BGEMMPK1"
 _PK_HEADER = struct.Struct("<8sIIqqqq16x")
 
 
 def save_packed(path, packed):
     """Writes a PackedBits (e.g. prepacked weights) to `path`."""
-    head = _PK_HEADER.pack(_PK_MAGIC, _b.ABI_VERSION, 2 if packed.ternary else 1, packed.batch, packed.rows,
+    head = _PK_HEADER.pack(_PK_MAGIC, _b.LAYOUT_VERSION, 2 if packed.ternary else 1, packed.batch, packed.rows,
                            packed.K, packed.words)
     with open(path, "wb") as f:
         f.write(head)
@@ -518,9 +520,9 @@ def read_packed_header(path):
     magic, version, planes, batch, rows, K, words = _PK_HEADER.unpack(raw)
     if magic != _PK_MAGIC:
         raise ValueError("%s: not a packed-operand file" % path)
-    if version != _b.ABI_VERSION:
+    if version != _b.LAYOUT_VERSION:
         raise ValueError("%s: tiled layout version %d, this library reads %d: pack the weights again" %
-                         (path, version, _b.ABI_VERSION))
+                         (path, version, _b.LAYOUT_VERSION))
     if planes not in (1, 2) or batch < 1 or rows < 1 or K < 1 or words != ((rows + 31) // 32) * ((K + 255) // 256) * 256:
         raise ValueError("%s: inconsistent header" % path)
     return planes, batch, rows, K, words

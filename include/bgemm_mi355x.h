@@ -173,11 +173,13 @@ int bgemm_packed_forward(int mode, const void* W_tiled, const void* X_tiled, con
                          int64_t strideW, int64_t strideX, int64_t strideC,
                          int splitK, int variant, void* ws, size_t ws_bytes,
                          void* counters, size_t counter_bytes, void* stream);
-/* The kernel (BGEMM_KERNEL_*) the three bgemm_packed_forward* entry points run for these arguments, or a
- * negative BGEMM_E* code for arguments they would reject.  The reference's dispatch is the N-bucket switch
+/* The kernel (BGEMM_KERNEL_*) the three bgemm_packed_forward* entry points run for these arguments (out_dtype:
+ * any BGEMM_OUT_* kind; 2-byte and 4-byte outputs can take different tiles), or a negative BGEMM_E* code for
+ * arguments they would reject.  The reference's dispatch is the N-bucket switch
  * of bin_pack_linear_kernel (fp6_linear.cu:292-330), which lands on one tile for every shape; here the
  * choice depends on the shape, and tests and benchmarks ask which kernel they are looking at. */
-int bgemm_packed_kernel_id(int mode, int64_t batch, int64_t M, int64_t N, int64_t K, int splitK, int variant);
+int bgemm_packed_kernel_id(int mode, int out_dtype, int64_t batch, int64_t M, int64_t N, int64_t K, int splitK,
+                           int variant);
 
 /* The same GEMM with the binary Linear's output scaling fused into the store, replacing the
  * separate elementwise kernels of `bgemm(...) * sw * sa (+ bias)`

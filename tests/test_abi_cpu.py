@@ -29,7 +29,7 @@ def test_header_symbols_exported():
 
 def test_layout_sizes():
     L = _lib.lib()
-    assert L.bgemm_abi_version() == _lib.ABI_VERSION == 7
+    assert L.bgemm_abi_version() == _lib.ABI_VERSION == 8
     assert L.bgemm_tiled_words(1, 1) == 256
     assert L.bgemm_tiled_words(32, 256) == 256
     assert L.bgemm_tiled_words(33, 257) == 4 * 256
@@ -95,7 +95,7 @@ def test_dispatch_of_the_benchmark_configurations():
     """Which kernel each benchmark configuration runs (what the profiles and the bench lines are about):
     the query is host code and needs no GPU."""
     B = _lib
-    kid = B.lib().bgemm_packed_kernel_id
+    kid = lambda mode, *rest: B.lib().bgemm_packed_kernel_id(mode, B.OUT_I32, *rest)
     MODE_XOR, MODE_BWTA, MODE_ATTN_X, VARIANT_AUTO, VARIANT_VALU, force_kernel = (
         B.MODE_XOR, B.MODE_BWTA, B.MODE_ATTN_X, B.VARIANT_AUTO, B.VARIANT_VALU, B.force_kernel)
     TILES = (0, 1, 2, 3, 4, 5, 6, 7)
@@ -107,6 +107,9 @@ def test_dispatch_of_the_benchmark_configurations():
     assert kid(MODE_ATTN_X, 192, 64, 512, 512, 1, A) == B.KERNEL_MFMA_64x64
     assert kid(MODE_ATTN_X, 384, 64, 512, 512, 1, A) == B.KERNEL_MFMA_128x64
     assert kid(MODE_XOR, 1, 4096, 2048, 4096, 1, A) == B.KERNEL_MFMA_256x128
+    # a short K with a 2-byte output takes the tile with 512-byte rows
+    assert B.lib().bgemm_packed_kernel_id(MODE_XOR, B.OUT_F16, 192, 512, 512, 64, 1, A) == B.KERNEL_MFMA_32x256
+    assert kid(MODE_XOR, 192, 512, 512, 64, 1, A) == B.KERNEL_MFMA_128x128
     assert kid(MODE_ATTN_X, 24, 64, 512, 512, 1, A) == B.KERNEL_MFMA_64x64
     assert kid(MODE_BWTA, 1, 11008, 1, 4096, 8, A) == B.KERNEL_SKINNY_POPC
     assert kid(MODE_BWTA, 1, 11008, 16, 4096, 8, A) == B.KERNEL_SKINNY_SPLITK
