@@ -37,12 +37,10 @@ SCALE_PARAMS = ('sw', 'sa', 'zpw', 'zpa')
 
 
 def seed_all(seed=1029):
-    random.seed(seed)
+    """Same seed for every generator the demo draws from (the reference's default, test_model_demo.py:19-27)."""
     os.environ['PYTHONHASHSEED'] = str(seed)
-    np.random.seed(seed)
-    torch.manual_seed(seed)
-    if torch.cuda.is_available():
-        torch.cuda.manual_seed_all(seed)
+    for set_seed in (random.seed, np.random.seed, torch.manual_seed):
+        set_seed(seed)                    # torch.manual_seed also seeds every GPU's generator
 
 
 def synthetic_dataset(samples, features=512, seed=0):
@@ -67,22 +65,23 @@ class FC_half2float(nn.Linear):
 
 
 class MLP(nn.Module):
+    """Three stages of (linear, batch norm, dropout, ReLU) and a float head.  Only the first stage's linear is
+    always full precision; `Linear` picks the kind of the other two.  Attribute names are the reference's
+    (lin1..3, bn1..3, fc), so its state dicts load."""
+
     def __init__(self, Linear=BGEMMLinear, dtype=torch.half, bias=True,
                  input_size=512, hidden1=128, hidden2=128, hidden3=128, num_classes=1):
         super().__init__()
-        self.lin1 = nn.Linear(input_size, hidden1, bias=bias)
-        self.lin2 = Linear(hidden1, hidden2, bias=bias)
-        self.lin3 = Linear(hidden2, hidden3, bias=bias)
-        self.relu = nn.ReLU()
-        self.dropout = nn.Dropout(0.5)
-        self.bn1 = nn.BatchNorm1d(hidden1)
-        self.bn2 = nn.BatchNorm1d(hidden2)
-        self.bn3 = nn.BatchNorm1d(hidden3)
+        widths = (input_size, hidden1, hidden2, hidden3)
+        for stage, kind in enumerate((nn.Linear, Linear, Linear), start=1):
+            self.add_module("lin%d" % stage, kind(widths[stage - 1], widths[stage], bias=bias))
+            self.add_module("bn%d" % stage, nn.BatchNorm1d(widths[stage]))
         self.fc = FC_half2float(hidden3, num_classes, bias=True)
+        self.act = nn.Sequential(nn.Dropout(0.5), nn.ReLU())
 
     def forward(self, x):
-        for lin, bn in ((self.lin1, self.bn1), (self.lin2, self.bn2), (self.lin3, self.bn3)):
-            x = self.relu(self.dropout(bn(lin(x))))
+        for stage in (1, 2, 3):
+            x = self.act(getattr(self, "bn%d" % stage)(getattr(self, "lin%d" % stage)(x)))
         return self.fc(x)
 
 
