@@ -16,7 +16,10 @@ namespace bgemm {
 
 // Block = WGN x WGM waves, each wave owns WN x WM tiles of 32x32 outputs, PL activation planes.
 template <typename Eng, int WGN, int WGM, int WN, int WM, int PL, bool PIPE>
-__global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mfma_kernel(const GemmArgs a, const int tiles_n,
+// (Second launch bound: from two waves a SIMD on, a wave's register budget is the 256 architected registers, and the
+// compiler then keeps the accumulators there instead of in the accumulation registers, which the epilogue could
+// only reach through one copy per value.)
+__global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void gemm_mfma_kernel(const GemmArgs a, const int tiles_n,
                                                                    const int tiles_m)
 {
     // the wave index as a scalar: tile coordinates and operand bases stay on the scalar unit
@@ -60,28 +63,36 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
         xp[0][i] = Xb + (rt * a.KT) * TILE_U4 + lane;
         if (PL == 2) xp[PL - 1][i] = X2b + (rt * a.KT) * TILE_U4 + lane;
     }
+    // Plain fp16 output on a tile with an even number of weight tiles per wave: the two weight fragments of a
+    // pair take the even and the odd rows of the pair's 64 weight rows (lane l: rows 2l and 2l + 1), so that a
+    // lane ends up with two neighbouring outputs of a row, one 4-byte store of two halves, and a half-wave
+    // with a whole 128-byte line (see the epilogue).  The popcounts travel with the lane, nothing else changes.
+    const bool pair_cols = !PIPE && WM % 2 == 0 && a.out_kind == BGEMM_OUT_F16 && a.vec_store == 8 &&
+                           a.K <= (1 << 20) && a.M < (1 << 28);
 #pragma unroll
     for (int j = 0; j < WM; j++) {
-        const int64_t rt = min(mt0 + j, a.MT - 1);
-        wp[j] = Wb + (rt * a.KT) * TILE_U4 + lane;
+        if (pair_cols) {
+            const int r = 2 * (lane & 31) + (j & 1);                                  // row within the pair's 64
+            const int64_t rt = min(mt0 + (j & ~1) + (r >> 5), a.MT - 1);
+            wp[j] = Wb + (rt * a.KT) * TILE_U4 + (lane & 32) + (r & 31);
+        } else {
+            const int64_t rt = min(mt0 + j, a.MT - 1);
+            wp[j] = Wb + (rt * a.KT) * TILE_U4 + lane;
+        }
     }
 
     typename Eng::Acc acc[PL][WN][WM];
-#pragma unroll
-    for (int p = 0; p < PL; p++)
-#pragma unroll
-        for (int i = 0; i < WN; i++)
-#pragma unroll
-            for (int j = 0; j < WM; j++)
-#pragma unroll
-                for (int v = 0; v < 16; v++) acc[p][i][j][v] = 0;
     int pa[WM], pb[PL][WN];
+    if constexpr (PIPE) {           // (the other loop starts every sum with its first K-tile)
 #pragma unroll
-    for (int j = 0; j < WM; j++) pa[j] = 0;
+        for (int p = 0; p < PL; p++)
 #pragma unroll
-    for (int p = 0; p < PL; p++)
+            for (int i = 0; i < WN; i++)
 #pragma unroll
-        for (int i = 0; i < WN; i++) pb[p][i] = 0;
+                for (int j = 0; j < WM; j++)
+#pragma unroll
+                    for (int v = 0; v < 16; v++) acc[p][i][j][v] = 0;
+    }
 
     if constexpr (PIPE) {
         // ---- main loop, software-pipelined by hand -------------------------------------------------
@@ -155,16 +166,21 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
         for (int j = 0; j < WM; j++) pa[j] = pop[WN + j];
     } else {
     // ---- main loop: raw tiles are prefetched one K-tile ahead ----------------------------------
+    // The first K-tile is a copy of its own: its first MFMA step takes a constant zero as the sum to add to (no
+    // accumulator is cleared beforehand) and the popcounts start from it; and when all of K is at most 64 bits
+    // (attention scores at head size 64) only the first two words of a lane hold any, so two words a fragment
+    // are expanded instead of four.  A launch with one K-tile is mostly prologue and epilogue, and every wave
+    // pays them: instructions saved here are a fifth of such a launch.
     uint4 xf[PL][WN], wf[WM], xn[PL][WN], wn_[WM];
-    if (kt0 < kt1) {
 #pragma unroll
-        for (int p = 0; p < PL; p++)
+    for (int p = 0; p < PL; p++)
 #pragma unroll
-            for (int i = 0; i < WN; i++) xn[p][i] = xp[p][i][(int64_t)kt0 * TILE_U4];
+        for (int i = 0; i < WN; i++) xn[p][i] = xp[p][i][(int64_t)kt0 * TILE_U4];
 #pragma unroll
-        for (int j = 0; j < WM; j++) wn_[j] = wp[j][(int64_t)kt0 * TILE_U4];
-    }
-    for (int kt = kt0; kt < kt1; kt++) {
+    for (int j = 0; j < WM; j++) wn_[j] = wp[j][(int64_t)kt0 * TILE_U4];
+    const bool two_words = a.K <= 64;
+    auto k_tile = [&](auto first_c, auto two_c, const int kt) {
+        constexpr bool FIRST = decltype(first_c)::value, TWO = decltype(two_c)::value;
 #pragma unroll
         for (int p = 0; p < PL; p++)
 #pragma unroll
@@ -179,27 +195,34 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
 #pragma unroll
             for (int j = 0; j < WM; j++) wn_[j] = wp[j][(int64_t)(kt + 1) * TILE_U4];
         }
+        auto count = [](const uint4 w) { return TWO ? __popc(w.x) + __popc(w.y) : popc4(w); };
 #pragma unroll
-        for (int j = 0; j < WM; j++) pa[j] += popc4(wf[j]);
+        for (int j = 0; j < WM; j++) pa[j] = (FIRST ? 0 : pa[j]) + count(wf[j]);
 #pragma unroll
         for (int p = 0; p < PL; p++)
 #pragma unroll
-            for (int i = 0; i < WN; i++) pb[p][i] += popc4(xf[p][i]);
+            for (int i = 0; i < WN; i++) pb[p][i] = (FIRST ? 0 : pb[p][i]) + count(xf[p][i]);
+        typename Eng::Acc zero;
+#pragma unroll
+        for (int v = 0; v < 16; v++) zero[v] = 0;
 #pragma unroll
         for (int s = 0; s < Eng::STEPS; s++) {
             typename Eng::Frag bw[WM];
 #pragma unroll
-            for (int j = 0; j < WM; j++) bw[j] = Eng::expand_w(wf[j], s);
+            for (int j = 0; j < WM; j++) bw[j] = TWO ? Eng::expand_w2(wf[j], s) : Eng::expand_w(wf[j], s);
 #pragma unroll
             for (int p = 0; p < PL; p++)
 #pragma unroll
                 for (int i = 0; i < WN; i++) {
-                    const typename Eng::Frag ax = Eng::expand_x(xf[p][i], s);
+                    const typename Eng::Frag ax = TWO ? Eng::expand_x2(xf[p][i], s) : Eng::expand_x(xf[p][i], s);
 #pragma unroll
-                    for (int j = 0; j < WM; j++) acc[p][i][j] = Eng::mma(ax, bw[j], acc[p][i][j]);
+                    for (int j = 0; j < WM; j++) acc[p][i][j] = Eng::mma(ax, bw[j], FIRST && s == 0 ? zero : acc[p][i][j]);
                 }
         }
-    }
+    };
+    if (two_words) k_tile(std::true_type{}, std::true_type{}, kt0);
+    else k_tile(std::true_type{}, std::false_type{}, kt0);
+    for (int kt = kt0 + 1; kt < kt1; kt++) k_tile(std::false_type{}, std::false_type{}, kt);
 
     }
 
@@ -304,6 +327,57 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM == 8 ? 2 : 1)) void gemm_mf
         if (a.nt_store) rows_out(std::true_type{});
         else rows_out(std::false_type{});
         return;
+    }
+
+    // ---- plain fp16 from paired columns: straight from the accumulators ---------------------------
+    // With the weight rows dealt as above, a lane's accumulators 2p and 2p + 1 are the outputs (n, m) and
+    // (n, m + 1): rounded together (v_cvt_pk_f16_f32) they are one 4-byte store, 32 lanes one 128-byte line, as in
+    // the int32 case.  The arithmetic runs in fp32, where it is exact: every term is an integer below 2^24 for
+    // K <= 2^20, so the rounding to fp16 starts from the same number as on the integer path.
+    if constexpr (!PIPE && WM % 2 == 0) {
+        if (pair_cols) {
+            typedef _Float16 h2v __attribute__((ext_vector_type(2)));
+            typedef float f2v __attribute__((ext_vector_type(2)));
+            const float cdf = (float)mc.cd, cd2f = (float)mc.cd2;
+            float capaf[WM];
+#pragma unroll
+            for (int j = 0; j < WM; j++) capaf[j] = (float)capa[j];
+            const int64_t row_b = a.M * 2;
+            char* const out_b = reinterpret_cast<char*>(a.out) + (int64_t)b * a.strideC * 2;
+            const uint32_t voff = (uint32_t)(half * 4 * row_b + col * 4);
+#pragma unroll
+            for (int i = 0; i < WN; i++) {
+                const int64_t nrow0 = (int64_t)(nt0 + i) * 32;
+                if (nrow0 >= a.N) break;                          // the whole strip lies past the last row
+                int4 r4[4];
+#pragma unroll
+                for (int g = 0; g < 4; g++) r4[g] = *reinterpret_cast<const int4*>(rp + i * 32 + 8 * g + 4 * half);
+                char* const ub = out_b + nrow0 * row_b + (int64_t)mt0 * 64;       // uniform: scalar registers
+                const bool whole = nrow0 + 32 <= a.N && (int64_t)(mt0 + WM) * 32 <= a.M;
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const int4 q = r4[v >> 2];
+                    const float rowterm = (float)((v & 3) == 0 ? q.x : (v & 3) == 1 ? q.y : (v & 3) == 2 ? q.z : q.w);
+                    const int r = 8 * (v >> 2) + (v & 3);         // the lane's row is r + 4 * half
+                    unsigned* const row = reinterpret_cast<unsigned*>(ub + r * row_b + voff);
+#pragma unroll
+                    for (int pr = 0; pr < WM / 2; pr++) {
+                        f2v f;
+#pragma unroll
+                        for (int e = 0; e < 2; e++) {
+                            const int j = 2 * pr + e;
+                            float t = fmaf(cdf, Eng::to_float(acc[0][i][j], v), capaf[j] + rowterm);
+                            if (PL == 2) t = fmaf(cd2f, Eng::to_float(acc[PL - 1][i][j], v), t);
+                            f[e] = t;
+                        }
+                        const unsigned w = __builtin_bit_cast(unsigned, __builtin_convertvector(f, h2v));
+                        if (whole || ((int64_t)(mt0 + 2 * pr) * 32 + 2 * col < a.M && nrow0 + r + 4 * half < a.N))
+                            __builtin_nontemporal_store(w, row + pr * 32);
+                    }
+                }
+            }
+            return;
+        }
     }
 
     // ---- store ------------------------------------------------------------------------------
@@ -554,7 +628,8 @@ static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int pla
     auto blocks = [&](int bn, int bm) { return batch * cdiv(N, bn) * cdiv(M, bm); };
     if (M <= 64) return blocks(128, 64) >= 1024 ? MfmaCfg{BGEMM_KERNEL_MFMA_128x64, 128, 64} : MfmaCfg{BGEMM_KERNEL_MFMA_64x64, 64, 64};   // narrow outputs
     // a short K with a 2-byte output is all store path: rows of 512 bytes per block, many blocks in flight
-    // (192 x [512 x 512] x 64 -> fp16: 23.3 us against 25.0 to 28 on the other tiles; int32 output shows no preference)
+    // (192 x [512 x 512] x 64 -> fp16: 19.4 us against 20.4 on 128 x 128 and 25 to 29 on the tiles without paired
+    // columns; int32 output, 32 us for 201 MB, shows no preference)
     if (KT < 4 && out_shift == 1 && M >= 256 && blocks(32, 256) >= 512) return {BGEMM_KERNEL_MFMA_32x256, 32, 256};
     if (planes == 1 && blocks(256, 256) >= 512 && KT >= 32) return {BGEMM_KERNEL_MFMA_256x256, 256, 256};
     if (planes == 1 && blocks(256, 128) >= (KT >= 16 ? 256 : 512) && (KT >= 4 || blocks(128, 128) < 512)) return {BGEMM_KERNEL_MFMA_256x128, 256, 128};

@@ -28,6 +28,13 @@ struct EngI8 {
     __device__ static __forceinline__ Frag expand_x(const uint4 w, const int s) { return expand(w, s); }
     __device__ static __forceinline__ unsigned expand1_w(const unsigned w, const int s) { return expand1(w, s); }
     __device__ static __forceinline__ unsigned expand1_x(const unsigned w, const int s) { return expand1(w, s); }
+    // a K of at most 64 bits: only the first two words of a lane hold any
+    __device__ static __forceinline__ Frag expand_w2(const uint4 w, const int s)
+    {
+        Frag r = {(int)expand1(w.x, s), (int)expand1(w.y, s), 0, 0};
+        return r;
+    }
+    __device__ static __forceinline__ Frag expand_x2(const uint4 w, const int s) { return expand_w2(w, s); }
     __device__ static __forceinline__ Frag make(const unsigned (&f)[4])
     {
         Frag r = {(int)f[0], (int)f[1], (int)f[2], (int)f[3]};
@@ -38,6 +45,7 @@ struct EngI8 {
         return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
     }
     __device__ static __forceinline__ int to_int(const Acc& c, const int v) { return c[v]; }
+    __device__ static __forceinline__ float to_float(const Acc& c, const int v) { return (float)c[v]; }
 };
 
 // fp4 engine: the same tile is four 64-deep steps of v_mfma_f32_32x32x64_f8f6f4 with E2M1
@@ -72,6 +80,17 @@ struct EngF4 {
         r[0] = expand1_x(w.x, s); r[1] = expand1_x(w.y, s); r[2] = expand1_x(w.z, s); r[3] = expand1_x(w.w, s);
         return r;
     }
+    // a K of at most 64 bits: only the first two words of a lane hold any
+    __device__ static __forceinline__ Frag expand_w2(const uint4 w, const int s)
+    {
+        Frag r = {(int)expand1_w(w.x, s), (int)expand1_w(w.y, s), 0, 0, 0, 0, 0, 0};
+        return r;
+    }
+    __device__ static __forceinline__ Frag expand_x2(const uint4 w, const int s)
+    {
+        Frag r = {(int)expand1_x(w.x, s), (int)expand1_x(w.y, s), 0, 0, 0, 0, 0, 0};
+        return r;
+    }
     __device__ static __forceinline__ Frag make(const unsigned (&f)[4])
     {
         Frag r = {(int)f[0], (int)f[1], (int)f[2], (int)f[3], 0, 0, 0, 0};
@@ -83,6 +102,7 @@ struct EngF4 {
         return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 4, 4, 0, 0, 0, 0);
     }
     __device__ static __forceinline__ int to_int(const Acc& c, const int v) { return (int)c[v]; }
+    __device__ static __forceinline__ float to_float(const Acc& c, const int v) { return c[v]; }
 };
 
 __device__ __forceinline__ int popc4(const uint4 w)
