@@ -33,7 +33,7 @@ for _p in (ROOT, os.path.join(ROOT, "bgemm-cuda_amd")):
 INT8_MFMA_PEAK_TOPS = 5000.0      # MI355X dense int8 MFMA, published
 FP4_MFMA_PEAK_TOPS = 10100.0      # MI355X dense fp4 MFMA, published
 HBM_PEAK_GBS = 8000.0             # MI355X HBM3E, published
-PRE_ROLL = 100                    # untimed launches of the headline GEMM before its warm-up steps (see bench_c5)
+PRE_ROLL = 300                    # untimed launches of the headline GEMM before its warm-up steps (see bench_c5)
 C5_PROFILE = os.path.join(ROOT, "profiles", "gemm_mfma_f4_bgemm_8192x8192x8192.txt")
 PROBES_SO = os.path.join(ROOT, "libbench_probes.so")
 
@@ -169,8 +169,11 @@ def row(name, ms, ops, bytes_alg, ok, kernel, bound, **more):
 # ---------------------------------------------------------------- configuration 5: 8192^3 and its sweep
 def bench_c5(steps, warmup, M=8192, N=8192, K=8192, splitK=1, variant=0, pre_roll=0):
     """pre_roll: launches of the same GEMM issued (and waited for) before the warm-up steps, untimed: the GPU's
-    clocks take some tens of milliseconds of matrix-core load to settle, which five warm-up steps of 0.2 ms do
-    not give them.  The reference's drivers warm up with 100 launches (lowbit_kernel/csrc/kernel_test.h:10)."""
+    clocks take some tens of milliseconds of matrix-core load to settle (the launch runs at 0.19 ms for the first
+    hundred launches, 0.174 for the next and 0.171 from about 250 on), which five warm-up steps of 0.2 ms do not
+    give them.  The reference's drivers warm up with 100 launches and time 10 000
+    (lowbit_kernel/csrc/kernel_test.h:10-11): a steady-state figure, which is what the pre-roll makes of the
+    few timed steps here."""
     import torch
     import lowbit_kernel as lk
     dev = torch.device("cuda:0")
@@ -604,6 +607,8 @@ def main():
     ap.add_argument("--split-k", type=int, default=1,
                     help="splitK of the headline launch: the most K ranges a tile may be computed in (same bits for any value)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--pre-roll", type=int, default=PRE_ROLL,
+                    help="untimed launches of the headline GEMM before the warm-up steps (clock ramp)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run a 256 MiB device-to-device copy (known traffic, for scaling rocprof counters)")
     args = ap.parse_args()
@@ -641,7 +646,7 @@ def main():
         del cold
         torch.cuda.empty_cache()
 
-    c5, (w16, x16) = bench_c5(args.steps, args.warmup, splitK=args.split_k, variant=args.variant, pre_roll=PRE_ROLL)
+    c5, (w16, x16) = bench_c5(args.steps, args.warmup, splitK=args.split_k, variant=args.variant, pre_roll=args.pre_roll)
     log("C5:", json.dumps(c5))
     cpu = None if args.no_cpu else cpu_baseline_c5(w16, x16)
     del w16, x16
@@ -672,7 +677,7 @@ def main():
                    "op_count": "2*M*N*K binary multiply-accumulate ops per launch, the convention of the reference's "
                                "drivers (lowbit_kernel/csrc/benchmark.cu:291 prints it as TFLOPs)",
                    "pre_roll": "%d untimed launches of the same GEMM before the %d warm-up steps (clock ramp; the reference's "
-                               "drivers warm up with 100 launches, lowbit_kernel/csrc/kernel_test.h:10)" % (PRE_ROLL, args.warmup),
+                               "drivers warm up with 100 launches and time 10 000, lowbit_kernel/csrc/kernel_test.h:10-11)" % (args.pre_roll, args.warmup),
                    "bit_exact_sampled": c5["bit_exact"], "hbm_gbs_algorithmic": c5["gbs"],
                    "activation_pack_ms": c5["act_pack_ms"],
                    "frac_of_int8_mfma_peak": c5["tops"] / INT8_MFMA_PEAK_TOPS},

@@ -147,6 +147,42 @@ def test_each_tile_every_mode_batched(tile, engine):
 
 
 @pytest.mark.parametrize("engine", list(ENGINES))
+@pytest.mark.parametrize("tile", ["128x128", "32x256"])
+def test_fp16_pairs_straight_from_the_accumulators(tile, engine):
+    """Plain fp16 output with rows of a multiple of eight on the tiles whose waves hold an even number of weight
+    tiles: weight rows are dealt in pairs and two halves leave in one store.  Every mode (two bit planes included),
+    a ragged last weight tile (M = 328: the block's later tiles do not exist), a ragged last strip, and K of
+    one ragged word, two words (both take the two-words-a-fragment loop), one K-tile and three."""
+    rng = np.random.default_rng(97 + TILES[tile])
+    variant = force_kernel(TILES[tile], ENGINES[engine])
+    Bn, M, N = 2, 328, 77
+    for K in (40, 64, 200, 600):
+        w, x = pm1(rng, Bn, M, K), pm1(rng, Bn, N, K)
+        x[rng.random(x.shape) < 0.3] = 0
+        wp, xp, xt = lk.pack_sign(to_dev(w)), lk.pack_sign(to_dev(x)), lk.pack_ternary(to_dev(x))
+        assert lk.packed_kernel_id(wp, xp, MODE_XOR, 1, variant, torch.half) == TILES[tile]
+        for mode in (MODE_AND, MODE_XOR, MODE_ATTN, MODE_ATTN_X, MODE_BWTA):
+            got = lk.bgemm_packed_forward(wp, xt if mode == MODE_BWTA else xp, mode, torch.half, 1, variant).cpu().numpy()
+            assert (bits_of(got) == bits_of(f16_of(dense(mode, w, x)))).all(), (K, mode)
+
+
+@pytest.mark.parametrize("engine", list(ENGINES))
+@pytest.mark.parametrize("tile", [t for t in TILES if t not in ("256x256", "256x128")])
+def test_k_of_at_most_two_words_on_every_tile(tile, engine):
+    """K <= 64 expands two words a fragment instead of four (the loop of the tiles that are not hand-pipelined):
+    int32, every mode, K = 1, 33 and 64."""
+    rng = np.random.default_rng(131 + TILES[tile])
+    variant = force_kernel(TILES[tile], ENGINES[engine])
+    for K in (1, 33, 64):
+        w, x = pm1(rng, 2, 100, K), pm1(rng, 2, 45, K)
+        x[rng.random(x.shape) < 0.3] = 0
+        wp, xp, xt = lk.pack_sign(to_dev(w)), lk.pack_sign(to_dev(x)), lk.pack_ternary(to_dev(x))
+        for mode in (MODE_AND, MODE_XOR, MODE_ATTN, MODE_ATTN_X, MODE_BWTA):
+            got = lk.bgemm_packed_forward(wp, xt if mode == MODE_BWTA else xp, mode, torch.int32, 1, variant).cpu().numpy()
+            assert (got == dense(mode, w, x)).all(), (K, mode)
+
+
+@pytest.mark.parametrize("engine", list(ENGINES))
 @pytest.mark.parametrize("M,N,K,want_kernel", [
     (5907, 5903, 33 * 256 - 5, B.KERNEL_MFMA_256x256),       # the 8192^3 kernel: ragged edges, 33 K-tiles
     (8195, 2053, 17 * 256 - 7, B.KERNEL_MFMA_256x128),       # the 8192 x 2048 x 4096 kernel likewise
