@@ -208,6 +208,12 @@ def bench_sweep(steps=40, warmup=5):
     return rows
 
 
+def _lib_kernel_id(M, N, K):
+    """The kernel the library runs for an [N,K] x [M,K] sign product with fp16 output."""
+    import _lib
+    return _lib.lib().bgemm_packed_kernel_id(_lib.MODE_XOR, _lib.OUT_F16, 1, M, N, K, 1, _lib.VARIANT_AUTO)
+
+
 def bench_c5_dropin(steps, warmup, M=8192, N=8192, K=8192):
     """The same GEMM through the reference's own entry point, `bgemm_linear_forward_cuda(in_feats, weights)`:
     fp16 operands in, both sign-packed on every call (one launch), fp16 out."""
@@ -225,7 +231,8 @@ def bench_c5_dropin(steps, warmup, M=8192, N=8192, K=8192):
     want = (x16[cs].float() @ w16[rs].float().T).half()
     ok = bool(torch.equal(out[0][cs][:, rs], want))
     return row("C5 through the fp16 drop-in call %dx%dx%d (packs both operands per call, fp16 out)" % (M, N, K),
-               ms, 2.0 * M * N * K, 2.0 * (M * K + N * K + M * N), ok, "pack + mfma 256x256", "mfma")
+               ms, 2.0 * M * N * K, 2.0 * (M * K + N * K + M * N), ok,
+               "pack + " + KERNEL_NAMES.get(_lib_kernel_id(M, N, K), "?"), "mfma")
 
 
 def cpu_baseline_c5(w16, x16, budget_s=12.0):

@@ -631,9 +631,20 @@ static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int pla
     // (192 x [512 x 512] x 64 -> fp16: 19.4 us against 20.4 on 128 x 128 and 25 to 29 on the tiles without paired
     // columns; int32 output, 32 us for 201 MB, shows no preference)
     if (KT < 4 && out_shift == 1 && M >= 256 && blocks(32, 256) >= 512) return {BGEMM_KERNEL_MFMA_32x256, 32, 256};
-    if (planes == 1 && blocks(256, 256) >= 512 && KT >= 32) return {BGEMM_KERNEL_MFMA_256x256, 256, 256};
-    if (planes == 1 && blocks(256, 128) >= (KT >= 16 ? 256 : 512) && (KT >= 4 || blocks(128, 128) < 512)) return {BGEMM_KERNEL_MFMA_256x128, 256, 128};
+    // 256 x 256 (one wave a SIMD, the epilogue in the open) against 256 x 128 (two resident blocks a unit, one
+    // storing while the other multiplies, but half again as many expansions per MFMA): the smaller tile is 2 to 4 %
+    // faster at 32 K-tiles (8192^3: 0.168 against 0.172 ms), the larger one from 64 on (K = 16384: 0.308 against 0.319)
+    if (planes == 1 && blocks(256, 256) >= 512 && KT >= 64) return {BGEMM_KERNEL_MFMA_256x256, 256, 256};
+    // from two blocks a unit, or from one with 16 K-tiles; a few blocks more than one a unit (11008 x 768 x 4096:
+    // 258) would leave the launch waiting for two units that run two blocks each, and go to the next tile down
+    const int64_t b21 = blocks(256, 128);
+    if (planes == 1 && (b21 >= 512 || (KT >= 16 && (b21 == 256 || b21 >= 320 || (b21 > 256 && blocks(128, 128) < 512)))) &&
+        (KT >= 4 || blocks(128, 128) < 512))
+        return {BGEMM_KERNEL_MFMA_256x128, 256, 128};
     if (blocks(128, 128) >= 512) return {BGEMM_KERNEL_MFMA_128x128, 128, 128};
+    // two bit planes on few blocks: 32 x 256 shares every weight expansion between the planes of one row tile
+    // (W[11008,4096] x 128 ternary rows 9.7 us against 10.9 / 11.3 on the next two), once it has 160 blocks
+    if (planes == 2 && blocks(64, 128) < 512 && blocks(32, 256) >= 160) return {BGEMM_KERNEL_MFMA_32x256, 32, 256};
     if (blocks(64, 128) >= 512) return {BGEMM_KERNEL_MFMA_64x128, 64, 128};      // below two blocks a unit, twice as many 32-row tiles are faster
     return {BGEMM_KERNEL_MFMA_32x128, 32, 128};
 }

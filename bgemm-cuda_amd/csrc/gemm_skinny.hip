@@ -749,17 +749,16 @@ static bool skinny_quad_shape(int planes, int64_t batch, int64_t MT, int64_t NT,
 // Shapes the skinny kernels take: one group of activation rows always (32 rows, or 16 rows of two bit planes).
 // More groups where splitting K inside the block buys more than the general kernel's 32 x 128 tiles do (timed
 // over sweeps of shapes, pieces = 32 x 32 outputs): up to 512 pieces from four K-tiles on and up to 1024 from
-// eight; two bit planes (two operands a block against one weight expansion) up to 1792 from sixteen K-tiles on
-// (1024 from 24 on, where the four-pieces kernel takes over).  The last bounds are set by weights that come
-// from HBM rather than from a warm cache (a model's layers): there the general kernel's serial K loop pays the
-// full memory latency per step.  Beyond, the four-pieces kernel where that pays (see above), else the general one.
+// eight, one bit plane or two (two operands a block against one weight expansion).  The last bound is set by
+// weights that come from HBM rather than from a warm cache (a model's layers): there the general kernel's serial
+// K loop pays the full memory latency per step.  Beyond, the four-pieces kernel where that pays (see above),
+// else the general one (W[11008,4096] x 128 ternary rows, 1376 pieces: 9.7 us there against 12.5 here).
 bool gemm_skinny_shape(int planes, int64_t batch, int64_t M, int64_t N, int64_t K)
 {
     if (batch > 65535) return false;             // these kernels walk the batch in the grid's third dimension
     if (N <= (planes == 2 ? 16 : 32)) return true;
     const int64_t pieces = batch * row_tiles(M) * row_tiles(N), KT = k_tiles(K);
     if (skinny_quad_shape(planes, batch, row_tiles(M), row_tiles(N), KT)) return true;
-    if (KT >= 16 && planes == 2) return pieces <= (KT >= 24 ? 1024 : 1792);
     if (KT >= 8) return pieces <= 1024;
     return KT >= 4 && pieces <= 512;
 }

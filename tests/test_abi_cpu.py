@@ -100,7 +100,11 @@ def test_dispatch_of_the_benchmark_configurations():
         B.MODE_XOR, B.MODE_BWTA, B.MODE_ATTN_X, B.VARIANT_AUTO, B.VARIANT_VALU, B.force_kernel)
     TILES = (0, 1, 2, 3, 4, 5, 6, 7)
     A = VARIANT_AUTO
-    assert kid(MODE_XOR, 1, 8192, 8192, 8192, 1, A) == B.KERNEL_MFMA_256x256
+    assert kid(MODE_XOR, 1, 8192, 8192, 8192, 1, A) == B.KERNEL_MFMA_256x128
+    assert kid(MODE_XOR, 1, 8192, 8192, 16384, 1, A) == B.KERNEL_MFMA_256x256
+    assert kid(MODE_XOR, 1, 11008, 768, 4096, 1, A) == B.KERNEL_MFMA_128x128     # 258 blocks of 256 x 128: one too many
+    assert kid(MODE_BWTA, 1, 11008, 128, 4096, 1, A) == B.KERNEL_MFMA_32x256
+    assert kid(MODE_BWTA, 1, 11008, 64, 4096, 1, A) == B.KERNEL_SKINNY_SPLITK
     assert kid(MODE_XOR, 1, 8192, 2048, 4096, 1, A) == B.KERNEL_MFMA_256x128
     assert kid(MODE_XOR, 1, 8192, 2048, 16384, 4, A) == B.KERNEL_MFMA_256x128
     assert kid(MODE_XOR, 1, 8192, 256, 16384, 1, A) == B.KERNEL_SKINNY_QUAD

@@ -184,7 +184,8 @@ def test_k_of_at_most_two_words_on_every_tile(tile, engine):
 
 @pytest.mark.parametrize("engine", list(ENGINES))
 @pytest.mark.parametrize("M,N,K,want_kernel", [
-    (5907, 5903, 33 * 256 - 5, B.KERNEL_MFMA_256x256),       # the 8192^3 kernel: ragged edges, 33 K-tiles
+    (5907, 5903, 65 * 256 - 5, B.KERNEL_MFMA_256x256),       # the tile of the longest K: ragged edges, 65 K-tiles
+    (5907, 5903, 33 * 256 - 5, B.KERNEL_MFMA_256x128),       # the 8192^3 kernel: ragged edges, 33 K-tiles
     (8195, 2053, 17 * 256 - 7, B.KERNEL_MFMA_256x128),       # the 8192 x 2048 x 4096 kernel likewise
 ])
 def test_headline_tiles_where_the_library_picks_them(oracle, engine, M, N, K, want_kernel):
