@@ -167,7 +167,7 @@ def row(name, ms, ops, bytes_alg, ok, kernel, bound, **more):
 
 
 # ---------------------------------------------------------------- configuration 5: 8192^3 and its sweep
-def bench_c5(steps, warmup, M=8192, N=8192, K=8192, splitK=1, variant=0, pre_roll=0):
+def bench_c5(steps, warmup, M=8192, N=8192, K=8192, splitK=1, variant=0, pre_roll=0, counted=False):
     """pre_roll: launches of the same GEMM issued (and waited for) before the warm-up steps, untimed: the GPU's
     clocks take some tens of milliseconds of matrix-core load to settle (the launch runs at 0.19 ms for the first
     hundred launches, 0.174 for the next and 0.171 from about 250 on), which five warm-up steps of 0.2 ms do not
@@ -178,7 +178,11 @@ def bench_c5(steps, warmup, M=8192, N=8192, K=8192, splitK=1, variant=0, pre_rol
     import lowbit_kernel as lk
     dev = torch.device("cuda:0")
     w16, x16 = pm1_f16((M, K), 5001, dev), pm1_f16((N, K), 5002, dev)
+    # prepacked operands: the tiled bits.  `counted`: with their row popcounts as well (the large tiles then count
+    # nothing in their main loop); the headline is timed without, and with them beside it.
     wp, xp = lk.pack_sign(w16), lk.pack_sign(x16)
+    if counted and (variant & 0xff) != 1:
+        lk.row_popcounts(wp), lk.row_popcounts(xp)
     out = torch.empty((1, N, M), dtype=torch.int32, device=dev)
     fn = lambda i: lk.bgemm_packed_forward(wp, xp, lk.MODE_XOR, torch.int32, splitK, variant, out=out)
     for i in range(pre_roll):
@@ -186,12 +190,27 @@ def bench_c5(steps, warmup, M=8192, N=8192, K=8192, splitK=1, variant=0, pre_rol
     torch.cuda.synchronize()
     ms = time_gpu(fn, warmup, steps)
     ok = check_sampled(out[0], w16, x16)
+    ms_counted = count_ms = None
+    if pre_roll and xp.counts is None and (variant & 0xff) != 1:
+        # beside the headline row: the same launches on operands that bring their row popcounts along
+        lk.row_popcounts(wp), lk.row_popcounts(xp)
+        for i in range(pre_roll):          # the check above left the GPU idle: its clocks have to settle again
+            fn(i)
+        torch.cuda.synchronize()
+        ms_counted = time_gpu(fn, warmup, steps)
+        ok = ok and check_sampled(out[0], w16, x16)
+
+        def count_again(i):
+            xp.counts = None
+            lk.row_popcounts(xp)
+        count_ms = time_gpu(count_again, 2, 10)
     ops = 2.0 * M * N * K
     bytes_alg = M * K / 8 + N * K / 8 + 4.0 * M * N
     pack_ms = time_gpu(lambda i: lk.pack_sign(x16), 2, 10)
     return {"name": "C5 BGEMM %dx%dx%d xor int32 splitK=%d" % (M, N, K, splitK), "ms": ms,
             "tops": ops / ms / 1e9, "gbs": bytes_alg / ms / 1e6, "ops": ops, "bytes": bytes_alg,
-            "bit_exact": ok, "act_pack_ms": pack_ms, "kernel": kernel_of(wp, xp, lk.MODE_XOR, splitK, variant)}, (w16, x16)
+            "bit_exact": ok, "act_pack_ms": pack_ms, "act_popcount_ms": count_ms, "ms_counted": ms_counted,
+            "kernel": kernel_of(wp, xp, lk.MODE_XOR, splitK, variant)}, (w16, x16)
 
 
 def bench_sweep(steps=40, warmup=5):
@@ -616,6 +635,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--pre-roll", type=int, default=PRE_ROLL,
                     help="untimed launches of the headline GEMM before the warm-up steps (clock ramp)")
+    ap.add_argument("--counted", action="store_true",
+                    help="time the headline on operands that bring their row popcounts (bgemm_packed_forward_counted)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run a 256 MiB device-to-device copy (known traffic, for scaling rocprof counters)")
     args = ap.parse_args()
@@ -653,7 +674,8 @@ def main():
         del cold
         torch.cuda.empty_cache()
 
-    c5, (w16, x16) = bench_c5(args.steps, args.warmup, splitK=args.split_k, variant=args.variant, pre_roll=args.pre_roll)
+    c5, (w16, x16) = bench_c5(args.steps, args.warmup, splitK=args.split_k, variant=args.variant, pre_roll=args.pre_roll,
+                                  counted=args.counted)
     log("C5:", json.dumps(c5))
     cpu = None if args.no_cpu else cpu_baseline_c5(w16, x16)
     del w16, x16
@@ -686,7 +708,8 @@ def main():
                    "pre_roll": "%d untimed launches of the same GEMM before the %d warm-up steps (clock ramp; the reference's "
                                "drivers warm up with 100 launches and time 10 000, lowbit_kernel/csrc/kernel_test.h:10-11)" % (args.pre_roll, args.warmup),
                    "bit_exact_sampled": c5["bit_exact"], "hbm_gbs_algorithmic": c5["gbs"],
-                   "activation_pack_ms": c5["act_pack_ms"],
+                   "activation_pack_ms": c5["act_pack_ms"], "activation_popcount_ms": c5["act_popcount_ms"],
+                   "ms_per_step_with_row_popcounts_prepacked": c5["ms_counted"],
                    "frac_of_int8_mfma_peak": c5["tops"] / INT8_MFMA_PEAK_TOPS},
         "roofline": roofline,
         "cpu_baseline": cpu,

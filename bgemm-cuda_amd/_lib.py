@@ -13,7 +13,7 @@ OK, EINVAL, ENULL, EWORKSPACE, ELAUNCH, EALIGN = 0, -1, -2, -3, -4, -5
 MODE_AND, MODE_XOR, MODE_ATTN, MODE_BWTA, MODE_ATTN_X = 0, 1, 2, 3, 4
 OUT_I32, OUT_F16, OUT_F32_SCALED, OUT_F16_SCALED, OUT_BITS_F32, OUT_BITS_F16 = 0, 1, 2, 3, 4, 5
 SRC_F16, SRC_F32 = 0, 1
-ABI_VERSION = 8
+ABI_VERSION = 9
 LAYOUT_VERSION = 6     # of the tiled operand layout, written into packed files; changes only when the layout does
 STATIC_SCRATCH_BYTES = 32 << 20      # BGEMM_STATIC_SCRATCH_BYTES
 VARIANT_AUTO, VARIANT_VALU, VARIANT_MFMA, VARIANT_MFMA_F4 = 0, 1, 2, 3
@@ -46,6 +46,9 @@ SIGNATURES = {
     "bgemm_packed_forward": (_int, [_int, _p, _p, _p, _p, _int, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
                                     _int, _int, _p, _sz, _p, _sz, _p]),
     "bgemm_packed_kernel_id": (_int, [_int, _int, _i64, _i64, _i64, _i64, _int, _int]),
+    "bgemm_row_popcounts": (_int, [_p, _i64, _i64, _i64, _i64, _p, _p]),
+    "bgemm_packed_forward_counted": (_int, [_int, _p, _p, _p, _p, _p, _int, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
+                                            _int, _p]),
     "bgemm_packed_forward_scaled": (_int, [_int, _p, _p, _p, _p, _int, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
                                            _int, _int, _p, _sz, _p, _sz, _p, _p, _p, _p]),
     "bgemm_packed_forward_bits": (_int, [_int, _p, _p, _p, _p, _int, _i64, _i64, _i64, _i64, _i64, _i64, _i64,

@@ -71,7 +71,7 @@ __global__ void clear_counters_kernel(uint32_t* c, int64_t n)
 using namespace bgemm;
 
 extern "C" const char* bgemm_last_error(void) { return g_err; }
-extern "C" int bgemm_abi_version(void) { return 8; }
+extern "C" int bgemm_abi_version(void) { return 9; }
 
 static bool ws_query(int mode, int64_t batch, int64_t M, int64_t N, int64_t K, int splitK, int variant,
                      size_t* part, size_t* counters)
@@ -127,6 +127,8 @@ __global__ void fill_empty_bits_kernel(const GemmArgs a)
 
 // Unpacked activations for the decode kernel that packs them itself (null = X_tiled / X2_tiled are used).
 struct RawActivations { const void* src; int f32; int64_t ld; const void* zero_point; };
+// Row popcounts the caller brings for both operands (one bit plane), or null.
+struct RowCounts { const void* w; const void* x; };
 
 static int packed_forward(int mode, const void* W_tiled, const void* X_tiled, const void* X2_tiled,
                           void* out, int out_dtype, int64_t batch, int64_t M, int64_t N, int64_t K,
@@ -134,7 +136,8 @@ static int packed_forward(int mode, const void* W_tiled, const void* X_tiled, co
                           int splitK, int variant, void* ws, size_t ws_bytes,
                           void* counters, size_t counter_bytes,
                           const void* sw, const void* sa, const void* bias, const void* zp, void* stream,
-                          const RawActivations* raw = nullptr, const bool kernel_id_only = false)
+                          const RawActivations* raw = nullptr, const bool kernel_id_only = false,
+                          const RowCounts* counts = nullptr)
 {
     g_err[0] = 0;
     GemmArgs a;
@@ -197,6 +200,13 @@ static int packed_forward(int mode, const void* W_tiled, const void* X_tiled, co
     if (((uintptr_t)W_tiled & 15) || ((uintptr_t)X_tiled & 15) || ((uintptr_t)X2_tiled & 15))
         return fail(BGEMM_EALIGN, "bgemm_packed_forward: operands must be 16-byte aligned");
 
+    if (counts) {
+        if (!counts->w || !counts->x) return fail(BGEMM_ENULL, "bgemm_packed_forward_counted: a count array is NULL");
+        if (((uintptr_t)counts->w & 3) || ((uintptr_t)counts->x & 3))
+            return fail(BGEMM_EALIGN, "bgemm_packed_forward_counted: count arrays must be 4-byte aligned");
+        if (a.mc.planes != 1) return fail(BGEMM_EINVAL, "bgemm_packed_forward_counted: modes of one bit plane only");
+        a.cntW = (const int32_t*)counts->w; a.cntX = (const int32_t*)counts->x;
+    }
     a.W = (const uint4*)W_tiled; a.X = (const uint4*)X_tiled; a.X2 = (const uint4*)X2_tiled;
     a.MT = (int)row_tiles(M); a.NT = (int)row_tiles(N); a.KT = (int)k_tiles(K);
     a.strideW = strideW / 4; a.strideX = strideX / 4;
@@ -262,6 +272,21 @@ extern "C" int bgemm_packed_forward(int mode, const void* W_tiled, const void* X
         return fail(BGEMM_EINVAL, "bgemm_packed_forward: unknown output dtype %d", out_dtype);
     return packed_forward(mode, W_tiled, X_tiled, X2_tiled, out, out_dtype, batch, M, N, K, strideW, strideX, strideC,
                           splitK, variant, ws, ws_bytes, counters, counter_bytes, nullptr, nullptr, nullptr, nullptr, stream);
+}
+
+extern "C" int bgemm_packed_forward_counted(int mode, const void* W_tiled, const void* X_tiled, const void* W_counts,
+                                            const void* X_counts, void* out, int out_dtype, int64_t batch, int64_t M,
+                                            int64_t N, int64_t K, int64_t strideW, int64_t strideX, int64_t strideC,
+                                            int variant, void* stream)
+{
+    if (out_dtype != BGEMM_OUT_I32 && out_dtype != BGEMM_OUT_F16)
+        return fail(BGEMM_EINVAL, "bgemm_packed_forward_counted: unknown output dtype %d", out_dtype);
+    int family, force;
+    if (split_variant(variant, &family, &force) && family == BGEMM_VARIANT_VALU)
+        return fail(BGEMM_EINVAL, "bgemm_packed_forward_counted: the matrix-core kernels only");
+    const RowCounts counts = {W_counts, X_counts};
+    return packed_forward(mode, W_tiled, X_tiled, nullptr, out, out_dtype, batch, M, N, K, strideW, strideX, strideC, 1,
+                          variant, nullptr, 0, nullptr, 0, nullptr, nullptr, nullptr, nullptr, stream, nullptr, false, &counts);
 }
 
 extern "C" int bgemm_packed_forward_scaled(int mode, const void* W_tiled, const void* X_tiled, const void* X2_tiled,

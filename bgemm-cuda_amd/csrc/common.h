@@ -76,6 +76,8 @@ struct GemmArgs {
     int64_t strideW, strideX, strideC;   // uint4 units for W/X, elements for C
     int batch, splitK;
     int force;            // BGEMM_KERNEL_* the caller insists on (BGEMM_FORCE_KERNEL), or -1: chosen by shape
+    const int32_t* cntW; const int32_t* cntX;   // row popcounts of W and X ([batch][rows], a shared operand once), or null:
+                                                // the pipelined tiles then count nothing themselves
     ModeCoef mc;
     // activations not packed yet (the decode kernel packs them itself): X/X2 are null and these describe
     // the [N][K] source; with two planes the ternary planes of sign(x) are formed

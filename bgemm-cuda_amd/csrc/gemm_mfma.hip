@@ -15,7 +15,9 @@
 namespace bgemm {
 
 // Block = WGN x WGM waves, each wave owns WN x WM tiles of 32x32 outputs, PL activation planes.
-template <typename Eng, int WGN, int WGM, int WN, int WM, int PL, bool PIPE>
+// COUNTED (pipelined tiles only): the operands' row popcounts come with the call (GemmArgs::cntW / cntX) and the main
+// loop counts nothing: a sixth of its vector instructions on the 256 x 128 tile, 4 % of an 8192^3 launch.
+template <typename Eng, int WGN, int WGM, int WN, int WM, int PL, bool PIPE, bool COUNTED = false>
 // (Second launch bound: from two waves a SIMD on, a wave's register budget is the 256 architected registers, and the
 // compiler then keeps the accumulators there instead of in the accumulation registers, which the epilogue could
 // only reach through one copy per value.)
@@ -139,7 +141,7 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
                         nxt[d / 4][d % 4] = d / 4 < WN      // fragments 0 .. WN-1 are the activation side
                             ? (s + 1 < STEPS ? Eng::expand1_x(A[d / 4][d % 4], s + 1) : Eng::expand1_x(B[d / 4][d % 4], 0))
                             : (s + 1 < STEPS ? Eng::expand1_w(A[d / 4][d % 4], s + 1) : Eng::expand1_w(B[d / 4][d % 4], 0));
-                    if (s == 0 && q < NF) {     // v_bcnt adds into its accumulator: four instructions a fragment, written out
+                    if (!COUNTED && s == 0 && q < NF) {     // v_bcnt adds into its accumulator: four instructions a fragment, written out
 #pragma unroll                                  // because the compiler prefers four counts and two three-way adds
                         for (int c = 0; c < 4; c++) asm("v_bcnt_u32_b32 %0, %1, %0" : "+v"(pop[q]) : "v"(A[q][c]));
                     }
@@ -160,10 +162,20 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
                 k_tile(rawB, rawA, kt + 1);
             }
         }
+        if constexpr (COUNTED) {
+            // the lane's row of every fragment, read where the caller keeps the counts (rows past the end: any valid one,
+            // their outputs are never stored); halved below by nothing: these are whole rows, not K-halves
+            const int64_t cx = a.strideX ? (int64_t)b * a.N : 0, cw = a.strideW ? (int64_t)b * a.M : 0;
 #pragma unroll
-        for (int i = 0; i < WN; i++) pb[0][i] = pop[i];
+            for (int i = 0; i < WN; i++) pb[0][i] = a.cntX[cx + min((int64_t)(nt0 + i) * 32 + (lane & 31), a.N - 1)];
 #pragma unroll
-        for (int j = 0; j < WM; j++) pa[j] = pop[WN + j];
+            for (int j = 0; j < WM; j++) pa[j] = a.cntW[cw + min((int64_t)(mt0 + j) * 32 + (lane & 31), a.M - 1)];
+        } else {
+#pragma unroll
+            for (int i = 0; i < WN; i++) pb[0][i] = pop[i];
+#pragma unroll
+            for (int j = 0; j < WM; j++) pa[j] = pop[WN + j];
+        }
     } else {
     // ---- main loop: raw tiles are prefetched one K-tile ahead ----------------------------------
     // The first K-tile is a copy of its own: its first MFMA step takes a constant zero as the sum to add to (no
@@ -228,12 +240,14 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
 
     // ---- epilogue: rank-one terms turn the AND-dot into C -----------------------------------------
     const int bits = (int)a.K;
+    if constexpr (!COUNTED) {        // a lane counted its K-half of the row
 #pragma unroll
-    for (int j = 0; j < WM; j++) pa[j] += __shfl_xor(pa[j], 32);
+        for (int j = 0; j < WM; j++) pa[j] += __shfl_xor(pa[j], 32);
 #pragma unroll
-    for (int p = 0; p < PL; p++)
+        for (int p = 0; p < PL; p++)
 #pragma unroll
-        for (int i = 0; i < WN; i++) pb[p][i] += __shfl_xor(pb[p][i], 32);
+            for (int i = 0; i < WN; i++) pb[p][i] += __shfl_xor(pb[p][i], 32);
+    }
 
     // Per-element terms go through the full-rate unsigned 24-bit multiply (dot_term: the dots stay below
     // 2^24); v_mul_lo_u32 would cost four times as much per element, and is used for the few row and
@@ -663,7 +677,10 @@ static int launch_cfg(const GemmArgs& a, hipStream_t st)
                                dim3(WGN * WGM * 64), 0, st, a, tiles_n, tiles_m);
         else
             return fail(BGEMM_EINVAL, "gemm_mfma: tile not built for two planes");
-    } else
+    } else if ((WN * WM >= 8) && a.cntW && a.cntX)
+        hipLaunchKernelGGL((gemm_mfma_kernel<Eng, WGN, WGM, WN, WM, 1, (WN * WM >= 8), (WN * WM >= 8)>), dim3((unsigned)grid),
+                           dim3(WGN * WGM * 64), 0, st, a, tiles_n, tiles_m);
+    else
         hipLaunchKernelGGL((gemm_mfma_kernel<Eng, WGN, WGM, WN, WM, 1, (WN * WM >= 8)>), dim3((unsigned)grid),
                            dim3(WGN * WGM * 64), 0, st, a, tiles_n, tiles_m);
     return check_launch("gemm_mfma");

@@ -480,6 +480,54 @@ static int relayout(const void* src, void* dst, int64_t rows, int64_t K, int dir
     return check_launch(who);
 }
 
+// Row popcounts of a tiled operand: one block of sixteen waves per 32-row tile row, wave w takes K-tiles w, w + 16, ...
+// (two 16-byte loads in flight a lane: a launch of this size is one memory round trip), lanes 0-31 and 32-63 of a
+// wave hold the two K-halves of a row; the partial counts of a row meet in LDS.
+__global__ __launch_bounds__(1024) void row_popcount_kernel(const uint4* __restrict__ tiled, int32_t* __restrict__ counts,
+                                                            const int64_t rows, const int64_t KT, const int64_t stride_u4)
+{
+    __shared__ int part[1024];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t rt = blockIdx.x, b = blockIdx.y;
+    const uint4* base = tiled + b * stride_u4 + rt * KT * TILE_U4 + lane;
+    int n = 0;
+    int64_t kt = wave;
+    for (; kt + 16 < KT; kt += 32) {
+        const uint4 v0 = base[kt * TILE_U4], v1 = base[(kt + 16) * TILE_U4];
+        n += __popc(v0.x) + __popc(v0.y) + __popc(v0.z) + __popc(v0.w) + __popc(v1.x) + __popc(v1.y) + __popc(v1.z) + __popc(v1.w);
+    }
+    if (kt < KT) {
+        const uint4 v = base[kt * TILE_U4];
+        n += __popc(v.x) + __popc(v.y) + __popc(v.z) + __popc(v.w);
+    }
+    part[threadIdx.x] = n;
+    __syncthreads();
+    if (threadIdx.x < 32) {
+        int t = 0;
+#pragma unroll
+        for (int w = 0; w < 32; w++) t += part[w * 32 + threadIdx.x];     // 16 waves x 2 K-halves
+        const int64_t row = rt * 32 + threadIdx.x;
+        if (row < rows) counts[b * rows + row] = t;
+    }
+}
+
+extern "C" int bgemm_row_popcounts(const void* tiled, int64_t batch, int64_t rows, int64_t K, int64_t stride_words,
+                                   void* counts, void* stream)
+{
+    if (batch < 0 || rows < 0 || K < 0 || K >= (1LL << 24) || stride_words < 0 || (stride_words & 3))
+        return fail(BGEMM_EINVAL, "bgemm_row_popcounts: bad shape batch=%lld rows=%lld K=%lld stride=%lld", (long long)batch,
+                    (long long)rows, (long long)K, (long long)stride_words);
+    if (batch == 0 || rows == 0) return BGEMM_OK;
+    if (!counts || (K > 0 && !tiled)) return fail(BGEMM_ENULL, "bgemm_row_popcounts: null pointer");
+    if (((uintptr_t)tiled & 15) || ((uintptr_t)counts & 3)) return fail(BGEMM_EALIGN, "bgemm_row_popcounts: operand not aligned");
+    if (batch > 65535 || row_tiles(rows) > 0x7fffffffLL) return fail(BGEMM_EINVAL, "bgemm_row_popcounts: operand too large");
+    if (batch > 1 && stride_words < bgemm_tiled_words(rows, K))
+        return fail(BGEMM_EINVAL, "bgemm_row_popcounts: stride %lld smaller than one operand", (long long)stride_words);
+    hipLaunchKernelGGL(row_popcount_kernel, dim3((unsigned)row_tiles(rows), (unsigned)batch), dim3(1024), 0, (hipStream_t)stream,
+                       (const uint4*)tiled, (int32_t*)counts, rows, k_tiles(K), stride_words / 4);
+    return check_launch("bgemm_row_popcounts");
+}
+
 extern "C" int bgemm_tile_from_logical(const uint32_t* logical, int64_t rows, int64_t K,
                                        void* dst_tiled, void* stream)
 {

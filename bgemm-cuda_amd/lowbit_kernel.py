@@ -97,6 +97,7 @@ class PackedBits:
 
     def __init__(self, data, data2, batch, rows, K):
         self.data, self.data2, self.batch, self.rows, self.K = data, data2, batch, rows, K
+        self.counts = None        # int32 [batch, rows] row popcounts once row_popcounts() has been called
 
     @property
     def ternary(self):
@@ -120,6 +121,23 @@ def _check_packed(p, name):
                              "got %s %s" % (name, p.batch, words, p.rows, p.K, plane.dtype, tuple(plane.shape)))
         if plane.device != p.data.device:
             raise ValueError("%s: both planes must live on one device" % name)
+
+
+def row_popcounts(p):
+    """Computes (once) and attaches the row popcounts of a binary packed operand, ``p.counts`` int32
+    ``[batch, rows]``, and returns ``p``.  ``bgemm_packed_forward`` hands them to the library when both operands
+    carry them: they are part of a prepacked operand, and the large tiles then leave the counting out of their
+    main loop.  Call it again after writing new bits into ``p.data`` (it recomputes when ``p.counts`` is None)."""
+    if p.ternary:
+        raise ValueError("row popcounts are kept for binary operands")
+    if p.counts is None:
+        _check_packed(p, "p")
+        counts = torch.empty((p.batch, p.rows), dtype=torch.int32, device=p.data.device)
+        with _on(p.data.device):
+            _b.check(_b.lib().bgemm_row_popcounts(p.data.data_ptr(), p.batch, p.rows, p.K, p.words if p.batch > 1 else 0,
+                                                  counts.data_ptr(), _stream()))
+        p.counts = counts
+    return p
 
 
 def packed_kernel_id(w, x, mode=MODE_XOR, splitK=1, variant=VARIANT_AUTO, out_dtype=torch.int32):
@@ -326,7 +344,19 @@ def bgemm_packed_forward(w, x, mode=MODE_XOR, out_dtype=torch.int32, splitK=1, v
                 N * M if bits_out is None else bits_out.words, splitK, variant,
                 ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0,
                 cnt.data_ptr() if cnt is not None else None, cnt.numel() if cnt is not None else 0)
-        if scale is None:
+        counted = (scale is None and w.counts is not None and x.counts is not None and ws is None
+                   and (variant & 0xff) != VARIANT_VALU)
+        if counted:
+            for name, p in (("w", w), ("x", x)):
+                c = p.counts
+                if (c.dtype != torch.int32 or tuple(c.shape) != (p.batch, p.rows) or not c.is_contiguous()
+                        or c.device != dev):
+                    raise ValueError("%s.counts must be a contiguous int32 tensor of shape (%d, %d) on %s"
+                                     % (name, p.batch, p.rows, dev))
+            _b.check(L.bgemm_packed_forward_counted(mode, args[1], args[2], w.counts.data_ptr(), x.counts.data_ptr(),
+                                                    args[4], kind, batch, M, N, K, args[10], args[11], args[12],
+                                                    variant, _stream()))
+        elif scale is None:
             _b.check(L.bgemm_packed_forward(*args, _stream()))
         elif bits_out is not None:
             _b.check(L.bgemm_packed_forward_bits(*args, sw.data_ptr(), sa.data_ptr(),

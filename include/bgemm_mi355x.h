@@ -181,6 +181,23 @@ int bgemm_packed_forward(int mode, const void* W_tiled, const void* X_tiled, con
 int bgemm_packed_kernel_id(int mode, int out_dtype, int64_t batch, int64_t M, int64_t N, int64_t K, int splitK,
                            int variant);
 
+/* Row popcounts of a tiled operand, counts[b * rows + r] (int32) = set bits in row r of batch entry b
+ * (stride_words between entries; 0 with batch 1).  Every mode but AND needs them for its rank-one terms
+ * (bits - 2 popc(a) - 2 popc(b) + 4 popc(a & b) is the XOR form of ptx_mma.cuh:212-250); the kernels count
+ * while they multiply unless the caller brings the counts along, below.  They belong to a prepacked operand
+ * like its bits: computed once per weight (the reference's weight_prepacking.h has no such field; its kernel
+ * re-derives everything per call). */
+int bgemm_row_popcounts(const void* tiled, int64_t batch, int64_t rows, int64_t K, int64_t stride_words,
+                        void* counts, void* stream);
+/* bgemm_packed_forward for the modes of one bit plane, with the row popcounts of both operands supplied
+ * (W_counts [batch][M] or [M] when strideW is 0, X_counts likewise): same results; the large tiles leave the
+ * counting out of their main loop (a sixth of its vector instructions; 4 % of an 8192^3 launch), the other
+ * kernels ignore the counts.  Matrix-core families only; K is never split, no workspace. */
+int bgemm_packed_forward_counted(int mode, const void* W_tiled, const void* X_tiled, const void* W_counts,
+                                 const void* X_counts, void* out, int out_dtype, int64_t batch, int64_t M,
+                                 int64_t N, int64_t K, int64_t strideW, int64_t strideX, int64_t strideC,
+                                 int variant, void* stream);
+
 /* The same GEMM with the binary Linear's output scaling fused into the store, replacing the
  * separate elementwise kernels of `bgemm(...) * sw * sa (+ bias)`
  * (tests/python/bgemm_linear.py:482-484).  Every step is evaluated and rounded exactly as

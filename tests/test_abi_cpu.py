@@ -29,7 +29,7 @@ def test_header_symbols_exported():
 
 def test_layout_sizes():
     L = _lib.lib()
-    assert L.bgemm_abi_version() == _lib.ABI_VERSION == 8
+    assert L.bgemm_abi_version() == _lib.ABI_VERSION == 9
     assert L.bgemm_tiled_words(1, 1) == 256
     assert L.bgemm_tiled_words(32, 256) == 256
     assert L.bgemm_tiled_words(33, 257) == 4 * 256
@@ -124,6 +124,28 @@ def test_dispatch_of_the_benchmark_configurations():
     assert kid(MODE_XOR, 1, 64, 64, 64, 1, force_kernel(8)) == B.EINVAL    # no such kernel
     assert kid(MODE_XOR, 1, 64, 64, 64, 1, force_kernel(B.KERNEL_MFMA_64x64, VARIANT_VALU)) == B.EINVAL
     assert kid(9, 1, 64, 64, 64, 1, A) == B.EINVAL and kid(MODE_XOR, 1, 64, 0, 64, 1, A) == B.EINVAL
+
+
+def test_counted_entry_points_reject_without_touching_the_gpu():
+    """Argument checks of bgemm_row_popcounts and bgemm_packed_forward_counted are host code: every rejection
+    below returns before any launch."""
+    B, L = _lib, _lib.lib()
+    buf = (ctypes.c_char * 64)()
+    p = ctypes.addressof(buf) + (-ctypes.addressof(buf)) % 16
+    assert L.bgemm_row_popcounts(None, 1, 32, 256, 0, p, None) == B.ENULL
+    assert L.bgemm_row_popcounts(p, 1, 32, 256, 0, None, None) == B.ENULL
+    assert L.bgemm_row_popcounts(p + 4, 1, 32, 256, 0, p, None) == B.EALIGN
+    assert L.bgemm_row_popcounts(p, 1, 32, 1 << 24, 0, p, None) == B.EINVAL
+    assert L.bgemm_row_popcounts(p, 2, 32, 256, 4, p, None) == B.EINVAL              # batch stride below one operand
+    assert L.bgemm_row_popcounts(p, 0, 32, 256, 0, None, None) == 0                   # nothing to count
+    fwd = lambda mode, cw, cx, variant: L.bgemm_packed_forward_counted(mode, p, p, cw, cx, p, B.OUT_I32, 1, 32, 32, 256,
+                                                                        0, 0, 1024, variant, None)
+    assert fwd(B.MODE_XOR, None, p, B.VARIANT_AUTO) == B.ENULL
+    assert fwd(B.MODE_XOR, p, p + 2, B.VARIANT_AUTO) == B.EALIGN
+    assert fwd(B.MODE_BWTA, p, p, B.VARIANT_AUTO) in (B.EINVAL, B.ENULL)             # two bit planes: not this entry point
+    assert fwd(B.MODE_XOR, p, p, B.VARIANT_VALU) == B.EINVAL
+    assert L.bgemm_packed_forward_counted(B.MODE_XOR, p, p, p, p, p, B.OUT_F32_SCALED, 1, 32, 32, 256, 0, 0, 1024,
+                                          B.VARIANT_AUTO, None) == B.EINVAL
 
 
 def test_decode_entry_states_its_shapes_and_rejects_others():

@@ -183,6 +183,35 @@ def test_k_of_at_most_two_words_on_every_tile(tile, engine):
 
 
 @pytest.mark.parametrize("engine", list(ENGINES))
+@pytest.mark.parametrize("tile", ["256x256", "256x128", "128x128"])
+def test_row_popcounts_brought_by_the_caller(tile, engine):
+    """bgemm_row_popcounts against numpy, then bgemm_packed_forward_counted: every mode of one bit plane, int32 and
+    fp16, a weight operand shared by a batch of two, ragged M / N / K with an odd K-tile count.  The two pipelined
+    tiles must really use the counts (a count raised by one moves that row's XOR outputs by -2); the other tiles
+    count for themselves and ignore them."""
+    rng = np.random.default_rng(211 + TILES[tile])
+    variant = force_kernel(TILES[tile], ENGINES[engine])
+    M, N, K = 300, 290, 1275
+    w, x = pm1(rng, 1, M, K), pm1(rng, 2, N, K)
+    wp, xp = lk.row_popcounts(lk.pack_sign(to_dev(w))), lk.row_popcounts(lk.pack_sign(to_dev(x)))
+    for p, a in ((wp, w), (xp, x)):
+        assert (p.counts.cpu().numpy() == (a.view(np.uint16) >> 15).sum(-1)).all()
+    for mode in (MODE_AND, MODE_XOR, MODE_ATTN, MODE_ATTN_X):
+        want = dense(mode, w, x)
+        assert (lk.bgemm_packed_forward(wp, xp, mode, torch.int32, 1, variant).cpu().numpy() == want).all(), mode
+        got = lk.bgemm_packed_forward(wp, xp, mode, torch.half, 1, variant).cpu().numpy()
+        assert (bits_of(got) == bits_of(f16_of(want))).all(), mode
+    want = dense(MODE_XOR, w, x)
+    wp.counts[0, 7] += 1
+    xp.counts[1, 11] += 1
+    got = lk.bgemm_packed_forward(wp, xp, MODE_XOR, torch.int32, 1, variant).cpu().numpy()
+    if tile in ("256x256", "256x128"):
+        want[:, :, 7] -= 2
+        want[1, 11, :] -= 2
+    assert (got == want).all()
+
+
+@pytest.mark.parametrize("engine", list(ENGINES))
 @pytest.mark.parametrize("M,N,K,want_kernel", [
     (5907, 5903, 65 * 256 - 5, B.KERNEL_MFMA_256x256),       # the tile of the longest K: ragged edges, 65 K-tiles
     (5907, 5903, 33 * 256 - 5, B.KERNEL_MFMA_256x128),       # the 8192^3 kernel: ragged edges, 33 K-tiles
