@@ -52,7 +52,7 @@ __device__ __forceinline__ int skinny_value(const ModeCoef& mc, const bool two, 
 
 // ---- streaming kernel --------------------------------------------------------------------------
 template <typename Eng, int RT>
-__global__ __launch_bounds__(256) void gemm_skinny_stream_kernel(const GemmArgs a, const int groups)
+__global__ __launch_bounds__(256, 2) void gemm_skinny_stream_kernel(const GemmArgs a, const int groups)
 {
     constexpr int CH = 2;                        // K-tiles per chunk; two chunks are in flight
     const int lane = threadIdx.x & 63;
@@ -208,7 +208,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_stream_kernel(const GemmArgs 
 // the blocks and the weight traffic (64 to 128 rows: 8 to 15 % faster; up to 32 rows the half blocks win by
 // 10 to 20 %, twice the blocks with half the matrix-core chain each).
 template <typename Eng, int KW, bool FUSEX = false, bool PL2 = false>
-__global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 1) void gemm_skinny_splitk_kernel(const GemmArgs a)
+__global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 2) void gemm_skinny_splitk_kernel(const GemmArgs a)
 {
     static_assert(!(FUSEX && PL2), "in-kernel activation packing is built for up to four rows");
     constexpr int NT = KW * 64, NP = PL2 ? 2 : 1;
@@ -595,7 +595,7 @@ __global__ __launch_bounds__(KW * 64) void gemm_skinny_popc_kernel(const GemmArg
 // TWO: a ternary operand; the block's two activation tiles are the two bit planes of ONE tile row (32 rows), so a
 // block is a 32 x 64 piece of the output and the two accumulators of a weight tile combine in the epilogue.
 template <typename Eng, int KW, bool TWO = false>
-__global__ __launch_bounds__(KW * 64) void gemm_skinny_splitk_quad_kernel(const GemmArgs a)
+__global__ __launch_bounds__(KW * 64, 2) void gemm_skinny_splitk_quad_kernel(const GemmArgs a)
 {
     constexpr int NT = KW * 64, CH = 2;
     __shared__ int sAcc[2][2][16][64];           // [weight tile][activation tile], then the MFMA's [v][lane]
