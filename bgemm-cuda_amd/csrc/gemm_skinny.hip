@@ -693,15 +693,30 @@ __global__ __launch_bounds__(KW * 64, 2) void gemm_skinny_splitk_quad_kernel(con
     // ---- rank-one terms and store: a wave takes one output row of the piece, 64 consecutive columns ----
     const ModeCoef mc = a.mc;
     const int kbits = (int)a.K;
-    const int nout = min((int)a.N - nt0 * 32, TWO ? 32 : 64) * 64;
+    // A thread keeps its column (one of the piece's 64, so its weight-row count is read once) and walks the rows
+    // KW apart, four at a time with their LDS reads issued together.
+    const int nrows_out = min((int)a.N - nt0 * 32, TWO ? 32 : 64);
     auto outputs = [&](auto store) {
-        for (int o = threadIdx.x; o < nout; o += NT) {
-            const int mm = o & 63, nn = o >> 6;
-            const int i = mm >> 5, c = mm & 31, j = TWO ? 0 : nn >> 5, nl = nn & 31;
-            const int v = 4 * (nl >> 3) + (nl & 3), hh = (nl >> 2) & 1;       // accumulator slot of operand row nl
-            const int d = sAcc[i][j][v][hh * 32 + c];
-            const int d2 = TWO ? sAcc[i][1][v][hh * 32 + c] : 0, pb2 = TWO ? sPb[1][nl] : 0;
-            store(nt0 * 32 + nn, rt0 * 32 + mm, i, skinny_value(mc, TWO, kbits, sPa[i][c], sPb[j][nl], pb2, d, d2));
+        const int mm = threadIdx.x & 63, i = mm >> 5, c = mm & 31;
+        const int pa_c = sPa[i][c];
+        for (int n0 = threadIdx.x >> 6; n0 < nrows_out; n0 += 4 * KW) {
+            int d[4], d2[4], pbv[4], pb2[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int nn = min(n0 + u * KW, nrows_out - 1);
+                const int j = TWO ? 0 : nn >> 5, nl = nn & 31;
+                const int v = 4 * (nl >> 3) + (nl & 3), hh = (nl >> 2) & 1;   // accumulator slot of operand row nl
+                d[u] = sAcc[i][j][v][hh * 32 + c];
+                d2[u] = TWO ? sAcc[i][1][v][hh * 32 + c] : 0;
+                pbv[u] = sPb[j][nl];
+                pb2[u] = TWO ? sPb[1][nl] : 0;
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int nn = n0 + u * KW;
+                if (nn < nrows_out)
+                    store(nt0 * 32 + nn, rt0 * 32 + mm, i, skinny_value(mc, TWO, kbits, pa_c, pbv[u], pb2[u], d[u], d2[u]));
+            }
         }
     };
     const int64_t out0 = (int64_t)b * a.strideC;
