@@ -119,7 +119,11 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
             const uint4* base = (f < WN ? Xb : Wb) + rt * a.KT * TILE_U4;
             rs[f] = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint4*>(base), 0, a.KT * (TILE_U4 * 16), 0x00020000);
         }
-        unsigned rawA[NF][4], rawB[NF][4], buf[2][NF][4];
+        // Raw K-tiles in flight: two buffers (a K-tile requested one tile ahead of its first use), or three where the
+        // registers allow (two tiles ahead: the 256 x 128 tile's 32 MFMAs a K-tile are half a microsecond, less
+        // than a trip to a far L2 takes under load)
+        constexpr int NBUF = NM == 8 && STEPS == 4 ? 3 : 2;       // (the int8 engine's eight steps a tile leave no registers for it)
+        unsigned rawA[NF][4], rawB[NF][4], rawC[NBUF == 3 ? NF : 1][4], buf[2][NF][4];
         int pop[NF];
 #pragma unroll
         for (int f = 0; f < NF; f++) pop[f] = 0;
@@ -145,21 +149,38 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
 #pragma unroll                                  // because the compiler prefers four counts and two three-way adds
                         for (int c = 0; c < 4; c++) asm("v_bcnt_u32_b32 %0, %1, %0" : "+v"(pop[q]) : "v"(A[q][c]));
                     }
-                    if (s == STEPS - 1 && q < NF) load_frag(A[q], q, kt + 2);   // A is dead after step STEPS-2
+                    if (s == STEPS - 1 && q < NF) load_frag(A[q], q, kt + NBUF);   // A is dead after step STEPS-2
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
         };
         if (kt0 < kt1) {
 #pragma unroll
-            for (int f = 0; f < NF; f++) { load_frag(rawA[f], f, kt0); load_frag(rawB[f], f, kt0 + 1); }
+            for (int f = 0; f < NF; f++) {
+                load_frag(rawA[f], f, kt0); load_frag(rawB[f], f, kt0 + 1);
+                if constexpr (NBUF == 3) load_frag(rawC[f], f, kt0 + 2);
+            }
 #pragma unroll
             for (int f = 0; f < NF; f++)
 #pragma unroll
                 for (int c = 0; c < 4; c++) buf[0][f][c] = f < WN ? Eng::expand1_x(rawA[f][c], 0) : Eng::expand1_w(rawA[f][c], 0);
-            for (int kt = kt0; kt < kt1; kt += 2) {
-                k_tile(rawA, rawB, kt);
-                k_tile(rawB, rawA, kt + 1);
+            if constexpr (NBUF == 3) {
+                // whole rounds of three, then what is left in the same rotation (a K-tile past the range multiplies zeros)
+                int kt = kt0;
+                for (; kt + 3 <= kt1; kt += 3) {
+                    k_tile(rawA, rawB, kt);
+                    k_tile(rawB, rawC, kt + 1);
+                    k_tile(rawC, rawA, kt + 2);
+                }
+                if (kt < kt1) {
+                    k_tile(rawA, rawB, kt);
+                    if (kt + 1 < kt1) k_tile(rawB, rawC, kt + 1);
+                }
+            } else {
+                for (int kt = kt0; kt < kt1; kt += 2) {
+                    k_tile(rawA, rawB, kt);
+                    k_tile(rawB, rawA, kt + 1);
+                }
             }
         }
         if constexpr (COUNTED) {
