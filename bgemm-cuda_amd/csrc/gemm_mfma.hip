@@ -667,9 +667,10 @@ static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int pla
     // columns; int32 output, 32 us for 201 MB, shows no preference)
     if (KT < 4 && out_shift == 1 && M >= 256 && blocks(32, 256) >= 512) return {BGEMM_KERNEL_MFMA_32x256, 32, 256};
     // 256 x 256 (one wave a SIMD, the epilogue in the open) against 256 x 128 (two resident blocks a unit, one
-    // storing while the other multiplies, but half again as many expansions per MFMA): the smaller tile is 2 to 4 %
-    // faster at 32 K-tiles (8192^3: 0.168 against 0.172 ms), the larger one from 64 on (K = 16384: 0.308 against 0.319)
-    if (planes == 1 && blocks(256, 256) >= 512 && KT >= 64) return {BGEMM_KERNEL_MFMA_256x256, 256, 256};
+    // storing while the other multiplies, but half again as many expansions per MFMA).  With operands that come
+    // from HBM the smaller tile wins up to K = 16384 at least (8192^2 x 8192: 173 against 190 us, x 16384: 314 against
+    // 329); with operands that stay in the caches the two tie at K = 16384 and the larger one is 2 % ahead at 32768
+    if (planes == 1 && blocks(256, 256) >= 512 && KT >= 128) return {BGEMM_KERNEL_MFMA_256x256, 256, 256};
     // from two blocks a unit, or from one with 16 K-tiles; a few blocks more than one a unit (11008 x 768 x 4096:
     // 258) would leave the launch waiting for two units that run two blocks each, and go to the next tile down
     const int64_t b21 = blocks(256, 128);

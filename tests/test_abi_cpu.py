@@ -101,7 +101,8 @@ def test_dispatch_of_the_benchmark_configurations():
     TILES = (0, 1, 2, 3, 4, 5, 6, 7)
     A = VARIANT_AUTO
     assert kid(MODE_XOR, 1, 8192, 8192, 8192, 1, A) == B.KERNEL_MFMA_256x128
-    assert kid(MODE_XOR, 1, 8192, 8192, 16384, 1, A) == B.KERNEL_MFMA_256x256
+    assert kid(MODE_XOR, 1, 8192, 8192, 16384, 1, A) == B.KERNEL_MFMA_256x128
+    assert kid(MODE_XOR, 1, 8192, 8192, 32768, 1, A) == B.KERNEL_MFMA_256x256
     assert kid(MODE_XOR, 1, 11008, 768, 4096, 1, A) == B.KERNEL_MFMA_128x128     # 258 blocks of 256 x 128: one too many
     assert kid(MODE_BWTA, 1, 11008, 128, 4096, 1, A) == B.KERNEL_MFMA_32x256
     assert kid(MODE_BWTA, 1, 11008, 64, 4096, 1, A) == B.KERNEL_SKINNY_SPLITK

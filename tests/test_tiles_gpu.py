@@ -213,7 +213,7 @@ def test_row_popcounts_brought_by_the_caller(tile, engine):
 
 @pytest.mark.parametrize("engine", list(ENGINES))
 @pytest.mark.parametrize("M,N,K,want_kernel", [
-    (5907, 5903, 65 * 256 - 5, B.KERNEL_MFMA_256x256),       # the tile of the longest K: ragged edges, 65 K-tiles
+    (5907, 5903, 129 * 256 - 5, B.KERNEL_MFMA_256x256),      # the tile of the longest K: ragged edges, 129 K-tiles
     (5907, 5903, 33 * 256 - 5, B.KERNEL_MFMA_256x128),       # the 8192^3 kernel: ragged edges, 33 K-tiles
     (8195, 2053, 17 * 256 - 7, B.KERNEL_MFMA_256x128),       # the 8192 x 2048 x 4096 kernel likewise
 ])
