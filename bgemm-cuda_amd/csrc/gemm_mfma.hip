@@ -674,7 +674,8 @@ static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int pla
     // from two blocks a unit, or from one with 16 K-tiles; a few blocks more than one a unit (11008 x 768 x 4096:
     // 258) would leave the launch waiting for two units that run two blocks each, and go to the next tile down
     const int64_t b21 = blocks(256, 128);
-    if (planes == 1 && (b21 >= 512 || (KT >= 16 && (b21 == 256 || b21 >= 320 || (b21 > 256 && blocks(128, 128) < 512)))) &&
+    if (planes == 1 && (b21 >= 512 || (KT >= 16 && (b21 == 256 || b21 >= 320 || (b21 > 256 && blocks(128, 128) < 512))) ||
+                        (KT >= 48 && b21 >= 192)) &&       // a long K: even three quarters of a block a unit (8192 x 768 x 16384)
         (KT >= 4 || blocks(128, 128) < 512))
         return {BGEMM_KERNEL_MFMA_256x128, 256, 128};
     if (blocks(128, 128) >= 512) return {BGEMM_KERNEL_MFMA_128x128, 128, 128};
