@@ -671,14 +671,15 @@ static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int pla
     // from HBM the smaller tile wins up to K = 16384 at least (8192^2 x 8192: 173 against 190 us, x 16384: 314 against
     // 329); with operands that stay in the caches the two tie at K = 16384 and the larger one is 2 % ahead at 32768
     if (planes == 1 && blocks(256, 256) >= 512 && KT >= 128) return {BGEMM_KERNEL_MFMA_256x256, 256, 256};
-    // from two blocks a unit, or from one with 16 K-tiles; a few blocks more than one a unit (11008 x 768 x 4096:
-    // 258) would leave the launch waiting for two units that run two blocks each, and go to the next tile down
+    // from two blocks a unit; with 16 K-tiles or more from 160 blocks (0.6 a unit: 11008 x 512 x 8192, 172 blocks, 22.6 us
+    // against 29.6 to 33.2 on the smaller tiles; 8192 x 768 x 4096, 192 blocks, 14.9 against 17.1 to 18.9), except a
+    // few blocks more than one a unit (11008 x 768 x 4096: 258, 11008 x 640 x 8192 likewise), which would leave the
+    // launch waiting for the units that run two blocks each: those go to the next tile down
     const int64_t b21 = blocks(256, 128);
-    if (planes == 1 && (b21 >= 512 || (KT >= 16 && (b21 == 256 || b21 >= 320 || (b21 > 256 && blocks(128, 128) < 512))) ||
-                        (KT >= 48 && b21 >= 192)) &&       // a long K: even three quarters of a block a unit (8192 x 768 x 16384)
+    if (planes == 1 && (b21 >= 512 || (KT >= 16 && b21 >= 160 && !(b21 > 256 && b21 < 320))) &&
         (KT >= 4 || blocks(128, 128) < 512))
         return {BGEMM_KERNEL_MFMA_256x128, 256, 128};
-    if (blocks(128, 128) >= 512) return {BGEMM_KERNEL_MFMA_128x128, 128, 128};
+    if (blocks(128, 128) >= 512 || (planes == 1 && KT >= 16 && b21 > 256 && b21 < 320)) return {BGEMM_KERNEL_MFMA_128x128, 128, 128};
     // two bit planes on few blocks: 32 x 256 shares every weight expansion between the planes of one row tile
     // (W[11008,4096] x 128 ternary rows 9.7 us against 10.9 / 11.3 on the next two), once it has 160 blocks
     if (planes == 2 && blocks(64, 128) < 512 && blocks(32, 256) >= 160) return {BGEMM_KERNEL_MFMA_32x256, 32, 256};

@@ -105,6 +105,10 @@ def test_dispatch_of_the_benchmark_configurations():
     assert kid(MODE_XOR, 1, 8192, 8192, 32768, 1, A) == B.KERNEL_MFMA_256x256
     assert kid(MODE_XOR, 1, 11008, 768, 4096, 1, A) == B.KERNEL_MFMA_128x128     # 258 blocks of 256 x 128: one too many
     assert kid(MODE_BWTA, 1, 11008, 128, 4096, 1, A) == B.KERNEL_MFMA_32x256
+    assert kid(MODE_XOR, 1, 11008, 512, 8192, 1, A) == B.KERNEL_MFMA_256x128     # 172 blocks: 0.67 a unit is enough
+    assert kid(MODE_XOR, 1, 11008, 640, 8192, 1, A) == B.KERNEL_MFMA_128x128     # 258 again
+    assert kid(MODE_XOR, 1, 8192, 768, 16384, 1, A) == B.KERNEL_MFMA_256x128
+    assert kid(MODE_XOR, 1, 8192, 512, 16384, 1, A) == B.KERNEL_SKINNY_QUAD
     assert kid(MODE_BWTA, 1, 11008, 64, 4096, 1, A) == B.KERNEL_SKINNY_SPLITK
     assert kid(MODE_XOR, 1, 8192, 2048, 4096, 1, A) == B.KERNEL_MFMA_256x128
     assert kid(MODE_XOR, 1, 8192, 2048, 16384, 4, A) == B.KERNEL_MFMA_256x128
