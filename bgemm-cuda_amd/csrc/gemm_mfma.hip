@@ -661,29 +661,35 @@ struct MfmaCfg { int id, bn, bm; };
 static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int planes, int out_shift)
 {
     auto blocks = [&](int bn, int bm) { return batch * cdiv(N, bn) * cdiv(M, bm); };
+    // the share of a tiling's MFMA work that lands on real outputs: a batch of [1024 x 64] outputs would fill a quarter
+    // of its 256-row tiles (74 us against 32 on a tile that fits, for 384 of them with K = 2048)
+    auto filled = [&](int bn, int bm) { return (double)(N * M) / (double)(cdiv(N, bn) * bn * cdiv(M, bm) * bm); };
     if (M <= 64) return blocks(128, 64) >= 1024 ? MfmaCfg{BGEMM_KERNEL_MFMA_128x64, 128, 64} : MfmaCfg{BGEMM_KERNEL_MFMA_64x64, 64, 64};   // narrow outputs
     // a short K with a 2-byte output is all store path: rows of 512 bytes per block, many blocks in flight
     // (192 x [512 x 512] x 64 -> fp16: 19.4 us against 20.4 on 128 x 128 and 25 to 29 on the tiles without paired
     // columns; int32 output, 32 us for 201 MB, shows no preference)
-    if (KT < 4 && out_shift == 1 && M >= 256 && blocks(32, 256) >= 512) return {BGEMM_KERNEL_MFMA_32x256, 32, 256};
+    // (one K-tile only: from two on, 128 x 128 is 15 % ahead: 48 x [1024 x 512] x 512 -> fp16 13.3 against 15.6 us)
+    if (KT < 2 && out_shift == 1 && M >= 256 && blocks(32, 256) >= 512) return {BGEMM_KERNEL_MFMA_32x256, 32, 256};
     // 256 x 256 (one wave a SIMD, the epilogue in the open) against 256 x 128 (two resident blocks a unit, one
     // storing while the other multiplies, but half again as many expansions per MFMA).  With operands that come
     // from HBM the smaller tile wins up to K = 16384 at least (8192^2 x 8192: 173 against 190 us, x 16384: 314 against
     // 329); with operands that stay in the caches the two tie at K = 16384 and the larger one is 2 % ahead at 32768
-    if (planes == 1 && blocks(256, 256) >= 512 && KT >= 128) return {BGEMM_KERNEL_MFMA_256x256, 256, 256};
+    if (planes == 1 && blocks(256, 256) >= 512 && KT >= 128 && filled(256, 256) >= 0.8) return {BGEMM_KERNEL_MFMA_256x256, 256, 256};
     // from two blocks a unit; with 16 K-tiles or more from 160 blocks (0.6 a unit: 11008 x 512 x 8192, 172 blocks, 22.6 us
     // against 29.6 to 33.2 on the smaller tiles; 8192 x 768 x 4096, 192 blocks, 14.9 against 17.1 to 18.9), except a
     // few blocks more than one a unit (11008 x 768 x 4096: 258, 11008 x 640 x 8192 likewise), which would leave the
     // launch waiting for the units that run two blocks each: those go to the next tile down
     const int64_t b21 = blocks(256, 128);
     if (planes == 1 && (b21 >= 512 || (KT >= 16 && b21 >= 160 && !(b21 > 256 && b21 < 320))) &&
-        (KT >= 4 || blocks(128, 128) < 512))
+        (KT >= (out_shift == 1 ? 8 : 4) || blocks(128, 128) < 512) &&      // (2-byte outputs leave 128 x 128 without staging in LDS:
+        filled(256, 128) >= 0.75)                                          //  48 x [2048 x 2048] x 1024 -> fp16 117 against 131 us)
         return {BGEMM_KERNEL_MFMA_256x128, 256, 128};
-    if (blocks(128, 128) >= 512 || (planes == 1 && KT >= 16 && b21 > 256 && b21 < 320)) return {BGEMM_KERNEL_MFMA_128x128, 128, 128};
+    if ((blocks(128, 128) >= 512 || (planes == 1 && KT >= 16 && b21 > 256 && b21 < 320)) && filled(128, 128) >= 0.6)
+        return {BGEMM_KERNEL_MFMA_128x128, 128, 128};
     // two bit planes on few blocks: 32 x 256 shares every weight expansion between the planes of one row tile
     // (W[11008,4096] x 128 ternary rows 9.7 us against 10.9 / 11.3 on the next two), once it has 160 blocks
     if (planes == 2 && blocks(64, 128) < 512 && blocks(32, 256) >= 160) return {BGEMM_KERNEL_MFMA_32x256, 32, 256};
-    if (blocks(64, 128) >= 512) return {BGEMM_KERNEL_MFMA_64x128, 64, 128};      // below two blocks a unit, twice as many 32-row tiles are faster
+    if (blocks(64, 128) >= 512 && filled(64, 128) >= 0.6) return {BGEMM_KERNEL_MFMA_64x128, 64, 128};      // below two blocks a unit, twice as many 32-row tiles are faster
     return {BGEMM_KERNEL_MFMA_32x128, 32, 128};
 }
 
