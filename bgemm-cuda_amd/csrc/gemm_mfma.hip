@@ -686,9 +686,10 @@ static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int pla
         return {BGEMM_KERNEL_MFMA_256x128, 256, 128};
     if ((blocks(128, 128) >= 512 || (planes == 1 && KT >= 16 && b21 > 256 && b21 < 320)) && filled(128, 128) >= 0.6)
         return {BGEMM_KERNEL_MFMA_128x128, 128, 128};
-    // two bit planes on few blocks: 32 x 256 shares every weight expansion between the planes of one row tile
-    // (W[11008,4096] x 128 ternary rows 9.7 us against 10.9 / 11.3 on the next two), once it has 160 blocks
-    if (planes == 2 && blocks(64, 128) < 512 && blocks(32, 256) >= 160) return {BGEMM_KERNEL_MFMA_32x256, 32, 256};
+    // two bit planes: 32 x 256 shares every weight expansion between the planes of one row tile (W[11008,4096] x 128
+    // ternary rows 9.7 us against 10.9 / 11.3 on the next two; W[12288,11008] x 384 rows 47.4 against 55.7), once it
+    // has 160 blocks
+    if (planes == 2 && blocks(32, 256) >= 160) return {BGEMM_KERNEL_MFMA_32x256, 32, 256};
     if (blocks(64, 128) >= 512 && filled(64, 128) >= 0.6) return {BGEMM_KERNEL_MFMA_64x128, 64, 128};      // below two blocks a unit, twice as many 32-row tiles are faster
     return {BGEMM_KERNEL_MFMA_32x128, 32, 128};
 }
