@@ -106,6 +106,10 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
         constexpr int NF = WN + WM, ND = NF * 4, NM = WN * WM, STEPS = Eng::STEPS;
         static_assert(ND % NM == 0 && NF <= NM && STEPS % 2 == 0, "tile shape does not pipeline");
         constexpr int DPG = ND / NM;                       // expanded registers produced per MFMA
+        // Both operands have one layout and the two expansions are each other's mirror (every product of set bits
+        // is 1 either way round), so the side with more fragments a wave gets the cheaper one (five instructions a
+        // word against six): the activation side's four fragments on the 256 x 128 tile.
+        constexpr bool XS_FIRST = WN <= WM;                // true: activation fragments take the activation-side expansion
         // Every fragment's row of K-tiles is a buffer of its own (a wave-uniform base in scalar registers, KT KiB
         // long), so all loads of a K-tile share ONE per-lane offset, lane * 16 + kt * 1024: no address arithmetic
         // per load, and K-tiles past the range read as zero bits (a buffer load out of range returns 0; zero bits
@@ -142,7 +146,7 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
                     acc[0][i][j] = Eng::mma(Eng::make(cur[i]), Eng::make(cur[WN + j]), acc[0][i][j]);
 #pragma unroll
                     for (int d = q * DPG; d < (q + 1) * DPG; d++)
-                        nxt[d / 4][d % 4] = d / 4 < WN      // fragments 0 .. WN-1 are the activation side
+                        nxt[d / 4][d % 4] = (d / 4 < WN) == XS_FIRST      // fragments 0 .. WN-1 are the activation side
                             ? (s + 1 < STEPS ? Eng::expand1_x(A[d / 4][d % 4], s + 1) : Eng::expand1_x(B[d / 4][d % 4], 0))
                             : (s + 1 < STEPS ? Eng::expand1_w(A[d / 4][d % 4], s + 1) : Eng::expand1_w(B[d / 4][d % 4], 0));
                     if (!COUNTED && s == 0 && q < NF) {     // v_bcnt adds into its accumulator: four instructions a fragment, written out
@@ -163,7 +167,7 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
 #pragma unroll
             for (int f = 0; f < NF; f++)
 #pragma unroll
-                for (int c = 0; c < 4; c++) buf[0][f][c] = f < WN ? Eng::expand1_x(rawA[f][c], 0) : Eng::expand1_w(rawA[f][c], 0);
+                for (int c = 0; c < 4; c++) buf[0][f][c] = (f < WN) == XS_FIRST ? Eng::expand1_x(rawA[f][c], 0) : Eng::expand1_w(rawA[f][c], 0);
             if constexpr (NBUF == 3) {
                 // whole rounds of three, then what is left in the same rotation (a K-tile past the range multiplies zeros)
                 int kt = kt0;
