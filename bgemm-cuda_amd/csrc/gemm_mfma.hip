@@ -216,6 +216,8 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
 #pragma unroll
     for (int j = 0; j < WM; j++) wn_[j] = wp[j][(int64_t)kt0 * TILE_U4];
     const bool two_words = a.K <= 64;
+    // (the two expansions mirror each other, so the side with more fragments a wave takes the cheaper one)
+    constexpr bool XS_FIRST = WN * PL <= WM;
     auto k_tile = [&](auto first_c, auto two_c, const int kt) {
         constexpr bool FIRST = decltype(first_c)::value, TWO = decltype(two_c)::value;
 #pragma unroll
@@ -246,12 +248,15 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
         for (int s = 0; s < Eng::STEPS; s++) {
             typename Eng::Frag bw[WM];
 #pragma unroll
-            for (int j = 0; j < WM; j++) bw[j] = TWO ? Eng::expand_w2(wf[j], s) : Eng::expand_w(wf[j], s);
+            for (int j = 0; j < WM; j++)
+                bw[j] = XS_FIRST ? (TWO ? Eng::expand_w2(wf[j], s) : Eng::expand_w(wf[j], s))
+                                 : (TWO ? Eng::expand_x2(wf[j], s) : Eng::expand_x(wf[j], s));
 #pragma unroll
             for (int p = 0; p < PL; p++)
 #pragma unroll
                 for (int i = 0; i < WN; i++) {
-                    const typename Eng::Frag ax = TWO ? Eng::expand_x2(xf[p][i], s) : Eng::expand_x(xf[p][i], s);
+                    const typename Eng::Frag ax = XS_FIRST ? (TWO ? Eng::expand_x2(xf[p][i], s) : Eng::expand_x(xf[p][i], s))
+                                                           : (TWO ? Eng::expand_w2(xf[p][i], s) : Eng::expand_w(xf[p][i], s));
 #pragma unroll
                     for (int j = 0; j < WM; j++) acc[p][i][j] = Eng::mma(ax, bw[j], FIRST && s == 0 ? zero : acc[p][i][j]);
                 }
