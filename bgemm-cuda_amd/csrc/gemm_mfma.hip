@@ -55,6 +55,13 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
     // out with 10 to 25 % more registers (113 against 89 for the 64 x 128 tile: three waves a SIMD instead of four).
   auto do_tile = [&](const int tn) {
     const int nt0 = (tn * WGN + wn) * WN;
+    // Pipelined tiles: the two waves of a block that share their activation fragments (same wn) keep them in
+    // slots rotated by half against each other, slot i of wave wm holding tile row nt0 + (i ^ xs): each wave then
+    // counts the bits of its first WN / 2 slots only, which are different rows for the two, and they swap the
+    // counts through LDS before the epilogue (half the activation side's popcounts: 0.25 vector instructions a MFMA).
+    static_assert(!PIPE || (WGM == 2 && WN % 2 == 0), "the popcount split is laid out for two waves along M");
+    const int xs = PIPE ? wm * (WN / 2) : 0;
+    auto x_tile = [&](const int i) { return nt0 + (i ^ xs); };
 
     // per-fragment base pointers (row tile clamped so ragged edges re-read a valid tile)
     const uint4* xp[PL][WN];
@@ -119,7 +126,7 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
         __amdgpu_buffer_rsrc_t rs[NF];
 #pragma unroll
         for (int f = 0; f < NF; f++) {
-            const int64_t rt = f < WN ? min(nt0 + f, a.NT - 1) : min(mt0 + (f - WN), a.MT - 1);
+            const int64_t rt = f < WN ? min(x_tile(f), a.NT - 1) : min(mt0 + (f - WN), a.MT - 1);
             const uint4* base = (f < WN ? Xb : Wb) + rt * a.KT * TILE_U4;
             rs[f] = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint4*>(base), 0, a.KT * (TILE_U4 * 16), 0x00020000);
         }
@@ -149,7 +156,7 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
                         nxt[d / 4][d % 4] = (d / 4 < WN) == XS_FIRST      // fragments 0 .. WN-1 are the activation side
                             ? (s + 1 < STEPS ? Eng::expand1_x(A[d / 4][d % 4], s + 1) : Eng::expand1_x(B[d / 4][d % 4], 0))
                             : (s + 1 < STEPS ? Eng::expand1_w(A[d / 4][d % 4], s + 1) : Eng::expand1_w(B[d / 4][d % 4], 0));
-                    if (!COUNTED && s == 0 && q < NF) {     // v_bcnt adds into its accumulator: four instructions a fragment, written out
+                    if (!COUNTED && s == 0 && (q < WN / 2 || (q >= WN && q < NF))) {     // v_bcnt adds into its accumulator: four instructions a fragment, written out
 #pragma unroll                                  // because the compiler prefers four counts and two three-way adds
                         for (int c = 0; c < 4; c++) asm("v_bcnt_u32_b32 %0, %1, %0" : "+v"(pop[q]) : "v"(A[q][c]));
                     }
@@ -192,14 +199,22 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
             // their outputs are never stored); halved below by nothing: these are whole rows, not K-halves
             const int64_t cx = a.strideX ? (int64_t)b * a.N : 0, cw = a.strideW ? (int64_t)b * a.M : 0;
 #pragma unroll
-            for (int i = 0; i < WN; i++) pb[0][i] = a.cntX[cx + min((int64_t)(nt0 + i) * 32 + (lane & 31), a.N - 1)];
+            for (int i = 0; i < WN; i++) pb[0][i] = a.cntX[cx + min((int64_t)x_tile(i) * 32 + (lane & 31), a.N - 1)];
 #pragma unroll
             for (int j = 0; j < WM; j++) pa[j] = a.cntW[cw + min((int64_t)(mt0 + j) * 32 + (lane & 31), a.M - 1)];
         } else {
+            // the two K-halves of a row meet, then the two waves that share these rows exchange what each counted
+            __shared__ int xcnt[WGN][WN][32];
 #pragma unroll
-            for (int i = 0; i < WN; i++) pb[0][i] = pop[i];
+            for (int i = 0; i < WN / 2; i++) {
+                const int n = pop[i] + __shfl_xor(pop[i], 32);
+                if (lane < 32) xcnt[wn][i ^ xs][lane] = n;
+            }
+            __syncthreads();
 #pragma unroll
-            for (int j = 0; j < WM; j++) pa[j] = pop[WN + j];
+            for (int i = 0; i < WN; i++) pb[0][i] = xcnt[wn][i ^ xs][lane & 31];
+#pragma unroll
+            for (int j = 0; j < WM; j++) pa[j] = pop[WN + j] + __shfl_xor(pop[WN + j], 32);
         }
     } else {
     // ---- main loop: raw tiles are prefetched one K-tile ahead ----------------------------------
@@ -270,7 +285,7 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
 
     // ---- epilogue: rank-one terms turn the AND-dot into C -----------------------------------------
     const int bits = (int)a.K;
-    if constexpr (!COUNTED) {        // a lane counted its K-half of the row
+    if constexpr (!COUNTED && !PIPE) {        // a lane counted its K-half of the row (the pipelined loop has summed already)
 #pragma unroll
         for (int j = 0; j < WM; j++) pa[j] += __shfl_xor(pa[j], 32);
 #pragma unroll
@@ -336,8 +351,8 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
         auto rows_out = [&](auto past_cache) {
 #pragma unroll
             for (int i = 0; i < WN; i++) {
-                const int64_t nrow0 = (int64_t)(nt0 + i) * 32;
-                if (nrow0 >= a.N) break;                          // the whole strip lies past the last row
+                const int64_t nrow0 = (int64_t)x_tile(i) * 32;
+                if (nrow0 >= a.N) continue;                       // the whole strip lies past the last row
                 int val[WM][16];
                 tile_row_vals(i, val);
                 auto put = [&](int* const to, const int v) {
@@ -391,8 +406,8 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
             const uint32_t voff = (uint32_t)(half * 4 * row_b + col * 4);
 #pragma unroll
             for (int i = 0; i < WN; i++) {
-                const int64_t nrow0 = (int64_t)(nt0 + i) * 32;
-                if (nrow0 >= a.N) break;                          // the whole strip lies past the last row
+                const int64_t nrow0 = (int64_t)x_tile(i) * 32;
+                if (nrow0 >= a.N) continue;                       // the whole strip lies past the last row
                 int4 r4[4];
 #pragma unroll
                 for (int g = 0; g < 4; g++) r4[g] = *reinterpret_cast<const int4*>(rp + i * 32 + 8 * g + 4 * half);
@@ -458,8 +473,8 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
         const int64_t m = (int64_t)mt0 * 32 + c8 * 8;
 #pragma unroll
         for (int i = 0; i < WN; i++) {
-            const int64_t nrow0 = (int64_t)(nt0 + i) * 32;
-            if (nrow0 >= a.N) break;                              // the whole strip lies past the last row
+            const int64_t nrow0 = (int64_t)x_tile(i) * 32;
+            if (nrow0 >= a.N) continue;                           // the whole strip lies past the last row
             int val[WM][16];
             tile_row_vals(i, val);
 #pragma unroll
@@ -488,7 +503,7 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
 #pragma unroll
             for (int j = 0; j < WM; j++) st[(8 * (v >> 2) + 4 * half + (v & 3)) * ROW_I + j * 32 + col] = val[j][v];
         wave_sync();
-        const int64_t nrow0 = (int64_t)(nt0 + i) * 32, mcol0 = (int64_t)mt0 * 32;
+        const int64_t nrow0 = (int64_t)x_tile(i) * 32, mcol0 = (int64_t)mt0 * 32;
         constexpr int C4 = WM * 8;               // int4 per staged row
         constexpr int NP = 32 * C4 / 64;
         if (a.vec_store && a.out_kind == BGEMM_OUT_I32) {
