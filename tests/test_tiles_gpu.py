@@ -124,6 +124,23 @@ def test_each_tile_every_output_kind(oracle, tile, engine, M):
     check_all_kinds(oracle, wp, xp, dense(MODE_XOR, w, x), M, N, variant, rng)
 
 
+@pytest.mark.parametrize("M", [520, 517])
+@pytest.mark.parametrize("engine", list(ENGINES))
+def test_128x128_takes_the_pipelined_loop_from_eight_k_tiles(oracle, engine, M):
+    """From eight K-tiles on the 128 x 128 tile runs the hand-pipelined loop (except for fp16 pairs, which stay on the
+    plain one): nine K-tiles, the last ragged, every output kind, ragged M and N; and with the operands' row
+    popcounts brought along."""
+    N, K = 515, 9 * 256 - 5
+    rng = np.random.default_rng(M * 17 + 5)
+    w, x = pm1(rng, M, K), pm1(rng, N, K)
+    wp, xp = lk.pack_sign(to_dev(w)), lk.pack_sign(to_dev(x))
+    variant = force_kernel(TILES["128x128"], ENGINES[engine])
+    acc = dense(MODE_XOR, w, x)
+    check_all_kinds(oracle, wp, xp, acc, M, N, variant, rng)
+    lk.row_popcounts(wp), lk.row_popcounts(xp)
+    assert (lk.bgemm_packed_forward(wp, xp, MODE_XOR, torch.int32, 1, variant)[0].cpu().numpy() == acc).all()
+
+
 @pytest.mark.parametrize("engine", list(ENGINES))
 @pytest.mark.parametrize("tile", list(TILES))
 def test_each_tile_every_mode_batched(tile, engine):
