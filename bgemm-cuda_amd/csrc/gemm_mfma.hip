@@ -704,11 +704,18 @@ static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int pla
     // few blocks more than one a unit (11008 x 768 x 4096: 258, 11008 x 640 x 8192 likewise), which would leave the
     // launch waiting for the units that run two blocks each: those go to the next tile down
     const int64_t b21 = blocks(256, 128);
-    if (planes == 1 && (b21 >= 512 || (KT >= 16 && b21 >= 160 && !(b21 > 256 && b21 < 320))) &&
+    // a last round that leaves most of the GPU idle (576 blocks on 512 places: 6144 x 3072 x 4096 42.5 us against 34.9 on
+    // 128 x 128, whose 1152 blocks fill one and a half rounds of 768 places) goes to the smaller tile
+    auto round_fill = [](int64_t b, int64_t places) { return (double)b / (double)(cdiv(b, places) * places); };
+    const bool last_round_idle = KT >= 8 && KT <= 16 && b21 > 256 &&      // (on a longer K the larger tile's cheaper loop makes up for it)
+                                 round_fill(blocks(128, 128), 768) >= round_fill(b21, 512) + 0.18 &&
+                                 filled(128, 128) >= 0.6;
+    if (planes == 1 && !last_round_idle && (b21 >= 512 || (KT >= 16 && b21 >= 160 && !(b21 > 256 && b21 < 320))) &&
         (KT >= (out_shift == 1 ? 8 : 4) || blocks(128, 128) < 512) &&      // (2-byte outputs leave 128 x 128 without staging in LDS:
         filled(256, 128) >= 0.75)                                          //  48 x [2048 x 2048] x 1024 -> fp16 117 against 131 us)
         return {BGEMM_KERNEL_MFMA_256x128, 256, 128};
-    if ((blocks(128, 128) >= 512 || (planes == 1 && KT >= 16 && b21 > 256 && b21 < 320)) && filled(128, 128) >= 0.6)
+    // (with its pipelined loop, from eight K-tiles on, 192 blocks are enough: 3072 x 1024 x 8192 15.9 us against 17.3 to 20.1)
+    if ((blocks(128, 128) >= 512 || (planes == 1 && KT >= 8 && blocks(128, 128) >= 192)) && filled(128, 128) >= 0.6)
         return {BGEMM_KERNEL_MFMA_128x128, 128, 128};
     // two bit planes: 32 x 256 shares every weight expansion between the planes of one row tile (W[11008,4096] x 128
     // ternary rows 9.7 us against 10.9 / 11.3 on the next two; W[12288,11008] x 384 rows 47.4 against 55.7), once it
