@@ -289,6 +289,31 @@ def test_narrow_outputs_ragged_batch():
     assert (bits_of(got) == bits_of(f16_of(dense(MODE_AND, w, x)))).all()
 
 
+@pytest.mark.parametrize("engine", list(ENGINES))
+def test_stream_kernel_up_to_four_rows_one_store_a_row(engine):
+    """The streaming decode kernel writes a row's 64 outputs of a wave's two weight tiles as one store when there are
+    at most four rows: every row count from 1 to 5 (5: the other path), sign and ternary activations, a weight matrix
+    whose last tile pair is incomplete (M = 100: tiles 2 and 3, the last with four rows) and one with an odd number
+    of tiles (M = 90), int32 and fp16."""
+    rng = np.random.default_rng(977)
+    variant = force_kernel(B.KERNEL_SKINNY_STREAM, ENGINES[engine])
+    for M in (100, 90, 128):
+        Bn, K = 1100, 300
+        w = pm1(rng, Bn, M, K)
+        wp = lk.pack_sign(to_dev(w))
+        for N in (1, 2, 3, 4, 5):
+            x = pm1(rng, 1, N, K)
+            x[rng.random(x.shape) < 0.3] = 0
+            xp, xt = lk.pack_sign(to_dev(x)), lk.pack_ternary(to_dev(x))
+            for mode, xop in ((MODE_XOR, xp), (MODE_BWTA, xt)):
+                assert lk.packed_kernel_id(wp, xop, mode, 1, variant) == B.KERNEL_SKINNY_STREAM
+                want = dense(mode, w, x)
+                got = lk.bgemm_packed_forward(wp, xop, mode, torch.int32, 1, variant).cpu().numpy()
+                assert (got == want).all(), (M, N, mode)
+                got = lk.bgemm_packed_forward(wp, xop, mode, torch.half, 1, variant).cpu().numpy()
+                assert (bits_of(got) == bits_of(f16_of(want))).all(), (M, N, mode)
+
+
 @pytest.mark.parametrize("N,want_kernel", [(256, B.KERNEL_SKINNY_QUAD), (2048, B.KERNEL_MFMA_256x128)])
 def test_config5_sweep_long_k(N, want_kernel):
     """The K = 16384 points of configuration 5's sweep, split-K 1 / 2 / 4: sampled rows and columns against the
