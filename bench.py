@@ -536,6 +536,8 @@ THRESHOLD_SHAPES = [
     # under one 256 x 128 block a unit, and a few more than one
     (1, 1, 8192, 768, 8192), (1, 1, 8192, 768, 4096), (1, 1, 11008, 512, 8192), (1, 1, 5120, 1024, 8192), (1, 1, 11008, 640, 8192),
     (1, 1, 4096, 1024, 4096), (1, 1, 8192, 512, 16384),
+    # a short K into int32 rows of a power of two in bytes, and the same beside a power of two
+    (1, 1, 2048, 4096, 1024), (1, 1, 2000, 4000, 1024), (1, 1, 4096, 2048, 1024), (1, 1, 8192, 1024, 1024),
     (1, 1, 4096, 256, 4096), (1, 1, 11008, 128, 4096), (1, 1, 4096, 384, 4096), (1, 1, 2048, 256, 16384),
     (1, 1, 256, 256, 16384), (1, 1, 4096, 128, 4096), (1, 192, 512, 512, 64), (1, 192, 64, 512, 512),
     (2, 1, 11008, 32, 4096), (2, 1, 11008, 64, 4096), (2, 1, 11008, 128, 4096), (2, 1, 4096, 128, 11008),

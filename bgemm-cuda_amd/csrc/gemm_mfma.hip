@@ -694,6 +694,14 @@ static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int pla
     // columns; int32 output, 32 us for 201 MB, shows no preference)
     // (one K-tile only: from two on, 128 x 128 is 15 % ahead: 48 x [1024 x 512] x 512 -> fp16 13.3 against 15.6 us)
     if (KT < 2 && out_shift == 1 && M >= 256 && blocks(32, 256) >= 512) return {BGEMM_KERNEL_MFMA_32x256, 32, 256};
+    // a short K with int32 rows of a power of two in bytes (4 to 32 KiB): the few large blocks of such a launch all
+    // run in step, and the rows they store at one moment lie a multiple of 1 MiB apart, on few memory channels;
+    // four times as many 32-row blocks drift apart (2048 x 4096 x 1024: 9.5 us against 12.6 on 128 x 128, 4096 x 2048 x
+    // 1024: 9.5 against 11.3, 8192 x 1024 x 1024: 9.8 against 11.2; 2000 x 4000 x 1024 shows no difference).  Up to 64 MiB
+    // of output; beyond, the larger tiles' rounds have drifted apart as well.
+    if (batch == 1 && planes == 1 && out_shift == 2 && KT <= 6 && M >= 1024 && M <= 8192 && (M & (M - 1)) == 0 &&
+        N * M <= (16 << 20) && blocks(32, 256) >= 512)
+        return {BGEMM_KERNEL_MFMA_32x256, 32, 256};
     // 256 x 256 (one wave a SIMD, the epilogue in the open) against 256 x 128 (two resident blocks a unit, one
     // storing while the other multiplies, but half again as many expansions per MFMA).  With operands that come
     // from HBM the smaller tile wins up to K = 16384 at least (8192^2 x 8192: 173 against 190 us, x 16384: 314 against

@@ -233,6 +233,7 @@ def test_row_popcounts_brought_by_the_caller(tile, engine):
     (5907, 5903, 129 * 256 - 5, B.KERNEL_MFMA_256x256),      # the tile of the longest K: ragged edges, 129 K-tiles
     (5907, 5903, 33 * 256 - 5, B.KERNEL_MFMA_256x128),       # the 8192^3 kernel: ragged edges, 33 K-tiles
     (8195, 2053, 17 * 256 - 7, B.KERNEL_MFMA_256x128),       # the 8192 x 2048 x 4096 kernel likewise
+    (2048, 3997, 5 * 256 - 5, B.KERNEL_MFMA_32x256),         # int32 rows of 8 KiB on a short K: the 32-row tile
 ])
 def test_headline_tiles_where_the_library_picks_them(oracle, engine, M, N, K, want_kernel):
     """No forcing: shapes that the library itself sends to the two large tiles, ragged in M, N and K with an odd
@@ -246,6 +247,7 @@ def test_headline_tiles_where_the_library_picks_them(oracle, engine, M, N, K, wa
     assert lk.packed_kernel_id(wp, xp, MODE_XOR, 1, variant) == want_kernel
     rows = np.unique(np.concatenate([rng.choice(N, 90, replace=False), [0, N - 1, N - 2, (N // 32) * 32, (N // 256) * 256]]))
     cols = np.unique(np.concatenate([rng.choice(M, 120, replace=False), [0, M - 1, M - 2, (M // 32) * 32, (M // 128) * 128]]))
+    rows, cols = rows[rows < N], cols[cols < M]               # (a size that is a whole number of tiles has no ragged tile)
     wsub = w16[torch.from_numpy(cols).to(DEV)].float().cpu()
     xsub = x16[torch.from_numpy(rows).to(DEV)].float().cpu()
     acc = (xsub @ wsub.T).to(torch.int32).numpy()
