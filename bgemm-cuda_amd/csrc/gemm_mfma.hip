@@ -694,31 +694,34 @@ static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int pla
     // columns; int32 output, 32 us for 201 MB, shows no preference)
     // (one K-tile only: from two on, 128 x 128 is 15 % ahead: 48 x [1024 x 512] x 512 -> fp16 13.3 against 15.6 us)
     if (KT < 2 && out_shift == 1 && M >= 256 && blocks(32, 256) >= 512) return {BGEMM_KERNEL_MFMA_32x256, 32, 256};
-    // a short K with int32 rows of a power of two in bytes (4 to 32 KiB): the few large blocks of such a launch all
+    // a short K with int32 rows of a power of two in bytes (4 to 64 KiB): the few large blocks of such a launch all
     // run in step, and the rows they store at one moment lie a multiple of 1 MiB apart, on few memory channels;
     // four times as many 32-row blocks drift apart (2048 x 4096 x 1024: 9.5 us against 12.6 on 128 x 128, 4096 x 2048 x
-    // 1024: 9.5 against 11.3, 8192 x 1024 x 1024: 9.8 against 11.2; 2000 x 4000 x 1024 shows no difference).  Up to 64 MiB
-    // of output; beyond, the larger tiles' rounds have drifted apart as well.
-    if (batch == 1 && planes == 1 && out_shift == 2 && KT <= 6 && M >= 1024 && M <= 8192 && (M & (M - 1)) == 0 &&
-        N * M <= (16 << 20) && blocks(32, 256) >= 512)
+    // 1024: 9.5 against 11.3, 16384 x 1024 x 1024: 17.7 against 21.9 on 256 x 128; 2000 x 4000 x 1024 shows no difference).
+    // From 1024 such blocks, up to 64 MiB of output; beyond, the larger tiles' rounds have drifted apart as well.
+    if (batch == 1 && planes == 1 && out_shift == 2 && KT <= 6 && M >= 1024 && M <= 16384 && (M & (M - 1)) == 0 &&
+        N * M <= (16 << 20) && blocks(32, 256) >= 1024)
         return {BGEMM_KERNEL_MFMA_32x256, 32, 256};
     // 256 x 256 (one wave a SIMD, the epilogue in the open) against 256 x 128 (two resident blocks a unit, one
     // storing while the other multiplies, but half again as many expansions per MFMA).  With operands that come
     // from HBM the smaller tile wins up to K = 16384 at least (8192^2 x 8192: 173 against 190 us, x 16384: 314 against
     // 329); with operands that stay in the caches the two tie at K = 16384 and the larger one is 2 % ahead at 32768
     if (planes == 1 && blocks(256, 256) >= 512 && KT >= 128 && filled(256, 256) >= 0.8) return {BGEMM_KERNEL_MFMA_256x256, 256, 256};
-    // from two blocks a unit; with 16 K-tiles or more from 160 blocks (0.6 a unit: 11008 x 512 x 8192, 172 blocks, 22.6 us
-    // against 29.6 to 33.2 on the smaller tiles; 8192 x 768 x 4096, 192 blocks, 14.9 against 17.1 to 18.9), except a
-    // few blocks more than one a unit (11008 x 768 x 4096: 258, 11008 x 640 x 8192 likewise), which would leave the
-    // launch waiting for the units that run two blocks each: those go to the next tile down
+    // from two blocks a unit; with 16 K-tiles or more from 132 blocks, i.e. as soon as the next tile down no longer has
+    // a unit to itself for every block (11008 x 512 x 8192, 172 blocks, 22.6 us against 29.6 to 33.2 on the smaller tiles;
+    // 8192 x 768 x 4096, 192 blocks, 14.9 against 17.1 to 18.9; 4352 x 1024 x 8192, 136 blocks, 21.1 against 23.9; but
+    // 2560 x 1536 x 8192, 120 blocks, 21.0 against 16.5 on 240 blocks of 128 x 128), except from a few blocks more than one
+    // a unit (11008 x 768 x 4096: 258, 11008 x 640 x 8192 likewise) to one and a half (6144 x 2048 x 16384: 384 blocks, 72.6
+    // against 71.3), which would leave the launch waiting for the units that run two blocks each while three blocks of
+    // the next tile down fit every unit at once: those go to the next tile down
     const int64_t b21 = blocks(256, 128);
     // a last round that leaves most of the GPU idle (576 blocks on 512 places: 6144 x 3072 x 4096 42.5 us against 34.9 on
     // 128 x 128, whose 1152 blocks fill one and a half rounds of 768 places) goes to the smaller tile
     auto round_fill = [](int64_t b, int64_t places) { return (double)b / (double)(cdiv(b, places) * places); };
     const bool last_round_idle = KT >= 8 && KT <= 16 && b21 > 256 &&      // (on a longer K the larger tile's cheaper loop makes up for it)
-                                 round_fill(blocks(128, 128), 768) >= round_fill(b21, 512) + 0.18 &&
+                                 round_fill(blocks(128, 128), 768) >= round_fill(b21, 512) + 0.15 &&
                                  filled(128, 128) >= 0.6;
-    if (planes == 1 && !last_round_idle && (b21 >= 512 || (KT >= 16 && b21 >= 160 && !(b21 > 256 && b21 < 320))) &&
+    if (planes == 1 && !last_round_idle && (b21 >= 512 || (KT >= 16 && b21 >= 132 && !(b21 > 256 && b21 <= 384))) &&
         (KT >= (out_shift == 1 ? 8 : 4) || blocks(128, 128) < 512) &&      // (2-byte outputs leave 128 x 128 without staging in LDS:
         filled(256, 128) >= 0.75)                                          //  48 x [2048 x 2048] x 1024 -> fp16 117 against 131 us)
         return {BGEMM_KERNEL_MFMA_256x128, 256, 128};

@@ -123,6 +123,11 @@ def test_dispatch_of_the_benchmark_configurations():
     assert kid(MODE_XOR, 1, 2048, 4096, 1024, 1, A) == B.KERNEL_MFMA_32x256
     assert kid(MODE_XOR, 1, 2000, 4000, 1024, 1, A) == B.KERNEL_MFMA_128x128
     assert kid(MODE_XOR, 1, 2048, 4096, 2048, 1, A) == B.KERNEL_MFMA_128x128
+    # 256 x 128: from 132 blocks on 16 K-tiles or more, but not between one block a unit and one and a half
+    assert kid(MODE_XOR, 1, 4352, 1024, 8192, 1, A) == B.KERNEL_MFMA_256x128     # 136 blocks
+    assert kid(MODE_XOR, 1, 2560, 1536, 8192, 1, A) == B.KERNEL_MFMA_128x128     # 120: every 128 x 128 block has a unit to itself
+    assert kid(MODE_XOR, 1, 6144, 2048, 16384, 1, A) == B.KERNEL_MFMA_128x128    # 384
+    assert kid(MODE_XOR, 1, 6656, 2048, 16384, 1, A) == B.KERNEL_MFMA_256x128    # 416
     assert kid(MODE_ATTN_X, 24, 64, 512, 512, 1, A) == B.KERNEL_MFMA_64x64
     assert kid(MODE_BWTA, 1, 11008, 1, 4096, 8, A) == B.KERNEL_SKINNY_POPC
     assert kid(MODE_BWTA, 1, 11008, 16, 4096, 8, A) == B.KERNEL_SKINNY_SPLITK
