@@ -223,7 +223,7 @@ __global__ __launch_bounds__(256, 2) void gemm_skinny_stream_kernel(const GemmAr
 // the blocks and the weight traffic (64 to 128 rows: 8 to 15 % faster; up to 32 rows the half blocks win by
 // 10 to 20 %, twice the blocks with half the matrix-core chain each).
 template <typename Eng, int KW, bool FUSEX = false, bool PL2 = false>
-__global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 2) void gemm_skinny_splitk_kernel(const GemmArgs a)
+__global__ __launch_bounds__(KW * 64, FUSEX && KW <= 8 ? 4 : 2) void gemm_skinny_splitk_kernel(const GemmArgs a)
 {
     static_assert(!(FUSEX && PL2), "in-kernel activation packing is built for up to four rows");
     constexpr int NT = KW * 64, NP = PL2 ? 2 : 1;
@@ -290,21 +290,31 @@ __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 2) void gemm_skinny_splitk_ker
 
     // the wave's K range is short (K / KW) and requested MAXT K-tiles at a time: the kernel lives
     // on memory-level parallelism
-    for (int kb = kt0; kb < kt1 || kb == kt0; kb += MAXT) {
-        uint4 xq[MAXT], xq2[PL2 ? MAXT : 1], wq[MAXT], xraw[FUSEX ? MAXT : 1][FUSEX ? 2 : 1];
-        if (kb < kt1) {
-            if (FUSEX && xfast) {
+    // (FUSEX: the source rows of the first four activation rows are requested one round of K-tiles ahead, the first
+    // round before the loop, so that a wave with several rounds does not pay the trip to memory once per round:
+    // W[4096,11008] x 4 ternary rows 9.5 -> 8.6 us, and 7.2 with sixteen ways a block, see launch_splitk_fusex)
+    typedef uint4 XRaw[FUSEX ? MAXT : 1][FUSEX ? 2 : 1];
+    XRaw xraw;
+    auto x_request = [&](XRaw& to, const int kb) {
 #pragma unroll
-                for (int q = 0; q < MAXT; q++)
+        for (int q = 0; q < MAXT; q++)
 #pragma unroll
-                    for (int jr = 0; jr < 2; jr++) {
-                        const int n = xr + 2 * jr;
-                        const int64_t k0 = (int64_t)(kb + q) * TILE_KBITS + 8 * xc;
-                        xraw[q][jr] = (kb + q < kt1 && n < (int)a.N && k0 < a.K)
-                                          ? *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(a.xsrc) + (int64_t)n * a.xld + k0)
-                                          : make_uint4(0u, 0u, 0u, 0u);
-                    }
+            for (int jr = 0; jr < 2; jr++) {
+                const int n = xr + 2 * jr;
+                const int64_t k0 = (int64_t)(kb + q) * TILE_KBITS + 8 * xc;
+                to[FUSEX ? q : 0][FUSEX ? jr : 0] = (kb + q < kt1 && n < (int)a.N && k0 < a.K)
+                                  ? *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(a.xsrc) + (int64_t)n * a.xld + k0)
+                                  : make_uint4(0u, 0u, 0u, 0u);
             }
+    };
+    if (FUSEX && xfast) x_request(xraw, kt0);
+    // the operand rows that carry activation rows: every other lane's share of a tile built in LDS is zero and is
+    // not read (nor cleared) there
+    const bool x_real_row = (lane & 31) < (int)a.N || (two && (lane & 31) >= 16 && (lane & 31) - 16 < (int)a.N);
+    for (int kb = kt0; kb < kt1 || kb == kt0; kb += MAXT) {
+        uint4 xq[MAXT], xq2[PL2 ? MAXT : 1], wq[MAXT];
+        XRaw xahead;
+        if (kb < kt1) {
 #pragma unroll
             for (int q = 0; q < MAXT; q++) {
                 if (kb + q >= kt1) break;                       // wave-uniform: no load for a K-tile past the range
@@ -313,12 +323,12 @@ __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 2) void gemm_skinny_splitk_ker
                 if (PL2) xq2[q] = xp2[off];
                 wq[q] = load_stream(wp + off);
             }
+            if (FUSEX && xfast && kb + MAXT < kt1) x_request(xahead, kb + MAXT);
             if (FUSEX) {
 #pragma unroll
                 for (int q = 0; q < MAXT; q++) {
                     if (kb + q >= kt1) break;
                     unsigned char* const t = sX[wave][q];
-                    for (int i = lane; i < 256; i += 64) reinterpret_cast<uint32_t*>(t)[i] = 0u;
                     if (xfast) {
 #pragma unroll
                         for (int jr = 0; jr < 2; jr++) {
@@ -345,9 +355,16 @@ __global__ __launch_bounds__(KW * 64, FUSEX ? 4 : 2) void gemm_skinny_splitk_ker
                 __builtin_amdgcn_wave_barrier();
                 __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-                for (int q = 0; q < MAXT; q++) xq[q] = reinterpret_cast<const uint4*>(sX[wave][min(q, kt1 - 1 - kb)])[lane];
+                for (int q = 0; q < MAXT; q++)
+                    xq[q] = x_real_row ? reinterpret_cast<const uint4*>(sX[wave][min(q, kt1 - 1 - kb)])[lane] : make_uint4(0u, 0u, 0u, 0u);
                 __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");      // the next chunk overwrites the area
                 __builtin_amdgcn_wave_barrier();
+                if (xfast && kb + MAXT < kt1) {
+#pragma unroll
+                    for (int q = 0; q < MAXT; q++)
+#pragma unroll
+                        for (int jr = 0; jr < 2; jr++) xraw[FUSEX ? q : 0][FUSEX ? jr : 0] = xahead[FUSEX ? q : 0][FUSEX ? jr : 0];
+                }
             }
         }
         if (kb == kt0) {
@@ -480,31 +497,24 @@ __global__ __launch_bounds__(KW * 64) void gemm_skinny_popc_kernel(const GemmArg
 #pragma unroll
     for (int j = 0; j < NVEC; j++) d[j] = pb[j] = 0;
 
-    for (int kb = kt0; kb < kt1 || kb == kt0; kb += MAXT) {
-        uint4 wq[MAXT], xq[MAXT][NVEC];
-        if (kb < kt1) {
-            uint32_t xbyte[NVEC];
-            if (FUSEX) {                                        // the rows first: loads return in order
-                const int64_t k0 = (int64_t)kb * TILE_KBITS + 8 * lane;
-                const bool mine = kb + h < kt1;                 // the second K-tile of the pair may be another wave's
+    // FUSEX, aligned fp16 rows without a zero point: the 16 bytes a lane turns into bits are requested one pair of
+    // K-tiles ahead (the first pair before the loop, ahead of the weight loads: loads return in order), so that a wave
+    // with several pairs pays the trip to memory once
+    uint4 xraw[FUSEX ? ROWS : 1];
+    auto x_request = [&](uint4 (&to)[FUSEX ? ROWS : 1], const int kb) {
+        const int64_t k0 = (int64_t)kb * TILE_KBITS + 8 * lane;
+        const bool mine = kb + h < kt1;                         // the second K-tile of the pair may be another wave's
 #pragma unroll
-                for (int rr = 0; rr < ROWS; rr++) {
-                    const int n = min(rr, (int)a.N - 1);
-                    uint32_t sg, nz;
-                    if (xfast) {                                // aligned fp16 rows, no zero point: bits straight from one 16-byte load
-                        const uint4 v = (mine && k0 < a.K) ? *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(a.xsrc) + (int64_t)n * a.xld + k0)
-                                                           : make_uint4(0u, 0u, 0u, 0u);
-                        bits8(v, sg, nz);
-                    } else {
-                        uint16_t hb[8];
-                        load8_as_half(reinterpret_cast<const char*>(a.xsrc) + (int64_t)n * a.xld * (a.xsrc_f32 ? 4 : 2), a.xsrc_f32 != 0,
-                                      mine ? k0 : a.K, a.K, a.xzp != nullptr, xzf, hb);
-                        bits8(hb, sg, nz);
-                    }
-                    if (TWO) { xbyte[2 * rr] = nz; xbyte[TWO ? 2 * rr + 1 : 0] = sg & nz; }
-                    else xbyte[rr] = sg;
-                }
-            }
+        for (int rr = 0; rr < ROWS; rr++) {
+            const int n = min(rr, (int)a.N - 1);
+            to[FUSEX ? rr : 0] = (mine && k0 < a.K) ? *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(a.xsrc) + (int64_t)n * a.xld + k0)
+                                                    : make_uint4(0u, 0u, 0u, 0u);
+        }
+    };
+    if (FUSEX && xfast) x_request(xraw, kt0);
+    for (int kb = kt0; kb < kt1 || kb == kt0; kb += MAXT) {
+        uint4 wq[MAXT], xq[MAXT][NVEC], xahead[FUSEX ? ROWS : 1];
+        if (kb < kt1) {
 #pragma unroll
             for (int q = 0; q < MAXT; q++) {
                 if (kb + q >= kt1) break;                       // wave-uniform: no load for a K-tile past the range
@@ -515,7 +525,27 @@ __global__ __launch_bounds__(KW * 64) void gemm_skinny_popc_kernel(const GemmArg
                 }
                 wq[q] = load_stream(wp + off);
             }
+            if (FUSEX && xfast && kb + MAXT < kt1) x_request(xahead, kb + MAXT);
+            uint32_t xbyte[NVEC];
             if (FUSEX) {
+                const int64_t k0 = (int64_t)kb * TILE_KBITS + 8 * lane;
+                const bool mine = kb + h < kt1;
+#pragma unroll
+                for (int rr = 0; rr < ROWS; rr++) {
+                    const int n = min(rr, (int)a.N - 1);
+                    uint32_t sg, nz;
+                    if (xfast) {
+                        bits8(xraw[FUSEX ? rr : 0], sg, nz);
+                        if (kb + MAXT < kt1) xraw[FUSEX ? rr : 0] = xahead[FUSEX ? rr : 0];
+                    } else {
+                        uint16_t hb[8];
+                        load8_as_half(reinterpret_cast<const char*>(a.xsrc) + (int64_t)n * a.xld * (a.xsrc_f32 ? 4 : 2), a.xsrc_f32 != 0,
+                                      mine ? k0 : a.K, a.K, a.xzp != nullptr, xzf, hb);
+                        bits8(hb, sg, nz);
+                    }
+                    if (TWO) { xbyte[2 * rr] = nz; xbyte[TWO ? 2 * rr + 1 : 0] = sg & nz; }
+                    else xbyte[rr] = sg;
+                }
 #pragma unroll
                 for (int j = 0; j < NVEC; j++) sXb[wave][j][lane ^ 3] = (unsigned char)xbyte[j];
                 __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -802,6 +832,12 @@ static int launch_splitk_fusex(const GemmArgs& a, hipStream_t st)
     int kw = 1;
     while (kw < 8 && (kw < a.splitK || blocks * kw < 4096) && kw * 2 <= a.KT) kw *= 2;
     const dim3 g((unsigned)blocks);
+    // few row tiles against a long K: sixteen ways, as for packed activations (launch_splitk), and more to gain here,
+    // where every K-tile of a wave's range costs it the packing as well
+    if (kw == 8 && blocks * 8 < 2048 && a.KT >= 32) {
+        hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 16, true>), g, dim3(1024), 0, st, a);
+        return check_launch("gemm_skinny");
+    }
     if (kw == 1) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 1, true>), g, dim3(64), 0, st, a);
     else if (kw == 2) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 2, true>), g, dim3(128), 0, st, a);
     else if (kw == 4) hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 4, true>), g, dim3(256), 0, st, a);

@@ -562,7 +562,9 @@ def test_scaled_epilogue_empty_k_and_errors():
 
 # ------------------------------------------------------------------ decode step on unpacked activations
 @pytest.mark.parametrize("variant", [VARIANT_AUTO, VARIANT_MFMA, VARIANT_MFMA_F4])
-@pytest.mark.parametrize("M,N,K", [(11008, 1, 4096), (4100, 4, 1000), (300, 2, 40), (64, 4, 2500), (1000, 3, 256), (33, 1, 8), (500, 16, 512)])
+@pytest.mark.parametrize("M,N,K", [(11008, 1, 4096), (4100, 4, 1000), (300, 2, 40), (64, 4, 2500), (1000, 3, 256), (33, 1, 8), (500, 16, 512),
+                                   # several rounds of K-tiles a wave (rows requested a round ahead); sixteen ways a block
+                                   (8200, 4, 6400), (4096, 4, 11008), (1000, 3, 8200), (1000, 2, 11008)])
 def test_decode_step_packs_its_own_activations(variant, M, N, K):
     """One launch on fp16 / fp32 activations = pack launch + packed GEMM, bit for bit: every mode, ternary planes,
     zero point, strided rows, scaled output."""
