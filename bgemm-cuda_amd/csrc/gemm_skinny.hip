@@ -796,14 +796,15 @@ __global__ __launch_bounds__(KW * 64, 2) void gemm_skinny_splitk_quad_kernel(con
 // up to 1024 pieces from 16 K-tiles on, 2048 from 24, 4096 from 48 (2048^2 x 8192, 4096 pieces at 32 K-tiles: 18.4 us here,
 // 16.7 on the general kernel's pipelined 128 x 128 tile; 8192 x 768 x 16384, 6144 pieces: 49 us here, 42 on its
 // 256 x 128 tile even at three quarters of a block per unit).  Two planes (twice the
-// matrix-core work per piece): up to 2048 pieces from 24 K-tiles on, 3072 from 32, 4096 from 40.  Beyond that
+// matrix-core work per piece): up to 2048 pieces from 24 K-tiles on, 3072 from 32, 4096 from 40, from 256 blocks (192
+// from 40 K-tiles on: W[4096,11008] x 96 ternary rows 8.2 us against 9.3 on one piece a block).  Beyond that
 // the general kernel's 128- and 256-row tiles re-read less.
 static bool skinny_quad_shape(int planes, int64_t batch, int64_t MT, int64_t NT, int64_t KT)
 {
     if (MT < 2 || NT < 2) return false;
     const int64_t pieces = batch * MT * NT;
     if (planes == 2)
-        return batch * cdiv(MT, 2) * NT >= 256 && pieces <= (KT >= 40 ? 4096 : KT >= 32 ? 3072 : KT >= 24 ? 2048 : 0);
+        return batch * cdiv(MT, 2) * NT >= (KT >= 40 ? 192 : 256) && pieces <= (KT >= 40 ? 4096 : KT >= 32 ? 3072 : KT >= 24 ? 2048 : 0);
     if (batch * cdiv(MT, 2) * cdiv(NT, 2) < 256) return false;
     return pieces <= (KT >= 48 ? 4096 : KT >= 24 ? 2048 : KT >= 16 ? 1024 : 0);
 }
@@ -853,16 +854,14 @@ static int launch_splitk_quad(const GemmArgs& a, hipStream_t st)
     const int64_t gx = cdiv(a.MT, 2), gy = TWO ? a.NT : cdiv(a.NT, 2);
     if (gy > 65535 || a.batch > 65535)
         return fail(BGEMM_EINVAL, "gemm_skinny: grid of %lld x %lld x %lld blocks", (long long)gx, (long long)gy, (long long)a.batch);
-    // K ways per block: the kernel's registers allow two waves a SIMD, 2048 on the chip at once, and the grid
-    // should come out as whole rounds of that (1536 blocks: four ways are three full rounds, two ways one and
-    // a half).  Fewest ways among the best fits.
+    // K ways per block.  The kernel's registers allow two waves a SIMD, eight a CU: eight ways are one block a CU, which is
+    // what up to 256 blocks want; beyond that every block more on a CU is a round more, and four ways (two blocks a CU,
+    // each wave on twice the K range, half as many meetings in LDS and store loops per unit of work) are 15 to 25 %
+    // faster (8192 x 160 ternary rows x 8192, 640 blocks: 15.9 against 19.0 us; 11008 x 192 x 8192, 1032 blocks: 24.5 against
+    // 31.3; 8192 x 384 x 16384 sign rows, 768 blocks: 26.9 against 33.5).  Two ways where four blocks a CU are one full round
+    // (769 to 1024 blocks: 8192 x 512 x 16384 31.9 against 33.8 on four ways).
     const int64_t blocks = gx * gy * a.batch;
-    int kw = 8;
-    int64_t best_w = blocks * 8, best_r = cdiv(best_w, 2048);
-    for (int c = 4; c >= 2; c /= 2) {
-        const int64_t w = blocks * c, r = cdiv(w, 2048);
-        if (w * best_r >= best_w * r) { kw = c; best_w = w; best_r = r; }      // w / r: waves per round
-    }
+    int kw = blocks <= 256 ? 8 : blocks > 768 && blocks <= 1024 ? 2 : 4;
     while (kw > 1 && kw > a.KT) kw /= 2;
     const dim3 g((unsigned)gx, (unsigned)gy, (unsigned)a.batch);
     if (kw == 1) hipLaunchKernelGGL((gemm_skinny_splitk_quad_kernel<Eng, 1, TWO>), g, dim3(64), 0, st, a);

@@ -316,7 +316,9 @@ def test_stream_kernel_up_to_four_rows_one_store_a_row(engine):
                 assert (bits_of(got) == bits_of(f16_of(want))).all(), (M, N, mode)
 
 
-@pytest.mark.parametrize("N,want_kernel", [(256, B.KERNEL_SKINNY_QUAD), (2048, B.KERNEL_MFMA_256x128)])
+@pytest.mark.parametrize("N,want_kernel", [(256, B.KERNEL_SKINNY_QUAD), (2048, B.KERNEL_MFMA_256x128),
+                                           # 640 and 1024 blocks of four pieces: four and two K ranges a block, several blocks a CU
+                                           (320, B.KERNEL_SKINNY_QUAD), (512, B.KERNEL_SKINNY_QUAD)])
 def test_config5_sweep_long_k(N, want_kernel):
     """The K = 16384 points of configuration 5's sweep, split-K 1 / 2 / 4: sampled rows and columns against the
     closed form, identities over the whole output, and agreement between the split-K values and the designs."""
