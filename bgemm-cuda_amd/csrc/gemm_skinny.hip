@@ -802,6 +802,7 @@ __global__ __launch_bounds__(KW * 64, 2) void gemm_skinny_splitk_quad_kernel(con
 static bool skinny_quad_shape(int planes, int64_t batch, int64_t MT, int64_t NT, int64_t KT)
 {
     if (MT < 2 || NT < 2) return false;
+    if (batch > 1 && KT < 24) return false;      // (a batch of small products: operands that were just written, see gemm_skinny_shape)
     const int64_t pieces = batch * MT * NT;
     if (planes == 2)
         return batch * cdiv(MT, 2) * NT >= (KT >= 40 ? 192 : 256) && pieces <= (KT >= 40 ? 4096 : KT >= 32 ? 3072 : KT >= 24 ? 2048 : 0);
@@ -822,7 +823,9 @@ bool gemm_skinny_shape(int planes, int64_t batch, int64_t M, int64_t N, int64_t 
     if (N <= (planes == 2 ? 16 : 32)) return true;
     const int64_t pieces = batch * row_tiles(M) * row_tiles(N), KT = k_tiles(K);
     if (skinny_quad_shape(planes, batch, row_tiles(M), row_tiles(N), KT)) return true;
-    if (KT >= 8) return pieces <= 1024;
+    // (a batch of products is attention-shaped work on operands that were just written and still sit in the caches:
+    // there the general kernel keeps up from 512 pieces on; 8 x [128 x 1024] x 2048, 1024 pieces: 4.3 us there, 5.1 here)
+    if (KT >= 8) return pieces <= (batch > 1 ? 512 : 1024);
     return KT >= 4 && pieces <= 512;
 }
 

@@ -16,6 +16,7 @@ pytestmark = pytest.mark.gpu
 import lowbit_kernel as lk
 from _lib import (MODE_AND, MODE_XOR, MODE_ATTN, MODE_BWTA, MODE_ATTN_X, VARIANT_AUTO, VARIANT_VALU, VARIANT_MFMA,
                   VARIANT_MFMA_F4)
+import _lib
 
 DEV = "cuda:0"
 VARIANTS = [VARIANT_VALU, VARIANT_MFMA, VARIANT_MFMA_F4]
@@ -278,8 +279,8 @@ def test_decode_batches_of_ternary_rows(M, N, K):
     assert torch.equal(got3[1], lk.bgemm_packed_forward(lk.PackedBits(wp.data.flip(1).contiguous(), None, 1, M, K), xt, MODE_BWTA, torch.int32)[0])
 
 
-@pytest.mark.parametrize("batch,M,N,K", [(1, 4040, 270, 6200), (4, 1000, 250, 4100), (1, 8192, 256, 8192),
-                                         (1, 4096, 1024, 8192), (1, 4096, 512, 8192)])      # the last two: two K ways, one plane / two planes
+@pytest.mark.parametrize("batch,M,N,K", [(1, 4040, 270, 6200), (4, 1000, 250, 6200), (1, 8192, 256, 8192),
+                                         (1, 4096, 768, 12288), (1, 4096, 512, 8192)])      # the last two: four / two K ways, several blocks a CU
 def test_split_k_in_block_four_pieces_a_block(oracle, batch, M, N, K):
     """Outputs of one to two thousand 32 x 32 pieces over a long K: a block takes two weight row tiles and two
     activation tile rows (odd tile counts, ragged M, N and K, batches); every one-plane mode, both engines,
@@ -289,6 +290,7 @@ def test_split_k_in_block_four_pieces_a_block(oracle, batch, M, N, K):
     x = rand_f16(rng, batch * N, K).reshape(batch, N, K)
     wp, xp = lk.pack_sign(to_dev(w)), lk.pack_sign(to_dev(x))
     xt = lk.pack_ternary(to_dev(x))
+    assert lk.packed_kernel_id(wp, xp, MODE_XOR, 8) == _lib.KERNEL_SKINNY_QUAD and lk.packed_kernel_id(wp, xt, MODE_BWTA, 8) == _lib.KERNEL_SKINNY_QUAD
     for mode in (MODE_XOR, MODE_AND, MODE_ATTN, MODE_ATTN_X, MODE_BWTA):     # ternary: the two planes of a tile row are the block's two operands
         want = np.stack([dense_ref(mode, w[b], x[b]) for b in range(batch)])
         xo = xt if mode == MODE_BWTA else xp
