@@ -695,6 +695,10 @@ static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int pla
     // (one K-tile only: from two on, 128 x 128 is 15 % ahead: 48 x [1024 x 512] x 512 -> fp16 13.3 against 15.6 us)
     // (from two such tiles a row on: 192 x [2048 x 256] x 256 -> fp16, one tile a row, 39.3 us against 35.5 on 128 x 128)
     if (KT < 2 && out_shift == 1 && M >= 512 && blocks(32, 256) >= 512) return {BGEMM_KERNEL_MFMA_32x256, 32, 256};
+    // one K-tile into more int32 output than the 256 MiB memory-side cache holds: the same tile again (48 x [1024 x 2048] x
+    // 64, 403 MB: 70.4 us against 84.5 on 128 x 128; 192 x [512 x 1024] x 64: 71.9 against 76.3; at 201 MB no difference)
+    if (KT < 2 && out_shift == 2 && M >= 512 && batch * N * M > (64 << 20) && blocks(32, 256) >= 512)
+        return {BGEMM_KERNEL_MFMA_32x256, 32, 256};
     // a short K with int32 rows of a power of two in bytes (4 to 64 KiB): the few large blocks of such a launch all
     // run in step, and the rows they store at one moment lie a multiple of 1 MiB apart, on few memory channels;
     // four times as many 32-row blocks drift apart (2048 x 4096 x 1024: 9.5 us against 12.6 on 128 x 128, 4096 x 2048 x

@@ -119,6 +119,7 @@ def test_dispatch_of_the_benchmark_configurations():
     # a short K with a 2-byte output takes the tile with 512-byte rows
     assert B.lib().bgemm_packed_kernel_id(MODE_XOR, B.OUT_F16, 192, 512, 512, 64, 1, A) == B.KERNEL_MFMA_32x256
     assert kid(MODE_XOR, 192, 512, 512, 64, 1, A) == B.KERNEL_MFMA_128x128
+    assert kid(MODE_XOR, 48, 2048, 1024, 64, 1, A) == B.KERNEL_MFMA_32x256      # 403 MB of int32 from one K-tile
     # int32 rows of a power of two in bytes on a short K: many 32-row blocks instead of few large ones in step
     assert kid(MODE_XOR, 1, 2048, 4096, 1024, 1, A) == B.KERNEL_MFMA_32x256
     assert kid(MODE_XOR, 1, 2000, 4000, 1024, 1, A) == B.KERNEL_MFMA_128x128
