@@ -718,7 +718,8 @@ static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int pla
     // 2560 x 1536 x 8192, 120 blocks, 21.0 against 16.5 on 240 blocks of 128 x 128), except from a few blocks more than one
     // a unit (11008 x 768 x 4096: 258, 11008 x 640 x 8192 likewise) to one and a half (6144 x 2048 x 16384: 384 blocks, 72.6
     // against 71.3), which would leave the launch waiting for the units that run two blocks each while three blocks of
-    // the next tile down fit every unit at once: those go to the next tile down
+    // the next tile down fit every unit at once: those go to the next tile down (up to 352 blocks for a 2-byte output, which
+    // 128 x 128 stores from its plain loop: 6144 x 2048 x 16384 -> fp16, 384 blocks, 72.6 us against 76.9)
     const int64_t b21 = blocks(256, 128);
     // a last round that leaves most of the GPU idle (576 blocks on 512 places: 6144 x 3072 x 4096 42.5 us against 34.9 on
     // 128 x 128, whose 1152 blocks fill one and a half rounds of 768 places) goes to the smaller tile
@@ -726,7 +727,7 @@ static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int pla
     const bool last_round_idle = KT >= 8 && KT <= 16 && b21 > 256 &&      // (on a longer K the larger tile's cheaper loop makes up for it)
                                  round_fill(blocks(128, 128), 768) >= round_fill(b21, 512) + 0.15 &&
                                  filled(128, 128) >= 0.6;
-    if (planes == 1 && !last_round_idle && (b21 >= 512 || (KT >= 16 && b21 >= 132 && !(b21 > 256 && b21 <= 384))) &&
+    if (planes == 1 && !last_round_idle && (b21 >= 512 || (KT >= 16 && b21 >= 132 && !(b21 > 256 && b21 <= (out_shift == 1 ? 352 : 384)))) &&
         (KT >= (out_shift == 1 ? 8 : 4) || blocks(128, 128) < 512) &&      // (2-byte outputs leave 128 x 128 without staging in LDS:
         filled(256, 128) >= 0.75)                                          //  48 x [2048 x 2048] x 1024 -> fp16 117 against 131 us)
         return {BGEMM_KERNEL_MFMA_256x128, 256, 128};

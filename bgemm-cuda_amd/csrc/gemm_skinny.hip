@@ -793,7 +793,7 @@ __global__ __launch_bounds__(KW * 64, 2) void gemm_skinny_splitk_quad_kernel(con
 // Shapes the four-pieces kernel takes: at least two tile rows on either side, enough blocks to give every
 // compute unit one, and a K long enough for the shared expansions to outweigh the larger meeting area (timed
 // against both neighbours, weights from HBM and from a warm cache, pieces = 32 x 32 outputs).  One bit plane:
-// up to 1024 pieces from 16 K-tiles on, 2048 from 24, 4096 from 48 (2048^2 x 8192, 4096 pieces at 32 K-tiles: 18.4 us here,
+// up to 1024 pieces from 16 K-tiles on, 2048 from 24, 3072 from 40 (6144 x 512 x 11008: 19.7 us against 24.6 on 128 x 128), 4096 from 48 (2048^2 x 8192, 4096 pieces at 32 K-tiles: 18.4 us here,
 // 16.7 on the general kernel's pipelined 128 x 128 tile; 8192 x 768 x 16384, 6144 pieces: 49 us here, 42 on its
 // 256 x 128 tile even at three quarters of a block per unit).  Two planes (twice the
 // matrix-core work per piece): up to 2048 pieces from 24 K-tiles on, 3072 from 32, 4096 from 40, from 256 blocks (192
@@ -807,7 +807,7 @@ static bool skinny_quad_shape(int planes, int64_t batch, int64_t MT, int64_t NT,
     if (planes == 2)
         return batch * cdiv(MT, 2) * NT >= (KT >= 40 ? 192 : 256) && pieces <= (KT >= 40 ? 4096 : KT >= 32 ? 3072 : KT >= 24 ? 2048 : 0);
     if (batch * cdiv(MT, 2) * cdiv(NT, 2) < 256) return false;
-    return pieces <= (KT >= 48 ? 4096 : KT >= 24 ? 2048 : KT >= 16 ? 1024 : 0);
+    return pieces <= (KT >= 48 ? 4096 : KT >= 40 ? 3072 : KT >= 24 ? 2048 : KT >= 16 ? 1024 : 0);
 }
 
 // Shapes the skinny kernels take: one group of activation rows always (32 rows, or 16 rows of two bit planes).
