@@ -718,8 +718,7 @@ static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int pla
     // 2560 x 1536 x 8192, 120 blocks, 21.0 against 16.5 on 240 blocks of 128 x 128), except from a few blocks more than one
     // a unit (11008 x 768 x 4096: 258, 11008 x 640 x 8192 likewise) to one and a half (6144 x 2048 x 16384: 384 blocks, 72.6
     // against 71.3), which would leave the launch waiting for the units that run two blocks each while three blocks of
-    // the next tile down fit every unit at once: those go to the next tile down (up to 352 blocks for a 2-byte output, which
-    // 128 x 128 stores from its plain loop: 6144 x 2048 x 16384 -> fp16, 384 blocks, 72.6 us against 76.9)
+    // the next tile down fit every unit at once: those go to the next tile down
     const int64_t b21 = blocks(256, 128);
     // a last round that leaves most of the GPU idle (576 blocks on 512 places: 6144 x 3072 x 4096 42.5 us against 34.9 on
     // 128 x 128, whose 1152 blocks fill one and a half rounds of 768 places) goes to the smaller tile
@@ -727,7 +726,7 @@ static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int pla
     const bool last_round_idle = KT >= 8 && KT <= 16 && b21 > 256 &&      // (on a longer K the larger tile's cheaper loop makes up for it)
                                  round_fill(blocks(128, 128), 768) >= round_fill(b21, 512) + 0.15 &&
                                  filled(128, 128) >= 0.6;
-    if (planes == 1 && !last_round_idle && (b21 >= 512 || (KT >= 16 && b21 >= 132 && !(b21 > 256 && b21 <= (out_shift == 1 ? 352 : 384)))) &&
+    if (planes == 1 && !last_round_idle && (b21 >= 512 || (KT >= 16 && b21 >= 132 && !(b21 > 256 && b21 <= 384))) &&
         (KT >= (out_shift == 1 ? 8 : 4) || blocks(128, 128) < 512) &&      // (2-byte outputs leave 128 x 128 without staging in LDS:
         filled(256, 128) >= 0.75)                                          //  48 x [2048 x 2048] x 1024 -> fp16 117 against 131 us)
         return {BGEMM_KERNEL_MFMA_256x128, 256, 128};
@@ -759,12 +758,13 @@ static int launch_cfg(const GemmArgs& a, hipStream_t st)
     } else {
         // The hand-pipelined loop: always on the tiles of eight and sixteen MFMA tiles a wave; on 128 x 128 from eight
         // K-tiles on (11008 x 640 x 8192: 31.6 against 34.9 us, 8192^2 x 2048: 90.5 against 98.6; at four K-tiles the plain
-        // loop is 4 % ahead), unless the output is fp16 pairs, which only the plain loop stores straight from registers.
+        // loop is 4 % ahead); where the output is fp16 pairs, which only the plain loop stores straight from registers, from
+        // sixteen K-tiles on (5120 x 2048 x 8192 -> fp16: 33.5 against 37.3 us, 6144 x 3072 x 4096: 31.2 against 33.8; level at eight).
         constexpr bool MUST_PIPE = WN * WM >= 8, CAN_PIPE = WN * WM >= 4 && WGM == 2 && WN % 2 == 0;
         const bool pairs = a.out_kind == BGEMM_OUT_F16 && a.vec_store == 8 && WM % 2 == 0;
         const dim3 g((unsigned)grid), blk(WGN * WGM * 64);
         if constexpr (CAN_PIPE) {
-            if (MUST_PIPE || (a.KT >= 8 && !pairs)) {
+            if (MUST_PIPE || (a.KT >= 8 && (!pairs || a.KT >= 16))) {
                 if (a.cntW && a.cntX)
                     hipLaunchKernelGGL((gemm_mfma_kernel<Eng, WGN, WGM, WN, WM, 1, true, true>), g, blk, 0, st, a, tiles_n, tiles_m);
                 else

@@ -124,13 +124,14 @@ def test_each_tile_every_output_kind(oracle, tile, engine, M):
     check_all_kinds(oracle, wp, xp, dense(MODE_XOR, w, x), M, N, variant, rng)
 
 
+@pytest.mark.parametrize("KT", [9, 17])
 @pytest.mark.parametrize("M", [520, 517])
 @pytest.mark.parametrize("engine", list(ENGINES))
-def test_128x128_takes_the_pipelined_loop_from_eight_k_tiles(oracle, engine, M):
-    """From eight K-tiles on the 128 x 128 tile runs the hand-pipelined loop (except for fp16 pairs, which stay on the
-    plain one): nine K-tiles, the last ragged, every output kind, ragged M and N; and with the operands' row
-    popcounts brought along."""
-    N, K = 515, 9 * 256 - 5
+def test_128x128_takes_the_pipelined_loop_from_eight_k_tiles(oracle, engine, M, KT):
+    """From eight K-tiles on the 128 x 128 tile runs the hand-pipelined loop (fp16 pairs, which the plain loop stores
+    straight from its registers, from sixteen): nine and seventeen K-tiles, the last ragged, every output kind, ragged
+    M and N; and with the operands' row popcounts brought along."""
+    N, K = 515, KT * 256 - 5
     rng = np.random.default_rng(M * 17 + 5)
     w, x = pm1(rng, M, K), pm1(rng, N, K)
     wp, xp = lk.pack_sign(to_dev(w)), lk.pack_sign(to_dev(x))
