@@ -806,7 +806,7 @@ static bool skinny_quad_shape(int planes, int64_t batch, int64_t MT, int64_t NT,
     const int64_t pieces = batch * MT * NT;
     if (planes == 2)
         return batch * cdiv(MT, 2) * NT >= (KT >= 40 ? 192 : 256) && pieces <= (KT >= 40 ? 4096 : KT >= 32 ? 3072 : KT >= 24 ? 2048 : 0);
-    if (batch * cdiv(MT, 2) * cdiv(NT, 2) < 256) return false;
+    if (batch * cdiv(MT, 2) * cdiv(NT, 2) < (KT >= 40 ? 192 : 256)) return false;      // (7168 x 128 x 11008, 224 blocks: 9.9 us against 11.8 on one piece a block)
     return pieces <= (KT >= 48 ? 4096 : KT >= 40 ? 3072 : KT >= 24 ? 2048 : KT >= 16 ? 1024 : 0);
 }
 
