@@ -132,8 +132,9 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
         }
         // Raw K-tiles in flight: two buffers (a K-tile requested one tile ahead of its first use), or three where the
         // registers allow (two tiles ahead: the 256 x 128 tile's 32 MFMAs a K-tile are half a microsecond, less
-        // than a trip to a far L2 takes under load)
-        constexpr int NBUF = NM == 8 && STEPS == 4 ? 3 : 2;       // (the int8 engine's eight steps a tile leave no registers for it)
+        // than a trip to a far L2 takes under load; on the 128 x 128 tile likewise: 3072 x 1024 x 8192 17.0 -> 15.3 us,
+        // 11008 x 640 x 8192 28.3 -> 25.8)
+        constexpr int NBUF = (NM == 8 || NM == 4) && STEPS == 4 ? 3 : 2;       // (the int8 engine's eight steps a tile leave no registers for it)
         unsigned rawA[NF][4], rawB[NF][4], rawC[NBUF == 3 ? NF : 1][4], buf[2][NF][4];
         int pop[NF];
 #pragma unroll
@@ -675,11 +676,11 @@ struct MfmaCfg { int id, bn, bm; };
 
 // Tile choice, from timings of every tile over a sweep of shapes (bench.py --only thresholds prints them): the
 // 256 x 256 tile (one block per CU, hand-pipelined loop, the fastest main loop) needs at least two rounds of
-// blocks and a long K (from 32 K-tiles) to pay for its epilogue, during which its CU computes nothing;
+// blocks and a long K (from 128 K-tiles) to pay for its epilogue, during which its CU computes nothing;
 // 256 x 128 (two resident blocks per CU that run half a tile apart, so one block's stores overlap the other's
-// main loop) from one block per CU upwards on 16 K-tiles or more (4096 x 2048 x 4096: 17.2 against 18.5 us on
-// 128 x 128), from two below that, except on very short K (under 4 K-tiles), where 128 x 128 keeps more waves
-// in flight for what is then all prologue and epilogue; below that the smaller tiles, down to 32 x 128, are
+// main loop) from half a block per CU upwards on a long K (see below), from two below that, except on very
+// short K (under 4 K-tiles), where 128 x 128 keeps more waves in flight for what is then all prologue and
+// epilogue; below that the smaller tiles, down to 32 x 128, are
 // chosen so that every CU gets a block.  Narrow outputs (M <= 64) take 64-wide tiles: 128 rows from four
 // blocks per CU on, else 64 (192 x [512 x 512] x [512 x 64]: 7.0 against 7.3 us).
 static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int planes, int out_shift)
@@ -718,20 +719,24 @@ static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int pla
     // 2560 x 1536 x 8192, 120 blocks, 21.0 against 16.5 on 240 blocks of 128 x 128), except from a few blocks more than one
     // a unit (11008 x 768 x 4096: 258, 11008 x 640 x 8192 likewise) to one and a half (6144 x 2048 x 16384: 384 blocks, 72.6
     // against 71.3), which would leave the launch waiting for the units that run two blocks each while three blocks of
-    // the next tile down fit every unit at once: those go to the next tile down
+    // the next tile down fit every unit at once: those go to the next tile down; so do 192 to 256 blocks on fewer than 24
+    // K-tiles (8192 x 768 x 4096: 14.7 us on 128 x 128 with three K-tiles in flight against 16.1)
     const int64_t b21 = blocks(256, 128);
     // a last round that leaves most of the GPU idle (576 blocks on 512 places: 6144 x 3072 x 4096 42.5 us against 34.9 on
     // 128 x 128, whose 1152 blocks fill one and a half rounds of 768 places) goes to the smaller tile
     auto round_fill = [](int64_t b, int64_t places) { return (double)b / (double)(cdiv(b, places) * places); };
-    const bool last_round_idle = KT >= 8 && KT <= 16 && b21 > 256 &&      // (on a longer K the larger tile's cheaper loop makes up for it)
+    const bool last_round_idle = KT >= 8 && (KT <= 16 || b21 <= 600) && b21 > 256 &&      // (on a longer K the larger tile's cheaper loop makes up for it,
+                                                                                           //  but for a few blocks past one round: 9216 x 2048 x 8192, 576 blocks, 56.4 against 59.8 us)
                                  round_fill(blocks(128, 128), 768) >= round_fill(b21, 512) + 0.15 &&
                                  filled(128, 128) >= 0.6;
-    if (planes == 1 && !last_round_idle && (b21 >= 512 || (KT >= 16 && b21 >= 132 && !(b21 > 256 && b21 <= 384))) &&
-        (KT >= (out_shift == 1 ? 8 : 4) || blocks(128, 128) < 512) &&      // (2-byte outputs leave 128 x 128 without staging in LDS:
-        filled(256, 128) >= 0.75)                                          //  48 x [2048 x 2048] x 1024 -> fp16 117 against 131 us)
+    if (planes == 1 && !last_round_idle && (b21 >= 512 || (KT >= 16 && b21 >= 132 && (b21 < 192 || KT >= 24) && !(b21 > 256 && b21 <= 384))) &&
+        (KT >= 8 || (out_shift == 2 && KT >= 4 && batch * N * M >= (64 << 20)) || blocks(128, 128) < 512) &&      // (2-byte outputs leave 128 x 128 without staging in LDS:
+        filled(256, 128) >= 0.75)                                          //  48 x [2048 x 2048] x 1024 -> fp16 117 against 131 us; int32 on 4 to 7 K-tiles: the larger tile
+                                                                           //  from 256 MiB of output on, 8192^2 x 1024 58.7 against 69.9 us, below that the smaller one, 16384 x 2048 x 1024 27.7 against 32.8)
         return {BGEMM_KERNEL_MFMA_256x128, 256, 128};
-    // (with its pipelined loop, from eight K-tiles on, 192 blocks are enough: 3072 x 1024 x 8192 15.9 us against 17.3 to 20.1)
-    if ((blocks(128, 128) >= 512 || (planes == 1 && KT >= 8 && blocks(128, 128) >= 192)) && filled(128, 128) >= 0.6)
+    // (with its pipelined loop, from eight K-tiles on, 192 blocks are enough: 3072 x 1024 x 8192 15.3 us against 17.3 to 20.1;
+    // from 32 K-tiles on 144: 6144 x 384 x 11008 16.9 against 18.9 to 22.9)
+    if ((blocks(128, 128) >= 512 || (planes == 1 && KT >= 8 && blocks(128, 128) >= (KT >= 32 ? 144 : 192))) && filled(128, 128) >= 0.6)
         return {BGEMM_KERNEL_MFMA_128x128, 128, 128};
     // two bit planes: 32 x 256 shares every weight expansion between the planes of one row tile (W[11008,4096] x 128
     // ternary rows 9.7 us against 10.9 / 11.3 on the next two; W[12288,11008] x 384 rows 47.4 against 55.7), once it

@@ -795,9 +795,9 @@ __global__ __launch_bounds__(KW * 64, 2) void gemm_skinny_splitk_quad_kernel(con
 // Shapes the four-pieces kernel takes: at least two tile rows on either side, enough blocks to give every
 // compute unit one, and a K long enough for the shared expansions to outweigh the larger meeting area (timed
 // against both neighbours, weights from HBM and from a warm cache, pieces = 32 x 32 outputs).  One bit plane:
-// up to 1024 pieces from 16 K-tiles on, 2048 from 24, 3072 from 40 (6144 x 512 x 11008: 19.7 us against 24.6 on 128 x 128), 4096 from 48 (2048^2 x 8192, 4096 pieces at 32 K-tiles: 18.4 us here,
-// 16.7 on the general kernel's pipelined 128 x 128 tile; 8192 x 768 x 16384, 6144 pieces: 49 us here, 42 on its
-// 256 x 128 tile even at three quarters of a block per unit).  Two planes (twice the
+// up to 1024 pieces from 16 K-tiles on, 2048 from 24 (8192 x 256 x 16384: 18.7 us against 23.8 on the general kernel's
+// pipelined 128 x 128 tile; beyond that the tile is ahead: 6144 x 384 x 11008, 2304 pieces, 16.9 against 18.9 here; 8192 x
+// 512 x 12288, 4096 pieces, 21.3 against 24.9).  Two planes (twice the
 // matrix-core work per piece): up to 2048 pieces from 24 K-tiles on, 3072 from 32, 4096 from 40, from 256 blocks (192
 // from 40 K-tiles on: W[4096,11008] x 96 ternary rows 8.2 us against 9.3 on one piece a block).  Beyond that
 // the general kernel's 128- and 256-row tiles re-read less.
@@ -809,7 +809,7 @@ static bool skinny_quad_shape(int planes, int64_t batch, int64_t MT, int64_t NT,
     if (planes == 2)
         return batch * cdiv(MT, 2) * NT >= (KT >= 40 ? 192 : 256) && pieces <= (KT >= 40 ? 4096 : KT >= 32 ? 3072 : KT >= 24 ? 2048 : 0);
     if (batch * cdiv(MT, 2) * cdiv(NT, 2) < (KT >= 40 ? 192 : 256)) return false;      // (7168 x 128 x 11008, 224 blocks: 9.9 us against 11.8 on one piece a block)
-    return pieces <= (KT >= 48 ? 4096 : KT >= 40 ? 3072 : KT >= 24 ? 2048 : KT >= 16 ? 1024 : 0);
+    return pieces <= (KT >= 24 ? 2048 : KT >= 16 ? 1024 : 0);
 }
 
 // Shapes the skinny kernels take: one group of activation rows always (32 rows, or 16 rows of two bit planes).

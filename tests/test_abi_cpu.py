@@ -108,14 +108,16 @@ def test_dispatch_of_the_benchmark_configurations():
     assert kid(MODE_XOR, 1, 11008, 512, 8192, 1, A) == B.KERNEL_MFMA_256x128     # 172 blocks: 0.67 a unit is enough
     assert kid(MODE_XOR, 1, 11008, 640, 8192, 1, A) == B.KERNEL_MFMA_128x128     # 258 again
     assert kid(MODE_XOR, 1, 8192, 768, 16384, 1, A) == B.KERNEL_MFMA_256x128
-    assert kid(MODE_XOR, 1, 8192, 512, 16384, 1, A) == B.KERNEL_SKINNY_QUAD
+    assert kid(MODE_XOR, 1, 8192, 512, 16384, 1, A) == B.KERNEL_MFMA_128x128     # 4096 pieces: past the four-pieces kernel's 2048
+    assert kid(MODE_XOR, 1, 6144, 384, 11008, 1, A) == B.KERNEL_MFMA_128x128     # 144 blocks on a long K
     assert kid(MODE_BWTA, 1, 11008, 64, 4096, 1, A) == B.KERNEL_SKINNY_SPLITK
     assert kid(MODE_XOR, 1, 8192, 2048, 4096, 1, A) == B.KERNEL_MFMA_256x128
     assert kid(MODE_XOR, 1, 8192, 2048, 16384, 4, A) == B.KERNEL_MFMA_256x128
     assert kid(MODE_XOR, 1, 8192, 256, 16384, 1, A) == B.KERNEL_SKINNY_QUAD
     assert kid(MODE_ATTN_X, 192, 64, 512, 512, 1, A) == B.KERNEL_MFMA_64x64
     assert kid(MODE_ATTN_X, 384, 64, 512, 512, 1, A) == B.KERNEL_MFMA_128x64
-    assert kid(MODE_XOR, 1, 4096, 2048, 4096, 1, A) == B.KERNEL_MFMA_256x128
+    assert kid(MODE_XOR, 1, 4096, 2048, 4096, 1, A) == B.KERNEL_MFMA_128x128     # 256 blocks of 256 x 128 on 16 K-tiles: the next tile down
+    assert kid(MODE_XOR, 1, 4096, 2048, 8192, 1, A) == B.KERNEL_MFMA_256x128
     # a short K with a 2-byte output takes the tile with 512-byte rows
     assert B.lib().bgemm_packed_kernel_id(MODE_XOR, B.OUT_F16, 192, 512, 512, 64, 1, A) == B.KERNEL_MFMA_32x256
     assert kid(MODE_XOR, 192, 512, 512, 64, 1, A) == B.KERNEL_MFMA_128x128

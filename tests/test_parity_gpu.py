@@ -280,7 +280,7 @@ def test_decode_batches_of_ternary_rows(M, N, K):
 
 
 @pytest.mark.parametrize("batch,M,N,K", [(1, 4040, 270, 6200), (4, 1000, 250, 6200), (1, 8192, 256, 8192),
-                                         (1, 4096, 768, 12288), (1, 4096, 512, 8192)])      # the last two: four / two K ways, several blocks a CU
+                                         (1, 4096, 384, 12288), (1, 4096, 512, 8192)])      # the last two: four / two K ways, several blocks a CU
 def test_split_k_in_block_four_pieces_a_block(oracle, batch, M, N, K):
     """Outputs of one to two thousand 32 x 32 pieces over a long K: a block takes two weight row tiles and two
     activation tile rows (odd tile counts, ragged M, N and K, batches); every one-plane mode, both engines,

@@ -318,8 +318,8 @@ def test_stream_kernel_up_to_four_rows_one_store_a_row(engine):
 
 
 @pytest.mark.parametrize("N,want_kernel", [(256, B.KERNEL_SKINNY_QUAD), (2048, B.KERNEL_MFMA_256x128),
-                                           # 640 and 1024 blocks of four pieces: four and two K ranges a block, several blocks a CU
-                                           (320, B.KERNEL_SKINNY_QUAD), (512, B.KERNEL_SKINNY_QUAD)])
+                                           # 192 and 256 blocks of 128 x 128 on 64 K-tiles (three K-tiles in flight)
+                                           (320, B.KERNEL_MFMA_128x128), (512, B.KERNEL_MFMA_128x128)])
 def test_config5_sweep_long_k(N, want_kernel):
     """The K = 16384 points of configuration 5's sweep, split-K 1 / 2 / 4: sampled rows and columns against the
     closed form, identities over the whole output, and agreement between the split-K values and the designs."""
