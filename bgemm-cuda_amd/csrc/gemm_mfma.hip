@@ -59,8 +59,8 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
     // slots rotated by half against each other, slot i of wave wm holding tile row nt0 + (i ^ xs): each wave then
     // counts the bits of its first WN / 2 slots only, which are different rows for the two, and they swap the
     // counts through LDS before the epilogue (half the activation side's popcounts: 0.25 vector instructions a MFMA).
-    static_assert(!PIPE || (WGM == 2 && WN % 2 == 0), "the popcount split is laid out for two waves along M");
-    const int xs = PIPE ? wm * (WN / 2) : 0;
+    static_assert(!PIPE || (WGM == 2 && (PL * WN) % 2 == 0), "the popcount split is laid out for two waves along M");
+    const int xs = PIPE && PL == 1 ? wm * (WN / 2) : 0;      // (two bit planes: every wave counts all its activation slots)
     auto x_tile = [&](const int i) { return nt0 + (i ^ xs); };
 
     // per-fragment base pointers (row tile clamped so ragged edges re-read a valid tile)
@@ -109,14 +109,15 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
         // ops that fit in the MFMA's shadow); a scheduling barrier after each such group keeps the
         // compiler from clustering them.  Two raw tile buffers ping-pong: while K-tile kt is consumed
         // from A, B holds kt+1, and A is refilled with kt+2 during kt's last step.
-        static_assert(PL == 1, "pipelined loop is built for one activation plane");
-        constexpr int NF = WN + WM, ND = NF * 4, NM = WN * WM, STEPS = Eng::STEPS;
+        // Two bit planes: the activation slots are the WN tile rows of the first plane, then the same rows of the second
+        // (XN = PL * WN slots); a 128 x 128 tile of two planes has the fragments and accumulators of a 256 x 128 tile of one.
+        constexpr int XN = PL * WN, NF = XN + WM, ND = NF * 4, NM = XN * WM, STEPS = Eng::STEPS;
         static_assert(ND % NM == 0 && NF <= NM && STEPS % 2 == 0, "tile shape does not pipeline");
         constexpr int DPG = ND / NM;                       // expanded registers produced per MFMA
         // Both operands have one layout and the two expansions are each other's mirror (every product of set bits
         // is 1 either way round), so the side with more fragments a wave gets the cheaper one (five instructions a
         // word against six): the activation side's four fragments on the 256 x 128 tile.
-        constexpr bool XS_FIRST = WN <= WM;                // true: activation fragments take the activation-side expansion
+        constexpr bool XS_FIRST = XN <= WM;                // true: activation fragments take the activation-side expansion
         // Every fragment's row of K-tiles is a buffer of its own (a wave-uniform base in scalar registers, KT KiB
         // long), so all loads of a K-tile share ONE per-lane offset, lane * 16 + kt * 1024: no address arithmetic
         // per load, and K-tiles past the range read as zero bits (a buffer load out of range returns 0; zero bits
@@ -126,8 +127,8 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
         __amdgpu_buffer_rsrc_t rs[NF];
 #pragma unroll
         for (int f = 0; f < NF; f++) {
-            const int64_t rt = f < WN ? min(x_tile(f), a.NT - 1) : min(mt0 + (f - WN), a.MT - 1);
-            const uint4* base = (f < WN ? Xb : Wb) + rt * a.KT * TILE_U4;
+            const int64_t rt = f < XN ? min(x_tile(f % WN), a.NT - 1) : min(mt0 + (f - XN), a.MT - 1);
+            const uint4* base = (f < WN ? Xb : f < XN ? X2b : Wb) + rt * a.KT * TILE_U4;
             rs[f] = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint4*>(base), 0, a.KT * (TILE_U4 * 16), 0x00020000);
         }
         // Raw K-tiles in flight: two buffers (a K-tile requested one tile ahead of its first use), or three where the
@@ -150,14 +151,14 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
                 unsigned (&nxt)[NF][4] = buf[(s + 1) & 1];
 #pragma unroll
                 for (int q = 0; q < NM; q++) {
-                    const int i = q / WM, j = q % WM;
-                    acc[0][i][j] = Eng::mma(Eng::make(cur[i]), Eng::make(cur[WN + j]), acc[0][i][j]);
+                    const int u = q / WM, j = q % WM;              // activation slot: plane u / WN, tile row u % WN
+                    acc[u / WN][u % WN][j] = Eng::mma(Eng::make(cur[u]), Eng::make(cur[XN + j]), acc[u / WN][u % WN][j]);
 #pragma unroll
                     for (int d = q * DPG; d < (q + 1) * DPG; d++)
-                        nxt[d / 4][d % 4] = (d / 4 < WN) == XS_FIRST      // fragments 0 .. WN-1 are the activation side
+                        nxt[d / 4][d % 4] = (d / 4 < XN) == XS_FIRST      // fragments 0 .. XN-1 are the activation side
                             ? (s + 1 < STEPS ? Eng::expand1_x(A[d / 4][d % 4], s + 1) : Eng::expand1_x(B[d / 4][d % 4], 0))
                             : (s + 1 < STEPS ? Eng::expand1_w(A[d / 4][d % 4], s + 1) : Eng::expand1_w(B[d / 4][d % 4], 0));
-                    if (!COUNTED && s == 0 && (q < WN / 2 || (q >= WN && q < NF))) {     // v_bcnt adds into its accumulator: four instructions a fragment, written out
+                    if (!COUNTED && s == 0 && (q < (PL == 1 ? WN / 2 : XN) || (q >= XN && q < NF))) {     // v_bcnt adds into its accumulator: four instructions a fragment, written out
 #pragma unroll                                  // because the compiler prefers four counts and two three-way adds
                         for (int c = 0; c < 4; c++) asm("v_bcnt_u32_b32 %0, %1, %0" : "+v"(pop[q]) : "v"(A[q][c]));
                     }
@@ -175,7 +176,7 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
 #pragma unroll
             for (int f = 0; f < NF; f++)
 #pragma unroll
-                for (int c = 0; c < 4; c++) buf[0][f][c] = (f < WN) == XS_FIRST ? Eng::expand1_x(rawA[f][c], 0) : Eng::expand1_w(rawA[f][c], 0);
+                for (int c = 0; c < 4; c++) buf[0][f][c] = (f < XN) == XS_FIRST ? Eng::expand1_x(rawA[f][c], 0) : Eng::expand1_w(rawA[f][c], 0);
             if constexpr (NBUF == 3) {
                 // whole rounds of three, then what is left in the same rotation (a K-tile past the range multiplies zeros)
                 int kt = kt0;
@@ -203,6 +204,11 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
             for (int i = 0; i < WN; i++) pb[0][i] = a.cntX[cx + min((int64_t)x_tile(i) * 32 + (lane & 31), a.N - 1)];
 #pragma unroll
             for (int j = 0; j < WM; j++) pa[j] = a.cntW[cw + min((int64_t)(mt0 + j) * 32 + (lane & 31), a.M - 1)];
+        } else if constexpr (PL == 2) {
+#pragma unroll
+            for (int u = 0; u < XN; u++) pb[u / WN][u % WN] = pop[u] + __shfl_xor(pop[u], 32);
+#pragma unroll
+            for (int j = 0; j < WM; j++) pa[j] = pop[XN + j] + __shfl_xor(pop[XN + j], 32);
         } else {
             // the two K-halves of a row meet, then the two waves that share these rows exchange what each counted
             __shared__ int xcnt[WGN][WN][32];
@@ -738,6 +744,7 @@ static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int pla
     // from 32 K-tiles on 144: 6144 x 384 x 11008 16.9 against 18.9 to 22.9)
     if ((blocks(128, 128) >= 512 || (planes == 1 && KT >= 8 && blocks(128, 128) >= (KT >= 32 ? 144 : 192))) && filled(128, 128) >= 0.6)
         return {BGEMM_KERNEL_MFMA_128x128, 128, 128};
+    if (planes == 2 && two_plane_tile_128(batch, M, N, KT)) return {BGEMM_KERNEL_MFMA_128x128, 128, 128};
     // two bit planes: 32 x 256 shares every weight expansion between the planes of one row tile (W[11008,4096] x 128
     // ternary rows 9.7 us against 10.9 / 11.3 on the next two; W[12288,11008] x 384 rows 47.4 against 55.7), once it
     // has 160 blocks
@@ -755,10 +762,20 @@ static int launch_cfg(const GemmArgs& a, hipStream_t st)
     if (grid <= 0 || grid > 0x7fffffffLL) return fail(BGEMM_EINVAL, "gemm_mfma: grid of %lld blocks", (long long)grid);
     if (a.mc.planes == 2) {
         // two accumulator sets: only the tiles whose registers fit are built for two planes
-        if constexpr (WN * WM <= 4)
+        if constexpr (WN * WM <= 4) {
+            // 128 x 128 of two planes has the fragments and accumulators of 256 x 128 of one and runs its hand-pipelined
+            // loop, from the same K on as the one-plane tile
+            if constexpr (WGN == 2 && WGM == 2 && WN == 2 && WM == 2) {
+                const bool pairs2 = a.out_kind == BGEMM_OUT_F16 && a.vec_store == 8;
+                if (a.KT >= 8 && (!pairs2 || a.KT >= 16)) {
+                    hipLaunchKernelGGL((gemm_mfma_kernel<Eng, WGN, WGM, WN, WM, 2, true>), dim3((unsigned)grid),
+                                       dim3(WGN * WGM * 64), 0, st, a, tiles_n, tiles_m);
+                    return check_launch("gemm_mfma");
+                }
+            }
             hipLaunchKernelGGL((gemm_mfma_kernel<Eng, WGN, WGM, WN, WM, 2, false>), dim3((unsigned)grid),
                                dim3(WGN * WGM * 64), 0, st, a, tiles_n, tiles_m);
-        else
+        } else
             return fail(BGEMM_EINVAL, "gemm_mfma: tile not built for two planes");
     } else {
         // The hand-pipelined loop: always on the tiles of eight and sixteen MFMA tiles a wave; on 128 x 128 from eight

@@ -801,11 +801,13 @@ __global__ __launch_bounds__(KW * 64, 2) void gemm_skinny_splitk_quad_kernel(con
 // matrix-core work per piece): up to 2048 pieces from 24 K-tiles on, 3072 from 32, 4096 from 40, from 256 blocks (192
 // from 40 K-tiles on: W[4096,11008] x 96 ternary rows 8.2 us against 9.3 on one piece a block).  Beyond that
 // the general kernel's 128- and 256-row tiles re-read less.
-static bool skinny_quad_shape(int planes, int64_t batch, int64_t MT, int64_t NT, int64_t KT)
+static bool skinny_quad_shape(int planes, int64_t batch, int64_t M, int64_t N, int64_t KT)
 {
+    const int64_t MT = row_tiles(M), NT = row_tiles(N);
     if (MT < 2 || NT < 2) return false;
     if (batch > 1 && KT < 24) return false;      // (a batch of small products: operands that were just written, see gemm_skinny_shape)
     const int64_t pieces = batch * MT * NT;
+    if (planes == 2 && two_plane_tile_128(batch, M, N, KT)) return false;      // (the general kernel's pipelined tile is ahead there)
     if (planes == 2)
         return batch * cdiv(MT, 2) * NT >= (KT >= 40 ? 192 : 256) && pieces <= (KT >= 40 ? 4096 : KT >= 32 ? 3072 : KT >= 24 ? 2048 : 0);
     if (batch * cdiv(MT, 2) * cdiv(NT, 2) < (KT >= 40 ? 192 : 256)) return false;      // (7168 x 128 x 11008, 224 blocks: 9.9 us against 11.8 on one piece a block)
@@ -824,7 +826,7 @@ bool gemm_skinny_shape(int planes, int64_t batch, int64_t M, int64_t N, int64_t 
     if (batch > 65535) return false;             // these kernels walk the batch in the grid's third dimension
     if (N <= (planes == 2 ? 16 : 32)) return true;
     const int64_t pieces = batch * row_tiles(M) * row_tiles(N), KT = k_tiles(K);
-    if (skinny_quad_shape(planes, batch, row_tiles(M), row_tiles(N), KT)) return true;
+    if (skinny_quad_shape(planes, batch, M, N, KT)) return true;
     // (a batch of products is attention-shaped work on operands that were just written and still sit in the caches:
     // there the general kernel keeps up from 512 pieces on; 8 x [128 x 1024] x 2048, 1024 pieces: 4.3 us there, 5.1 here)
     if (KT >= 8) return pieces <= (batch > 1 ? 512 : 1024);
@@ -851,7 +853,7 @@ static int launch_splitk_fusex(const GemmArgs& a, hipStream_t st)
     return check_launch("gemm_skinny");
 }
 
-static bool skinny_quad(const GemmArgs& a) { return skinny_quad_shape(a.mc.planes, a.batch, a.MT, a.NT, a.KT); }
+static bool skinny_quad(const GemmArgs& a) { return skinny_quad_shape(a.mc.planes, a.batch, a.M, a.N, a.KT); }
 
 template <typename Eng, bool TWO>
 static int launch_splitk_quad(const GemmArgs& a, hipStream_t st)

@@ -140,6 +140,13 @@ def test_128x128_takes_the_pipelined_loop_from_eight_k_tiles(oracle, engine, M, 
     check_all_kinds(oracle, wp, xp, acc, M, N, variant, rng)
     lk.row_popcounts(wp), lk.row_popcounts(xp)
     assert (lk.bgemm_packed_forward(wp, xp, MODE_XOR, torch.int32, 1, variant)[0].cpu().numpy() == acc).all()
+    # a ternary operand's two planes on the same loop (the tile then has the fragments of 256 x 128 of one plane)
+    t = x.copy()
+    t[rng.random(t.shape) < 0.3] = 0
+    xt, want = lk.pack_ternary(to_dev(t)), dense(MODE_BWTA, w, t)
+    assert (lk.bgemm_packed_forward(wp, xt, MODE_BWTA, torch.int32, 1, variant)[0].cpu().numpy() == want).all()
+    goth = lk.bgemm_packed_forward(wp, xt, MODE_BWTA, torch.half, 1, variant)[0].cpu().numpy()
+    assert (bits_of(goth) == bits_of(f16_of(want))).all()
 
 
 @pytest.mark.parametrize("engine", list(ENGINES))
