@@ -612,6 +612,32 @@ def section_decode(cold):
     return rows
 
 
+def bench_prefill(steps=20, warmup=5):
+    """Binary weights x a batch of ternary rows (a prefill step, or a batch of decode steps): the two bit planes of the
+    activations are two matrix-core products against one expansion of the weights, so the matrix cores do 4*M*N*K of work
+    for the 2*M*N*K effective operations that `tops` counts; `frac` is the matrix-core work against the fp4 peak."""
+    import torch
+    import lowbit_kernel as lk
+    dev = torch.device("cuda:0")
+    rows = []
+    for name, M, N, K in (("Llama-7B gate+up fused", 22016, 2048, 4096), ("Llama-7B down", 4096, 2048, 11008), ("square", 8192, 8192, 8192)):
+        w16, x16 = pm1_f16((M, K), 6001, dev), ternary_f16((N, K), 6002, dev)
+        wp, xt = lk.pack_sign(w16), lk.pack_ternary(x16)
+        out = torch.empty((1, N, M), dtype=torch.int32, device=dev)
+        fn = lambda i: lk.bgemm_packed_forward(wp, xt, lk.MODE_BWTA, torch.int32, 1, 0, out=out)
+        for i in range(50):
+            fn(i)
+        ms = time_gpu(fn, warmup, steps)
+        ok = check_sampled(out[0], w16, x16)
+        r = row("BWTA %s W[%d,%d] x %d ternary rows, int32" % (name, M, K, N), ms, 2.0 * M * N * K,
+                M * K / 8 + 2 * N * K / 8 + 4.0 * M * N, ok, kernel_of(wp, xt, lk.MODE_BWTA), "mfma")
+        r["roofline"] = {"bound": "mfma", "frac": round(2 * r["tops"] / FP4_MFMA_PEAK_TOPS, 4), "mfma_work": "two products a weight expansion: 4*M*N*K"}
+        rows.append(r)
+        log(json.dumps(r))
+        del w16, x16, wp, xt, out
+    return rows
+
+
 def all_configs(cold):
     rows = [bench_c2()]
     log(json.dumps(rows[-1]))
@@ -621,6 +647,7 @@ def all_configs(cold):
     log(json.dumps(rows[-1]))
     rows += section_decode(cold)
     rows += bench_sweep()
+    rows += bench_prefill()
     rows.append(bench_c5_dropin(20, 3))
     log(json.dumps(rows[-1]))
     return rows
@@ -632,7 +659,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--headline-only", action="store_true", help="time the 8192^3 launch only (profiling runs)")
-    ap.add_argument("--only", choices=["c2", "c3", "c4", "sweep", "floor", "peak", "thresholds"],
+    ap.add_argument("--only", choices=["c2", "c3", "c4", "sweep", "prefill", "floor", "peak", "thresholds"],
                     help="time just that section and print it (for profiling and for re-deriving the dispatch thresholds)")
     ap.add_argument("--variant", type=int, default=0, help="0 auto, 1 VALU, 2 MFMA int8, 3 MFMA fp4")
     ap.add_argument("--split-k", type=int, default=1,
@@ -662,7 +689,7 @@ def main():
         del src, dst
     if args.only:
         cold = ColdRead() if args.only in ("c4", "floor", "peak") else None
-        res = {"c2": lambda: [bench_c2()], "c3": lambda: [bench_c3(), bench_qk()], "c4": lambda: section_decode(cold),
+        res = {"c2": lambda: [bench_c2()], "c3": lambda: [bench_c3(), bench_qk()], "c4": lambda: section_decode(cold), "prefill": bench_prefill,
                "sweep": bench_sweep, "floor": lambda: bench_floor(cold), "peak": lambda: bench_mfma_peak(cold),
                "thresholds": bench_thresholds}[args.only]()
         print(json.dumps({args.only: res}), flush=True)
