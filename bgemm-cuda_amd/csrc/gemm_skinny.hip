@@ -804,7 +804,9 @@ __global__ __launch_bounds__(KW * 64, 2) void gemm_skinny_splitk_quad_kernel(con
 static bool skinny_quad_shape(int planes, int64_t batch, int64_t M, int64_t N, int64_t KT)
 {
     const int64_t MT = row_tiles(M), NT = row_tiles(N);
-    if (MT < 2 || NT < 2) return false;
+    // (two planes: one tile row of more than 16 rows as well: the block's two operands are its two planes; up to 16 rows
+    // both planes share ONE operand on the one-piece kernel, half the matrix-core work)
+    if (MT < 2 || (planes == 2 ? N <= 16 : NT < 2)) return false;
     if (batch > 1 && KT < 24) return false;      // (a batch of small products: operands that were just written, see gemm_skinny_shape)
     const int64_t pieces = batch * MT * NT;
     if (planes == 2 && two_plane_tile_128(batch, M, N, KT)) return false;      // (the general kernel's pipelined tile is ahead there)

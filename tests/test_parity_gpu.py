@@ -257,7 +257,8 @@ def test_config4_decode_bwta(N):
     assert (goth.view(np.uint16) == f16_of(want).view(np.uint16)).all()
 
 
-@pytest.mark.parametrize("M,N,K", [(11008, 17, 4096), (11008, 40, 4096), (4096, 100, 4096), (1000, 130, 2304), (70, 250, 1000)])
+@pytest.mark.parametrize("M,N,K", [(11008, 17, 4096), (11008, 40, 4096), (4096, 100, 4096), (1000, 130, 2304), (70, 250, 1000),
+                                   (16400, 20, 6200)])      # one tile row of two planes on the four-pieces kernel
 def test_decode_batches_of_ternary_rows(M, N, K):
     """More than 16 ternary rows (a batch of decode steps): the two bit planes are taken 16 rows at a time by the
     kernel that splits K inside a block, also over ragged M, N and K; same integers as the dense reference, and the
@@ -267,6 +268,8 @@ def test_decode_batches_of_ternary_rows(M, N, K):
     t = rng.choice(np.array([-1, 0, 0, 1], dtype=np.float16), size=(N, K)).astype(np.float16)
     want = dense_ref(MODE_BWTA, w, t)
     wp, xt = lk.pack_sign(to_dev(w)), lk.pack_ternary(to_dev(t))
+    if M == 16400:
+        assert lk.packed_kernel_id(wp, xt, MODE_BWTA) == _lib.KERNEL_SKINNY_QUAD
     for variant in [VARIANT_AUTO] + VARIANTS:
         got = lk.bgemm_packed_forward(wp, xt, MODE_BWTA, torch.int32, 1, variant)[0].cpu().numpy()
         assert (got == want).all(), variant
