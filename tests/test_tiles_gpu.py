@@ -147,6 +147,9 @@ def test_128x128_takes_the_pipelined_loop_from_eight_k_tiles(oracle, engine, M, 
     assert (lk.bgemm_packed_forward(wp, xt, MODE_BWTA, torch.int32, 1, variant)[0].cpu().numpy() == want).all()
     goth = lk.bgemm_packed_forward(wp, xt, MODE_BWTA, torch.half, 1, variant)[0].cpu().numpy()
     assert (bits_of(goth) == bits_of(f16_of(want))).all()
+    sw, sa = rng.uniform(1e-4, 3e-3, M).astype(np.float32), np.asarray(0.61, dtype=np.float32)
+    gots = lk.bgemm_packed_forward(wp, xt, MODE_BWTA, splitK=1, variant=variant, scale=(to_dev(sw), to_dev(sa.reshape(1)), None))[0].cpu().numpy()
+    assert (bits_of(gots) == bits_of(oracle.np_scale_epilogue(want, sw, sa, None))).all()
 
 
 @pytest.mark.parametrize("engine", list(ENGINES))
