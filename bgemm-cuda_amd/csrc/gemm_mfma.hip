@@ -59,7 +59,7 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
     // slots rotated by half against each other, slot i of wave wm holding tile row nt0 + (i ^ xs): each wave then
     // counts the bits of its first WN / 2 slots only, which are different rows for the two, and they swap the
     // counts through LDS before the epilogue (half the activation side's popcounts: 0.25 vector instructions a MFMA).
-    static_assert(!PIPE || (WGM == 2 && (PL * WN) % 2 == 0), "the popcount split is laid out for two waves along M");
+    static_assert(!PIPE || PL == 2 || (WGM == 2 && WN % 2 == 0), "the popcount split is laid out for two waves along M");
     const int xs = PIPE && PL == 1 ? wm * (WN / 2) : 0;      // (two bit planes: every wave counts all its activation slots)
     auto x_tile = [&](const int i) { return nt0 + (i ^ xs); };
 
@@ -747,8 +747,9 @@ static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int pla
     if (planes == 2 && two_plane_tile_128(batch, M, N, KT)) return {BGEMM_KERNEL_MFMA_128x128, 128, 128};
     // two bit planes: 32 x 256 shares every weight expansion between the planes of one row tile (W[11008,4096] x 128
     // ternary rows 9.7 us against 10.9 / 11.3 on the next two; W[12288,11008] x 384 rows 47.4 against 55.7), once it
-    // has 160 blocks
-    if (planes == 2 && blocks(32, 256) >= 160) return {BGEMM_KERNEL_MFMA_32x256, 32, 256};
+    // has 160 blocks (96 from eight K-tiles on, where it runs the pipelined loop: W[11008,4096] x 96 ternary rows 8.4 us
+    // against 10.0 on 32 x 128)
+    if (planes == 2 && blocks(32, 256) >= (KT >= 8 ? 96 : 160)) return {BGEMM_KERNEL_MFMA_32x256, 32, 256};
     if (blocks(64, 128) >= 512 && filled(64, 128) >= 0.6) return {BGEMM_KERNEL_MFMA_64x128, 64, 128};      // below two blocks a unit, twice as many 32-row tiles are faster
     return {BGEMM_KERNEL_MFMA_32x128, 32, 128};
 }
@@ -764,8 +765,10 @@ static int launch_cfg(const GemmArgs& a, hipStream_t st)
         // two accumulator sets: only the tiles whose registers fit are built for two planes
         if constexpr (WN * WM <= 4) {
             // 128 x 128 of two planes has the fragments and accumulators of 256 x 128 of one and runs its hand-pipelined
-            // loop, from the same K on as the one-plane tile
-            if constexpr (WGN == 2 && WGM == 2 && WN == 2 && WM == 2) {
+            // loop, from the same K on as the one-plane tile; so does 32 x 256 (a wave: one tile row of both planes against
+            // two weight tiles, four MFMAs a step; W[11008,4096] x 128 ternary rows 10.3 -> 9.1 us, W[22016,4096] x 128 17.5 ->
+            // 14.8, W[11008,8192] x 320 28.5 -> 24.0)
+            if constexpr ((WGN == 2 && WGM == 2 && WN == 2 && WM == 2) || (WGN == 1 && WGM == 4 && WN == 1 && WM == 2)) {
                 const bool pairs2 = a.out_kind == BGEMM_OUT_F16 && a.vec_store == 8;
                 if (a.KT >= 8 && (!pairs2 || a.KT >= 16)) {
                     hipLaunchKernelGGL((gemm_mfma_kernel<Eng, WGN, WGM, WN, WM, 2, true>), dim3((unsigned)grid),

@@ -798,9 +798,8 @@ __global__ __launch_bounds__(KW * 64, 2) void gemm_skinny_splitk_quad_kernel(con
 // up to 1024 pieces from 16 K-tiles on, 2048 from 24 (8192 x 256 x 16384: 18.7 us against 23.8 on the general kernel's
 // pipelined 128 x 128 tile; beyond that the tile is ahead: 6144 x 384 x 11008, 2304 pieces, 16.9 against 18.9 here; 8192 x
 // 512 x 12288, 4096 pieces, 21.3 against 24.9).  Two planes (twice the
-// matrix-core work per piece): up to 2048 pieces from 24 K-tiles on, 3072 from 32, 4096 from 40, from 256 blocks (192
-// from 40 K-tiles on: W[4096,11008] x 96 ternary rows 8.2 us against 9.3 on one piece a block).  Beyond that
-// the general kernel's 128- and 256-row tiles re-read less.
+// matrix-core work per piece): from 24 K-tiles on, from 256 blocks (192 from 40 K-tiles on: W[4096,11008] x 96 ternary
+// rows 8.2 us against 9.3 on one piece a block) up to 512.  Beyond that the general kernel's tiles re-read less.
 static bool skinny_quad_shape(int planes, int64_t batch, int64_t M, int64_t N, int64_t KT)
 {
     const int64_t MT = row_tiles(M), NT = row_tiles(N);
@@ -811,7 +810,14 @@ static bool skinny_quad_shape(int planes, int64_t batch, int64_t M, int64_t N, i
     const int64_t pieces = batch * MT * NT;
     if (planes == 2 && two_plane_tile_128(batch, M, N, KT)) return false;      // (the general kernel's pipelined tile is ahead there)
     if (planes == 2)
-        return batch * cdiv(MT, 2) * NT >= (KT >= 40 ? 192 : 256) && pieces <= (KT >= 40 ? 4096 : KT >= 32 ? 3072 : KT >= 24 ? 2048 : 0);
+    {
+        // one round of blocks (up to 512: four K ways, two blocks a CU); with more, the general kernel's 32 x 256 tile,
+        // which runs two planes on its pipelined loop, is ahead (8192 x 160 ternary rows x 8192, 640 blocks: 13.2 us
+        // there against 16.0 here; 11008 x 96 x 8192, 516 blocks: 13.4 against 16.7; 8192 x 128 x 8192, 512 blocks: 13.3
+        // against 11.7)
+        const int64_t blocks2 = batch * cdiv(MT, 2) * NT;
+        return KT >= 24 && blocks2 >= (KT >= 40 ? 192 : 256) && blocks2 <= 512;
+    }
     if (batch * cdiv(MT, 2) * cdiv(NT, 2) < (KT >= 40 ? 192 : 256)) return false;      // (7168 x 128 x 11008, 224 blocks: 9.9 us against 11.8 on one piece a block)
     return pieces <= (KT >= 24 ? 2048 : KT >= 16 ? 1024 : 0);
 }

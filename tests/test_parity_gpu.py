@@ -293,15 +293,19 @@ def test_split_k_in_block_four_pieces_a_block(oracle, batch, M, N, K):
     x = rand_f16(rng, batch * N, K).reshape(batch, N, K)
     wp, xp = lk.pack_sign(to_dev(w)), lk.pack_sign(to_dev(x))
     xt = lk.pack_ternary(to_dev(x))
-    assert lk.packed_kernel_id(wp, xp, MODE_XOR, 8) == _lib.KERNEL_SKINNY_QUAD and lk.packed_kernel_id(wp, xt, MODE_BWTA, 8) == _lib.KERNEL_SKINNY_QUAD
+    assert lk.packed_kernel_id(wp, xp, MODE_XOR, 8) == _lib.KERNEL_SKINNY_QUAD
+    # two planes take this kernel up to 512 blocks (one round); past that the general kernel's tiles: forced below
+    blocks2 = batch * -(-(-(-M // 32)) // 2) * -(-N // 32)
+    assert (lk.packed_kernel_id(wp, xt, MODE_BWTA, 8) == _lib.KERNEL_SKINNY_QUAD) == (blocks2 <= 512)
     for mode in (MODE_XOR, MODE_AND, MODE_ATTN, MODE_ATTN_X, MODE_BWTA):     # ternary: the two planes of a tile row are the block's two operands
         want = np.stack([dense_ref(mode, w[b], x[b]) for b in range(batch)])
         xo = xt if mode == MODE_BWTA else xp
-        for variant in (VARIANT_AUTO, VARIANT_MFMA):
+        for variant in (VARIANT_AUTO, VARIANT_MFMA, _lib.force_kernel(_lib.KERNEL_SKINNY_QUAD)):
             got = lk.bgemm_packed_forward(wp, xo, mode, torch.int32, 8, variant).cpu().numpy()
             assert (got == want).all(), (mode, variant)
-        goth = lk.bgemm_packed_forward(wp, xo, mode, torch.half, 1).cpu().numpy()
-        assert (goth.view(np.uint16) == f16_of(want).view(np.uint16)).all(), mode
+        for variant in (VARIANT_AUTO, _lib.force_kernel(_lib.KERNEL_SKINNY_QUAD)):
+            goth = lk.bgemm_packed_forward(wp, xo, mode, torch.half, 1, variant).cpu().numpy()
+            assert (goth.view(np.uint16) == f16_of(want).view(np.uint16)).all(), (mode, variant)
     acc = np.stack([dense_ref(MODE_XOR, w[b], x[b]) for b in range(batch)])
     acct = np.stack([dense_ref(MODE_BWTA, w[b], x[b]) for b in range(batch)]).reshape(batch * N, M)
     swt, sat = rng.uniform(1e-4, 3e-3, M).astype(np.float32), np.asarray(0.61, dtype=np.float32)

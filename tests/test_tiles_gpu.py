@@ -152,6 +152,28 @@ def test_128x128_takes_the_pipelined_loop_from_eight_k_tiles(oracle, engine, M, 
     assert (bits_of(gots) == bits_of(oracle.np_scale_epilogue(want, sw, sa, None))).all()
 
 
+@pytest.mark.parametrize("KT", [9, 17])
+@pytest.mark.parametrize("engine", list(ENGINES))
+@pytest.mark.parametrize("tile", ["128x128", "32x256"])
+def test_two_planes_on_the_pipelined_loop(oracle, tile, engine, KT):
+    """A ternary operand on the two tiles whose two-plane form runs the hand-pipelined loop (from eight K-tiles; fp16
+    pairs from sixteen): ragged M, N and K, an odd K-tile count, int32, fp16 and the scaled output against the dense
+    reference and the oracle's epilogue."""
+    rng = np.random.default_rng(TILES[tile] * 100 + KT)
+    variant = force_kernel(TILES[tile], ENGINES[engine])
+    for M, N in ((520, 515), (517, 130)):
+        K = KT * 256 - 5
+        w, t = pm1(rng, M, K), pm1(rng, N, K)
+        t[rng.random(t.shape) < 0.4] = 0
+        wp, xt, want = lk.pack_sign(to_dev(w)), lk.pack_ternary(to_dev(t)), dense(MODE_BWTA, w, t)
+        assert (lk.bgemm_packed_forward(wp, xt, MODE_BWTA, torch.int32, 1, variant)[0].cpu().numpy() == want).all()
+        goth = lk.bgemm_packed_forward(wp, xt, MODE_BWTA, torch.half, 1, variant)[0].cpu().numpy()
+        assert (bits_of(goth) == bits_of(f16_of(want))).all()
+        sw, sa = rng.uniform(1e-4, 3e-3, M).astype(np.float32), np.asarray(0.61, dtype=np.float32)
+        gots = lk.bgemm_packed_forward(wp, xt, MODE_BWTA, splitK=1, variant=variant, scale=(to_dev(sw), to_dev(sa.reshape(1)), None))[0].cpu().numpy()
+        assert (bits_of(gots) == bits_of(oracle.np_scale_epilogue(want, sw, sa, None))).all()
+
+
 @pytest.mark.parametrize("engine", list(ENGINES))
 @pytest.mark.parametrize("tile", list(TILES))
 def test_each_tile_every_mode_batched(tile, engine):
