@@ -292,7 +292,7 @@ def test_headline_tiles_where_the_library_picks_them(oracle, engine, M, N, K, wa
 
 
 def test_config3_attention_av_all_192_heads():
-    """BASELINE configuration 3 at its full size, every element: 16 x 12 heads, attn {0,1} [512,512] x value +-1 [512,64]."""
+    """The batched attention x value configuration at its full size, every element: 16 x 12 heads, attn {0,1} [512,512] x value +-1 [512,64]."""
     rng = np.random.default_rng(3192)
     Bn, S, D = 192, 512, 64
     attn_bits = rng.integers(0, 2, (Bn, S, S), dtype=np.int8)
