@@ -824,8 +824,8 @@ static bool skinny_quad_shape(int planes, int64_t batch, int64_t M, int64_t N, i
 
 // Shapes the skinny kernels take: one group of activation rows always (32 rows, or 16 rows of two bit planes).
 // More groups where splitting K inside the block buys more than the general kernel's 32 x 128 tiles do (timed
-// over sweeps of shapes, pieces = 32 x 32 outputs): up to 512 pieces from four K-tiles on and up to 1024 from
-// eight, one bit plane or two (two operands a block against one weight expansion).  The last bound is set by
+// over sweeps of shapes, pieces = 32 x 32 outputs): up to 1024 pieces from eight K-tiles on, one bit plane or two (two operands a block against one weight expansion); on four
+// to seven K-tiles up to 512 pieces of two bit planes, or up to two tile rows of activations.  The last bound is set by
 // weights that come from HBM rather than from a warm cache (a model's layers): there the general kernel's serial
 // K loop pays the full memory latency per step.  Beyond, the four-pieces kernel where that pays (see above),
 // else the general one (W[11008,4096] x 128 ternary rows, 1376 pieces: 9.7 us there against 12.5 here).
@@ -838,7 +838,12 @@ bool gemm_skinny_shape(int planes, int64_t batch, int64_t M, int64_t N, int64_t 
     // (a batch of products is attention-shaped work on operands that were just written and still sit in the caches:
     // there the general kernel keeps up from 512 pieces on; 8 x [128 x 1024] x 2048, 1024 pieces: 4.3 us there, 5.1 here)
     if (KT >= 8) return pieces <= (batch > 1 ? 512 : 1024);
-    return KT >= 4 && pieces <= 512;
+    if (KT < 4) return false;
+    if (planes == 2) return pieces <= 512 || (row_tiles(N) <= 2 && pieces <= 1024);      // (11008 x 48 ternary rows x 1792: 4.7 us here against 5.7)
+    // four to seven K-tiles, one bit plane: two tile rows of activations at most (1024 x 384 x 1024: 3.6 us here against 3.2
+    // on 32 x 128 tiles, 2048 x 192 x 1792: 4.1 against 3.7; 11008 x 40 x 1792: 4.3 here against 5.3, 16384 x 40 x 1024: 4.1
+    // against 4.5), and more than 384 pieces on four or five (6144 x 64 x 1024: 3.9 here against 3.3)
+    return row_tiles(N) <= 2 && pieces <= 1024 && (KT >= 6 || pieces > 384);
 }
 
 template <typename Eng>
