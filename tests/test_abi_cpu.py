@@ -131,6 +131,18 @@ def test_dispatch_of_the_benchmark_configurations():
     assert kid(MODE_XOR, 1, 2560, 1536, 8192, 1, A) == B.KERNEL_MFMA_128x128     # 120: every 128 x 128 block has a unit to itself
     assert kid(MODE_XOR, 1, 6144, 2048, 16384, 1, A) == B.KERNEL_MFMA_128x128    # 384
     assert kid(MODE_XOR, 1, 6656, 2048, 16384, 1, A) == B.KERNEL_MFMA_256x128    # 416
+    assert kid(MODE_XOR, 1, 9216, 256, 4096, 1, A) == B.KERNEL_MFMA_128x128      # 144 blocks from 16 K-tiles on
+    assert kid(MODE_XOR, 1, 9216, 256, 2048, 1, A) == B.KERNEL_MFMA_32x128
+    # four to seven K-tiles: split-K in the block for up to two activation tile rows
+    assert kid(MODE_XOR, 1, 11008, 40, 1792, 1, A) == B.KERNEL_SKINNY_SPLITK
+    assert kid(MODE_XOR, 1, 1024, 384, 1024, 1, A) == B.KERNEL_MFMA_32x128
+    assert kid(MODE_XOR, 1, 6144, 64, 1024, 1, A) == B.KERNEL_MFMA_32x128        # 384 pieces on four K-tiles
+    # two bit planes: four pieces a block for one round of blocks, then the pipelined 32 x 256 and 128 x 128 tiles
+    assert kid(MODE_BWTA, 1, 8192, 128, 8192, 1, A) == B.KERNEL_SKINNY_QUAD      # 512 blocks
+    assert kid(MODE_BWTA, 1, 8192, 160, 8192, 1, A) == B.KERNEL_MFMA_32x256      # 640
+    assert kid(MODE_BWTA, 1, 11008, 96, 4096, 1, A) == B.KERNEL_MFMA_32x256      # 129 blocks of 32 x 256
+    assert kid(MODE_BWTA, 1, 11008, 256, 8192, 1, A) == B.KERNEL_MFMA_128x128    # 172 blocks of 128 x 128
+    assert kid(MODE_BWTA, 1, 11008, 320, 11008, 1, A) == B.KERNEL_MFMA_32x256    # 258: between one block a unit and one and a quarter
     assert kid(MODE_ATTN_X, 24, 64, 512, 512, 1, A) == B.KERNEL_MFMA_64x64
     assert kid(MODE_BWTA, 1, 11008, 1, 4096, 8, A) == B.KERNEL_SKINNY_POPC
     assert kid(MODE_BWTA, 1, 11008, 16, 4096, 8, A) == B.KERNEL_SKINNY_SPLITK
