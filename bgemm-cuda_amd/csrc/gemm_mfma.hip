@@ -743,7 +743,10 @@ static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int pla
     // (with its pipelined loop, from eight K-tiles on, 192 blocks are enough: 3072 x 1024 x 8192 15.3 us against 17.3 to 20.1;
     // from 16 K-tiles on 144: 6144 x 384 x 11008 16.9 against 18.9 to 22.9, 9216 x 256 x 4096 9.2 against 10.2 to 10.9,
     // 11008 x 256 x 6144 12.0 against 14.5 to 17.5; level at eight K-tiles)
-    if ((blocks(128, 128) >= 512 || (planes == 1 && KT >= 8 && blocks(128, 128) >= (KT >= 16 ? 144 : 192))) && filled(128, 128) >= 0.6)
+    // (on 16 to 23 K-tiles and fewer than 192 blocks only where the tiles are full: 9216 x 160 x 4096, 0.63 of them, 9.0 against 8.1
+    // on 32 x 128)
+    if ((blocks(128, 128) >= 512 || (planes == 1 && KT >= 8 && blocks(128, 128) >= (KT >= 16 ? 144 : 192) &&
+                                     (blocks(128, 128) >= 192 || KT >= 24 || filled(128, 128) >= 0.85))) && filled(128, 128) >= 0.6)
         return {BGEMM_KERNEL_MFMA_128x128, 128, 128};
     if (planes == 2 && two_plane_tile_128(batch, M, N, KT)) return {BGEMM_KERNEL_MFMA_128x128, 128, 128};
     // two bit planes: 32 x 256 shares every weight expansion between the planes of one row tile (W[11008,4096] x 128

@@ -818,7 +818,11 @@ static bool skinny_quad_shape(int planes, int64_t batch, int64_t M, int64_t N, i
         const int64_t blocks2 = batch * cdiv(MT, 2) * NT;
         return KT >= 24 && blocks2 >= (KT >= 40 ? 192 : 256) && blocks2 <= 512;
     }
-    if (batch * cdiv(MT, 2) * cdiv(NT, 2) < (KT >= 40 ? 192 : 256)) return false;      // (7168 x 128 x 11008, 224 blocks: 9.9 us against 11.8 on one piece a block)
+    const int64_t blocks1 = batch * cdiv(MT, 2) * cdiv(NT, 2);
+    if (blocks1 < (KT >= 40 ? 192 : 256)) return false;      // (7168 x 128 x 11008, 224 blocks: 9.9 us against 11.8 on one piece a block)
+    // one round of blocks, as for two planes (odd tile counts make more blocks of the same pieces: 12288 x 160 x 8192, 576
+    // blocks, 16.2 us against 14.7 on 128 x 128; 10240 x 160 x 8192, 480 blocks: 12.7 against 14.1)
+    if (blocks1 > 512) return false;
     return pieces <= (KT >= 24 ? 2048 : KT >= 16 ? 1024 : 0);
 }
 
