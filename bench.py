@@ -645,6 +645,25 @@ def bench_prefill(steps=20, warmup=5):
         rows.append(r)
         log(json.dumps(r))
         del w16, x16, wp, xt, out
+    # batches of decode steps: a few hundred ternary rows against one layer, weights rotating through HBM as a model's do
+    for name, M, N, K in (("Llama-7B gate / up", 11008, 128, 4096), ("Llama-7B gate+up fused", 22016, 128, 4096),
+                          ("Llama-7B down", 4096, 128, 11008), ("Llama-7B gate / up", 11008, 512, 4096)):
+        copies = max(2, min(40, int(300e6 // (M * K // 8))))
+        w16, x16 = pm1_f16((M, K), 6003, dev), ternary_f16((N, K), 6004, dev)
+        xt = lk.pack_ternary(x16)
+        wps = [lk.pack_sign(w16 if c == 0 else pm1_f16((M, K), 6100 + c, dev)) for c in range(copies)]
+        out = torch.empty((1, N, M), dtype=torch.int32, device=dev)
+        fn = lambda i: lk.bgemm_packed_forward(wps[i % copies], xt, lk.MODE_BWTA, torch.int32, 1, 0, out=out)
+        fn(0)
+        ok = check_sampled(out[0], w16, x16)
+        ms = min(time_gpu_graph(fn, copies, 2, 5) for _ in range(3))
+        r = row("BWTA %s W[%d,%d] x %d ternary rows, int32, cold weights" % (name, M, K, N), ms, 2.0 * M * N * K,
+                M * K / 8 + 2 * N * K / 8 + 4.0 * M * N, ok, kernel_of(wps[0], xt, lk.MODE_BWTA), "mfma")
+        r["roofline"] = {"bound": "mfma", "frac": round(2 * r["tops"] / FP4_MFMA_PEAK_TOPS, 4), "mfma_work": "two products a weight expansion: 4*M*N*K",
+                         "frac_of_hbm": round(r["gbs"] / HBM_PEAK_GBS, 4)}
+        rows.append(r)
+        log(json.dumps(r))
+        del w16, x16, wps, xt, out
     return rows
 
 
