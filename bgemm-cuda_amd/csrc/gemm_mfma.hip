@@ -32,8 +32,13 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
     const unsigned bid = xcd_contiguous_id(blockIdx.x, gridDim.x);
     const int per_gemm = tiles_n * tiles_m;
     const int tile_id = bid % per_gemm, b = bid / per_gemm;
-    // group tiles in bands of 8 along n so a band reuses its weight panels
-    const int band = 8;
+    // Tiles are walked in bands along n, so that the blocks in flight share their weight panels: eight tile rows, or two
+    // of the 128- and 256-row tiles on fewer than 32 K-tiles.  With two, blocks that run together write 16 KiB and more of
+    // every output row they touch instead of 4 KiB (8192^2 x 2048: 77.0 -> 68.4 us, 16384 x 8192 x 2048: 156.5 -> 140.6,
+    // 11008 x 8192 x 1024: 89.8 -> 76.4, 16384 x 8192 x 4096: 220.5 -> 205.4; two tile rows of the small tiles are up
+    // to a quarter slower).  From 32 K-tiles on the operands' reuse weighs as much: 8192^3 is 3 % faster on two with
+    // weights that rotate through HBM and 1.5 % slower with the same operands every launch.
+    const int band = WGN * WN * 32 >= 128 && a.KT < 32 ? 2 : 8;
     const int band_id = tile_id / (band * tiles_m), in_band = tile_id % (band * tiles_m);
     const int band_n0 = band_id * band;
     const int band_h = min(band, tiles_n - band_n0);
