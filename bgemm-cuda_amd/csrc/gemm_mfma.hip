@@ -37,8 +37,9 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
     // every output row they touch instead of 4 KiB (8192^2 x 2048: 77.0 -> 68.4 us, 16384 x 8192 x 2048: 156.5 -> 140.6,
     // 11008 x 8192 x 1024: 89.8 -> 76.4, 16384 x 8192 x 4096: 220.5 -> 205.4; two tile rows of the small tiles are up
     // to a quarter slower).  From 32 K-tiles on the operands' reuse weighs as much: 8192^3 is 3 % faster on two with
-    // weights that rotate through HBM and 1.5 % slower with the same operands every launch.
-    const int band = WGN * WN * 32 >= 128 && a.KT < 32 ? 2 : 8;
+    // weights that rotate through HBM and 1.5 % slower with the same operands every launch; four there (rotating
+    // weights: 8192^3 176.0 -> 171.5 us, 16384 x 4096 x 8192 173.0 -> 169.9; the same operands every launch: level).
+    const int band = WGN * WN * 32 >= 128 && a.KT < 128 ? (a.KT < 32 ? 2 : 4) : 8;
     const int band_id = tile_id / (band * tiles_m), in_band = tile_id % (band * tiles_m);
     const int band_n0 = band_id * band;
     const int band_h = min(band, tiles_n - band_n0);
