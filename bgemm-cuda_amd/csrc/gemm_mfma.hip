@@ -40,10 +40,26 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
     // weights that rotate through HBM and 1.5 % slower with the same operands every launch; four there (rotating
     // weights: 8192^3 176.0 -> 171.5 us, 16384 x 4096 x 8192 173.0 -> 169.9; the same operands every launch: level).
     const int band = WGN * WN * 32 >= 128 && a.KT < 128 ? (a.KT < 32 ? 2 : 4) : 8;
-    const int band_id = tile_id / (band * tiles_m), in_band = tile_id % (band * tiles_m);
-    const int band_n0 = band_id * band;
-    const int band_h = min(band, tiles_n - band_n0);
-    const int tn_block = band_n0 + in_band % band_h, tm = in_band / band_h;
+    int tn_block, tm;
+    const int sn = a.KT < 16 ? 4 : 2, sm = 8 / sn;
+    if (WGN * WN * 32 >= 128 && gridDim.x == (unsigned)per_gemm && tiles_n % sn == 0 && tiles_m % sm == 0) {
+        // One GEMM on the tall tiles whose tile grid splits evenly: XCD x (the hardware's block id modulo 8) takes a
+        // sub-rectangle of the grid, 1/2 x 1/4 of it (1/4 x 1/2 on a short K), and walks that in bands: its L2 then
+        // fetches a half and a quarter of the operands instead of an eighth of one and all of the other (weights
+        // rotating through HBM: 8192^3 170.3 -> 164.9 us, 16384 x 8192 x 4096 205.7 -> 197.2, 8192 x 4096 x 4096 53.5 ->
+        // 51.2, 8192^2 x 2048 67.9 -> 62.5; the same operands every launch: level).
+        const int x = blockIdx.x % 8, y = blockIdx.x / 8, sub_n = tiles_n / sn, sub_m = tiles_m / sm;
+        const int bd = y / (band * sub_m), ib = y % (band * sub_m);
+        const int n0 = bd * band, bh = min(band, sub_n - n0);
+        tn_block = (x / sm) * sub_n + n0 + ib % bh;
+        tm = (x % sm) * sub_m + ib / bh;
+    } else {
+        const int band_id = tile_id / (band * tiles_m), in_band = tile_id % (band * tiles_m);
+        const int band_n0 = band_id * band;
+        const int band_h = min(band, tiles_n - band_n0);
+        tn_block = band_n0 + in_band % band_h;
+        tm = in_band / band_h;
+    }
 
     // K is never split across blocks here: outputs of so few tiles that a K split would pay go to the kernel
     // that splits K among the waves of a block (gemm_skinny_shape)

@@ -174,6 +174,26 @@ def test_two_planes_on_the_pipelined_loop(oracle, tile, engine, KT):
         assert (bits_of(gots) == bits_of(oracle.np_scale_epilogue(want, sw, sa, None))).all()
 
 
+@pytest.mark.parametrize("K", [512, 16 * 256 + 40])
+@pytest.mark.parametrize("tile,N,M", [("128x128", 1024, 512), ("128x128", 512, 1024), ("256x128", 1024, 1024),
+                                       ("256x128", 2048, 512), ("256x256", 1024, 2048), ("128x128", 1000, 500)])
+def test_tile_grids_that_split_evenly_among_the_xcds(tile, N, M, K):
+    """One product on the tall tiles whose tile grid divides by 4 x 2 (short K) or 2 x 4: every XCD walks a sub-rectangle of
+    its own; every tile must be computed exactly once (whole output against the dense form), and the two-plane and
+    batched calls, which walk the grid the other way, on the same operands."""
+    rng = np.random.default_rng(N + M + K)
+    w, x = pm1(rng, M, K), pm1(rng, N, K)
+    wp, xp, xt = lk.pack_sign(to_dev(w)), lk.pack_sign(to_dev(x)), lk.pack_ternary(to_dev(x))
+    for mode, xo in ((MODE_XOR, xp), (MODE_AND, xp)) + (((MODE_BWTA, xt),) if tile == "128x128" else ()):
+        want = dense(mode, w, x)
+        for dt in (torch.int32, torch.half):
+            got = lk.bgemm_packed_forward(wp, xo, mode, dt, 1, force_kernel(TILES[tile]))[0].cpu().numpy()
+            assert (got.astype(np.float32) == want.astype(np.float16 if dt == torch.half else np.int32).astype(np.float32)).all(), (mode, dt)
+    wp2 = lk.PackedBits(torch.cat([wp.data, wp.data]), None, 2, M, K)
+    got2 = lk.bgemm_packed_forward(wp2, xp, MODE_XOR, torch.int32, 1, force_kernel(TILES[tile])).cpu().numpy()
+    assert (got2[0] == dense(MODE_XOR, w, x)).all() and (got2[1] == got2[0]).all()
+
+
 @pytest.mark.parametrize("engine", list(ENGINES))
 @pytest.mark.parametrize("tile", list(TILES))
 def test_each_tile_every_mode_batched(tile, engine):
