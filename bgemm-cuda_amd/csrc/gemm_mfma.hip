@@ -45,9 +45,10 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
     if (WGN * WN * 32 >= 128 && gridDim.x == (unsigned)per_gemm && tiles_n % sn == 0 && tiles_m % sm == 0) {
         // One GEMM on the tall tiles whose tile grid splits evenly: XCD x (the hardware's block id modulo 8) takes a
         // sub-rectangle of the grid, 1/2 x 1/4 of it (1/4 x 1/2 on a short K), and walks that in bands: its L2 then
-        // fetches a half and a quarter of the operands instead of an eighth of one and all of the other (weights
+        // needs a half and a quarter of the operands instead of an eighth of one and all of the other (weights
         // rotating through HBM: 8192^3 170.3 -> 164.9 us, 16384 x 8192 x 4096 205.7 -> 197.2, 8192 x 4096 x 4096 53.5 ->
-        // 51.2, 8192^2 x 2048 67.9 -> 62.5; the same operands every launch: level).
+        // 51.2, 8192^2 x 2048 67.9 -> 62.5; the same operands every launch: level, and the bytes the L2s fetch there
+        // stay what they were, 123 MiB a launch of 8192^3).
         const int x = blockIdx.x % 8, y = blockIdx.x / 8, sub_n = tiles_n / sn, sub_m = tiles_m / sm;
         const int bd = y / (band * sub_m), ib = y % (band * sub_m);
         const int n0 = bd * band, bh = min(band, sub_n - n0);
