@@ -41,7 +41,11 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
     // weights: 8192^3 176.0 -> 171.5 us, 16384 x 4096 x 8192 173.0 -> 169.9; the same operands every launch: level).
     const int band = WGN * WN * 32 >= 128 && a.KT < 128 ? (a.KT < 32 ? 2 : 4) : 8;
     int tn_block, tm;
-    const int sn = a.KT < 16 ? 4 : 2, sm = 8 / sn;
+    int sn = a.KT < 16 ? 4 : 2;
+    // (the other way round where only that divides, below 32 K-tiles: 11008 x 2048 x 4096, 16 x 86 tiles, 44.2 -> 41.5 us; on
+    // 32 K-tiles the same shape loses 3 % that way)
+    if (a.KT < 32 && (tiles_n % sn != 0 || tiles_m % (8 / sn) != 0)) sn = 8 / sn;
+    const int sm = 8 / sn;
     if (WGN * WN * 32 >= 128 && gridDim.x == (unsigned)per_gemm && tiles_n % sn == 0 && tiles_m % sm == 0) {
         // One GEMM on the tall tiles whose tile grid splits evenly: XCD x (the hardware's block id modulo 8) takes a
         // sub-rectangle of the grid, 1/2 x 1/4 of it (1/4 x 1/2 on a short K), and walks that in bands: its L2 then

@@ -176,7 +176,7 @@ def test_two_planes_on_the_pipelined_loop(oracle, tile, engine, KT):
 
 @pytest.mark.parametrize("K", [512, 16 * 256 + 40])
 @pytest.mark.parametrize("tile,N,M", [("128x128", 1024, 512), ("128x128", 512, 1024), ("256x128", 1024, 1024),
-                                       ("256x128", 2048, 512), ("256x256", 1024, 2048), ("128x128", 1000, 500)])
+                                       ("256x128", 2048, 512), ("256x256", 1024, 2048), ("128x128", 1000, 500), ("128x128", 512, 768), ("128x128", 768, 512)])
 def test_tile_grids_that_split_evenly_among_the_xcds(tile, N, M, K):
     """One product on the tall tiles whose tile grid divides by 4 x 2 (short K) or 2 x 4: every XCD walks a sub-rectangle of
     its own; every tile must be computed exactly once (whole output against the dense form), and the two-plane and
