@@ -844,10 +844,13 @@ bool gemm_skinny_shape(int planes, int64_t batch, int64_t M, int64_t N, int64_t 
     if (KT >= 8) return pieces <= (batch > 1 ? 512 : 1024);
     if (KT < 4) return false;
     if (planes == 2) return pieces <= 512 || (row_tiles(N) <= 2 && pieces <= 1024);      // (11008 x 48 ternary rows x 1792: 4.7 us here against 5.7)
-    // four to seven K-tiles, one bit plane: two tile rows of activations at most (1024 x 384 x 1024: 3.6 us here against 3.2
+    // four to seven K-tiles, one bit plane: few tile rows of activations (1024 x 384 x 1024: 3.6 us here against 3.2
     // on 32 x 128 tiles, 2048 x 192 x 1792: 4.1 against 3.7; 11008 x 40 x 1792: 4.3 here against 5.3, 16384 x 40 x 1024: 4.1
     // against 4.5), and more than 384 pieces on four or five (6144 x 64 x 1024: 3.9 here against 3.3)
-    return row_tiles(N) <= 2 && pieces <= 1024 && (KT >= 6 || pieces > 384);
+    // (up to four tile rows and 512 pieces as well: the 784 -> 4096 layer of an MLP at batch 128, sign bits out, is
+    // 1.4 us faster here than on 32 x 128 tiles)
+    if (row_tiles(N) > 2) return row_tiles(N) <= 4 && pieces <= 512;
+    return pieces <= 1024 && (KT >= 6 || pieces > 384);
 }
 
 template <typename Eng>

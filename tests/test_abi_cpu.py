@@ -136,6 +136,7 @@ def test_dispatch_of_the_benchmark_configurations():
     # four to seven K-tiles: split-K in the block for up to two activation tile rows
     assert kid(MODE_XOR, 1, 11008, 40, 1792, 1, A) == B.KERNEL_SKINNY_SPLITK
     assert kid(MODE_XOR, 1, 1024, 384, 1024, 1, A) == B.KERNEL_MFMA_32x128
+    assert kid(MODE_XOR, 1, 4096, 128, 784, 1, A) == B.KERNEL_SKINNY_SPLITK       # four tile rows, 512 pieces: an MLP's first layer
     assert kid(MODE_XOR, 1, 6144, 64, 1024, 1, A) == B.KERNEL_MFMA_32x128        # 384 pieces on four K-tiles
     # two bit planes: four pieces a block for one round of blocks, then the pipelined 32 x 256 and 128 x 128 tiles
     assert kid(MODE_BWTA, 1, 8192, 128, 8192, 1, A) == B.KERNEL_SKINNY_QUAD      # 512 blocks
