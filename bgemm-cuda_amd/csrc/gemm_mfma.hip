@@ -777,7 +777,10 @@ static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int pla
     // (on 16 to 23 K-tiles and fewer than 192 blocks only where the tiles are full: 9216 x 160 x 4096, 0.63 of them, 9.0 against 8.1
     // on 32 x 128)
     if ((blocks(128, 128) >= 512 || (planes == 1 && KT >= 8 && blocks(128, 128) >= (KT >= 16 ? 144 : 192) &&
-                                     (blocks(128, 128) >= 192 || KT >= 24 || filled(128, 128) >= 0.85))) && filled(128, 128) >= 0.6)
+                                     (blocks(128, 128) >= 192 || KT >= 24 || filled(128, 128) >= 0.85) &&
+                                     // (between one block per CU and one and two thirds on a short K the launch waits for the CUs
+                                     //  that run two: 8192 x 640 x 2048, 320 blocks, 10.4 us against 9.6 on 64 x 128; level from 16 K-tiles)
+                                     !(KT < 12 && blocks(128, 128) > 256 && blocks(128, 128) < 416))) && filled(128, 128) >= 0.6)
         return {BGEMM_KERNEL_MFMA_128x128, 128, 128};
     if (planes == 2 && two_plane_tile_128(batch, M, N, KT)) return {BGEMM_KERNEL_MFMA_128x128, 128, 128};
     // two bit planes: 32 x 256 shares every weight expansion between the planes of one row tile (W[11008,4096] x 128
