@@ -533,6 +533,15 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
         }
         return;
     }
+    // fp16 scaled, eight elements a lane: the lane's eight columns are the same for every strip, so their parameters are
+    // fetched once, before the strips (inside the strip loop the stores between them keep the compiler from reusing them)
+    ColParams cp8[8];
+    float saf8 = 0.f;
+    if (a.vec_store == 8 && a.out_kind == BGEMM_OUT_F16_SCALED) {
+        saf8 = ep_scalar(a.out_kind, a.ep_sa);
+#pragma unroll
+        for (int e = 0; e < 8; e++) cp8[e] = col_params(a, (int64_t)mt0 * 32 + (lane % (WM * 4)) * 8 + e);
+    }
 #pragma unroll
     for (int i = 0; i < WN; i++) {
         int val[WM][16];
@@ -582,30 +591,45 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
             char* dst = out_base + (nrow0 + row0) * row_bytes + (m << 1);
             const int64_t dstep = RSTEP * row_bytes;
             const bool scaled = a.out_kind == BGEMM_OUT_F16_SCALED;
-            ColParams cp[8];                     // this lane's eight columns, the same for every row of the strip
-            float saf = 0.f;
-            if (scaled) {
-                saf = ep_scalar(a.out_kind, a.ep_sa);
-#pragma unroll
-                for (int e = 0; e < 8; e++) cp[e] = col_params(a, m + e);
-            }
+            const ColParams (&cp)[8] = cp8;      // this lane's eight columns, the same for every row of every strip
+            const float saf = saf8;
             const bool has_bias = a.ep_bias != nullptr;
-            auto put8 = [&](const int4 q0, const int4 q1, char* const to, const bool sc) {
-                const int q[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
-                union { __half h[8]; uint4 u; } pk;
+            // The scaled kind's two multiplications and its addition run on fp16 pairs.  scaled_f16 spells every step out as
+            // fp32 arithmetic on fp16 values rounded back to fp16 (what torch's kernels do); with 24 >= 2 * 11 + 2 significand
+            // bits in between, that double rounding gives the correctly rounded fp16 result for a product or a sum of two fp16
+            // values, which is what the fp16 instructions return.
+            __half2 swh[4], biash[4];
+            const __half2 sah = __float2half2_rn(saf);
 #pragma unroll
-                for (int e = 0; e < 8; e++) pk.h[e] = sc ? scaled_f16(q[e], cp[e], saf, has_bias) : __float2half_rn((float)q[e]);
+            for (int e = 0; e < 4; e++) {
+                swh[e] = scaled ? __floats2half2_rn(cp[2 * e].sw, cp[2 * e + 1].sw) : sah;
+                biash[e] = scaled && has_bias ? __floats2half2_rn(cp[2 * e].bias, cp[2 * e + 1].bias) : sah;
+            }
+            auto put8 = [&](const int4 q0, const int4 q1, char* const to, const bool sc) {
+#pragma clang fp contract(off)
+                const int q[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+                union { __half h[8]; __half2 h2[4]; uint4 u; } pk;
+#pragma unroll
+                for (int e = 0; e < 8; e++) pk.h[e] = __float2half_rn((float)q[e]);
+                if (sc) {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) pk.h2[e] = __hmul2(__hmul2(pk.h2[e], swh[e]), sah);
+                    if (has_bias) {
+#pragma unroll
+                        for (int e = 0; e < 4; e++) pk.h2[e] = __hadd2(pk.h2[e], biash[e]);
+                    }
+                }
                 store16(to, make_int4((int)pk.u.x, (int)pk.u.y, (int)pk.u.z, (int)pk.u.w), true);
             };
             if (m < a.M) {
-                if (nrow0 + 32 <= a.N && !scaled) {  // uniform: whole strip, plain conversion: reads issued in pairs of rows
+                if (nrow0 + 32 <= a.N) {             // uniform: whole strip: reads issued in pairs of rows
 #pragma unroll
                     for (int r = 0; r < 32 / RSTEP; r += 2, dst += 2 * dstep) {
                         const int* s0 = sp + r * RSTEP * ROW_I, * s1 = s0 + RSTEP * ROW_I;
                         const int4 a0 = *reinterpret_cast<const int4*>(s0), a1 = *reinterpret_cast<const int4*>(s0 + 4);
                         const int4 b0 = *reinterpret_cast<const int4*>(s1), b1 = *reinterpret_cast<const int4*>(s1 + 4);
-                        put8(a0, a1, dst, false);
-                        put8(b0, b1, dst + dstep, false);
+                        put8(a0, a1, dst, scaled);
+                        put8(b0, b1, dst + dstep, scaled);
                     }
                 } else {
 #pragma unroll 2
