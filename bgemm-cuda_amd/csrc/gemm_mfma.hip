@@ -542,6 +542,13 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
 #pragma unroll
         for (int e = 0; e < 8; e++) cp8[e] = col_params(a, (int64_t)mt0 * 32 + (lane % (WM * 4)) * 8 + e);
     }
+    // (the same for the scaled kinds stored four elements a lane: fp32, and fp16 rows that are no multiple of eight long)
+    ColParams cp4[4];
+    if (a.vec_store && a.vec_store != 8 && (a.out_kind == BGEMM_OUT_F32_SCALED || a.out_kind == BGEMM_OUT_F16_SCALED)) {
+        saf8 = ep_scalar(a.out_kind, a.ep_sa);
+#pragma unroll
+        for (int e = 0; e < 4; e++) cp4[e] = col_params(a, (int64_t)mt0 * 32 + (lane % (WM * 8)) * 4 + e);
+    }
 #pragma unroll
     for (int i = 0; i < WN; i++) {
         int val[WM][16];
@@ -647,13 +654,8 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
             const int64_t dstep = RSTEP * row_bytes;
             const bool scaled = a.out_kind == BGEMM_OUT_F32_SCALED || a.out_kind == BGEMM_OUT_F16_SCALED;
             const bool has_bias = a.ep_bias != nullptr;
-            ColParams cp[4];
-            float saf = 0.f;
-            if (scaled) {
-                saf = ep_scalar(a.out_kind, a.ep_sa);
-#pragma unroll
-                for (int e = 0; e < 4; e++) cp[e] = col_params(a, m + e);
-            }
+            const ColParams (&cp)[4] = cp4;
+            const float saf = saf8;
             if (m < a.M) {
 #pragma unroll 2
                 for (int row = row0; row < 32 && nrow0 + row < a.N; row += RSTEP, sp += RSTEP * ROW_I, dst += dstep) {
