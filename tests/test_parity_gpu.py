@@ -795,3 +795,29 @@ def test_bits_output_chains_two_layers_and_empty_k(oracle):
                                  next_zero_point=torch.full((1,), 0.25, device=DEV))
     wantb = oracle.c_pack_sign(np.tile((bias.cpu().numpy() - np.float32(0.25)).astype(np.float16), (9, 1)))
     assert (lk.logical_from_tiled(ob).cpu().numpy().view(np.uint32) == wantb).all()
+
+
+@pytest.mark.parametrize("M,N,K", [(1024, 512, 1024), (520, 300, 2304), (1032, 96, 8192)])
+def test_scaled_fp16_matches_torchs_fp16_kernels_from_denormal_to_overflow(M, N, K):
+    """The fp16 scaled kind against torch's own fp16 elementwise kernels on the int32 result (what the layers of
+    tests/python/bgemm_linear.py compute after the kernel, one rounded operation at a time): per-row scales from the
+    denormal range to overflow, both signs, activation scales, with and without a bias; bit for bit, NaN for NaN."""
+    g = torch.Generator(device=DEV).manual_seed(M + N + K)
+    rng = np.random.default_rng(M + N + K)
+    w, x = rand_f16(rng, M, K), rand_f16(rng, N, K)
+    wp, xp = lk.pack_sign(to_dev(w)), lk.pack_sign(to_dev(x))
+    acc = lk.bgemm_packed_forward(wp, xp, MODE_XOR, torch.int32, 1)[0]
+    for lo, hi in ((-24, -14), (-14, -6), (-6, 0), (0, 6), (-24, 6)):
+        e = torch.randint(lo, hi + 1, (M,), generator=g, device=DEV).float()
+        sign = torch.where(torch.rand(M, generator=g, device=DEV) < 0.5, -1.0, 1.0).half()
+        sw = (torch.exp2(e) * (1 + torch.rand(M, generator=g, device=DEV))).half() * sign
+        for sa_v in (0.7371, 3.1e-3, 61.0):
+            sa = torch.tensor([sa_v], device=DEV).half()
+            be = torch.randint(-20, 12, (M,), generator=g, device=DEV).float()
+            for bias in (None, (torch.randn(M, generator=g, device=DEV) * torch.exp2(be)).half()):
+                got = lk.bgemm_packed_forward(wp, xp, MODE_XOR, scale=(sw, sa, bias))[0]
+                want = acc.half() * sw * sa
+                if bias is not None:
+                    want = want + bias
+                same = (got.view(torch.int16) == want.view(torch.int16)) | (got.isnan() & want.isnan())
+                assert bool(same.all()), (lo, hi, sa_v, bias is not None, int((~same).sum()))
