@@ -270,15 +270,6 @@ __device__ __forceinline__ void store_out_as(const GemmArgs& a, const int64_t ro
     else if constexpr (KIND == BGEMM_OUT_F32_SCALED) reinterpret_cast<float*>(a.out)[row0 + m] = scaled_f32(a, m, v);
     else reinterpret_cast<__half*>(a.out)[row0 + m] = scaled_f16(a, m, v);
 }
-// The same with the column's parameters in registers (a thread that keeps its column fetches them once, early).
-template <int KIND>
-__device__ __forceinline__ void store_out_as(const GemmArgs& a, const int64_t row0, const int64_t m, const int v, const ColParams c,
-                                             const float sa, const bool has_bias)
-{
-    if constexpr (KIND == BGEMM_OUT_F32_SCALED) reinterpret_cast<float*>(a.out)[row0 + m] = scaled_f32(v, c, sa, has_bias);
-    else if constexpr (KIND == BGEMM_OUT_F16_SCALED) reinterpret_cast<__half*>(a.out)[row0 + m] = scaled_f16(v, c, sa, has_bias);
-    else store_out_as<KIND>(a, row0, m, v);
-}
 __device__ __forceinline__ void store_out(const GemmArgs& a, const int64_t row0, const int64_t m, const int v)
 {
     switch (a.out_kind) {

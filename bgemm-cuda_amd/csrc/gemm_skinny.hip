@@ -664,15 +664,6 @@ __global__ __launch_bounds__(KW * 64, 2) void gemm_skinny_splitk_quad_kernel(con
 #pragma unroll
     for (int v = 0; v < 16; v++) acc[0][0][v] = acc[0][1][v] = acc[1][0][v] = acc[1][1][v] = 0;
     int pa[2] = {0, 0}, pb[2] = {0, 0};
-    // scaled kinds: the parameters of the column this thread stores (one of the piece's 64) are requested here, so that
-    // they arrive during the walk over K instead of in front of every store
-    const bool scaled_kind = a.out_kind == BGEMM_OUT_F32_SCALED || a.out_kind == BGEMM_OUT_F16_SCALED;
-    ColParams colp = {0.f, 0.f};
-    float saf = 0.f;
-    if (scaled_kind) {
-        colp = col_params(a, (int64_t)rt0 * 32 + (threadIdx.x & 63));
-        saf = ep_scalar(a.out_kind, a.ep_sa);
-    }
 
     uint4 wA[CH][2], xA[CH][2], wB[CH][2], xB[CH][2], wC[CH][2], xC[CH][2];
     // Every fetch issues all of its loads, a K-tile past the range as the range's last one again (a cache hit,
@@ -777,10 +768,9 @@ __global__ __launch_bounds__(KW * 64, 2) void gemm_skinny_splitk_quad_kernel(con
     };
     const int64_t out0 = (int64_t)b * a.strideC;
     const int M = (int)a.M;
-    const bool has_bias = a.ep_bias != nullptr;
     auto elements = [&](auto kind) {
         outputs([&](const int n, const int m, const int, const int val) {
-            if (m < M) store_out_as<decltype(kind)::value>(a, out0 + (int64_t)n * M, m, val, colp, saf, has_bias);
+            if (m < M) store_out_as<decltype(kind)::value>(a, out0 + (int64_t)n * M, m, val);
         });
     };
     switch (a.out_kind) {
