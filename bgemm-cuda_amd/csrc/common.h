@@ -178,15 +178,16 @@ __device__ __forceinline__ float scaled_f32(const GemmArgs& a, const int64_t m, 
 __device__ __forceinline__ __half scaled_f16(const GemmArgs& a, const int64_t m, const int v)
 {
 #pragma clang fp contract(off)      // every step rounds by itself, as torch's separate kernels do
-    __half r = __float2half_rn((float)v);
-    r = __float2half_rn((__half2float(r) * __half2float(reinterpret_cast<const __half*>(a.ep_sw)[m])));
-    r = __float2half_rn((__half2float(r) * __half2float(*reinterpret_cast<const __half*>(a.ep_sa))));
-    if (a.ep_bias) r = __float2half_rn((__half2float(r) + __half2float(reinterpret_cast<const __half*>(a.ep_bias)[m])));
-    return r;
+    // fp16 instructions: correctly rounded, hence equal to torch's fp32 operation rounded back to fp16
+    _Float16 r = (_Float16)(float)v;
+    r = r * reinterpret_cast<const _Float16*>(a.ep_sw)[m];
+    r = r * *reinterpret_cast<const _Float16*>(a.ep_sa);
+    if (a.ep_bias) r = r + reinterpret_cast<const _Float16*>(a.ep_bias)[m];
+    __half_raw h; h.data = r;
+    return __half(h);
 }
 // The same with the column's parameters already in registers (a store loop walks rows of fixed columns:
-// the parameters are fetched once per column, not once per element).  fp16 parameters widened to fp32
-// are the values the functions above compute with, so the results are identical.
+// the parameters are fetched once per column, not once per element), fp16 parameters widened to fp32.
 struct ColParams { float sw, bias; };
 __device__ __forceinline__ bool f32_params(const int kind) { return kind == BGEMM_OUT_F32_SCALED || kind == BGEMM_OUT_BITS_F32; }
 __device__ __forceinline__ float ep_scalar(const int kind, const void* p)
@@ -215,14 +216,22 @@ __device__ __forceinline__ float scaled_f32(const int v, const ColParams c, cons
     if (has_bias) r = (r + c.bias);
     return r;
 }
+// fp16 parameters: every step is one fp16 instruction (v_mul_f16 / v_add_f16), whose result is the correctly rounded
+// fp16 value, i.e. what torch's kernels get from an fp32 operation on fp16 values rounded back to fp16 (24 >= 2 * 11 + 2
+// significand bits in between).  The steps must not be written as fp32 arithmetic on the widened parameters: the
+// compiler turns `half(float(r) * sw)` with an fp32 `sw` into `v_fma_mixlo_f16 r, sw, 0`, and the +0 it adds makes a
+// zero accumulator times a negative scale +0 where the multiplication gives -0 (one output in 80 at K = 1024).
+// c.sw, c.bias and sa were widened from fp16, so narrowing them again is exact; the narrowing does not depend on the
+// element and leaves a store loop.
 __device__ __forceinline__ __half scaled_f16(const int v, const ColParams c, const float sa, const bool has_bias)
 {
 #pragma clang fp contract(off)      // every step rounds by itself, as torch's separate kernels do
-    __half r = __float2half_rn((float)v);
-    r = __float2half_rn((__half2float(r) * c.sw));
-    r = __float2half_rn((__half2float(r) * sa));
-    if (has_bias) r = __float2half_rn((__half2float(r) + c.bias));
-    return r;
+    _Float16 r = (_Float16)(float)v;
+    r = r * (_Float16)c.sw;
+    r = r * (_Float16)sa;
+    if (has_bias) r = r + (_Float16)c.bias;
+    __half_raw h; h.data = r;
+    return __half(h);
 }
 // sign bit of half_rn(y - zp) for the bits kinds, y as above
 __device__ __forceinline__ unsigned next_sign_bit(const int kind, const int v, const ColParams c, const float sa,

@@ -363,6 +363,7 @@ def bgemm_packed_forward(w, x, mode=MODE_XOR, out_dtype=torch.int32, splitK=1, v
                                                  bias.data_ptr() if bias is not None else None,
                                                  next_zero_point.data_ptr() if next_zero_point is not None else None,
                                                  _stream()))
+            bits_out.counts = None       # row popcounts taken of the old contents no longer describe it
             return bits_out
         else:
             _b.check(L.bgemm_packed_forward_scaled(*args, sw.data_ptr(), sa.data_ptr(),

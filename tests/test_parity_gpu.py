@@ -798,7 +798,7 @@ def test_bits_output_chains_two_layers_and_empty_k(oracle):
 
 
 @pytest.mark.parametrize("M,N,K", [(1024, 512, 1024), (520, 300, 2304), (1032, 96, 8192), (4096, 256, 6144),      # the last: four pieces a block
-                                   (1027, 512, 1024)])                         # rows stored one element at a time
+                                   (1028, 512, 1024), (1027, 512, 1024)])     # rows stored four elements and one element at a time
 def test_scaled_fp16_matches_torchs_fp16_kernels_from_denormal_to_overflow(M, N, K):
     """The fp16 scaled kind against torch's own fp16 elementwise kernels on the int32 result (what the layers of
     tests/python/bgemm_linear.py compute after the kernel, one rounded operation at a time): per-row scales from the

@@ -436,3 +436,49 @@ def test_k_just_under_2_to_24_every_term_at_its_maximum(kernel):
         if two_planes:
             assert run(w1, tern(x1), MODE_BWTA) == K and run(w0, tern(x1), MODE_BWTA) == -K
             assert run(w1, tern(xh), MODE_BWTA) == pb
+
+
+KERNELS_FOR_SCALES = dict({"mfma " + t: (TILES[t], 96) for t in TILES},
+                          **{"split-K in the block": (B.KERNEL_SKINNY_SPLITK, 96), "four pieces": (B.KERNEL_SKINNY_QUAD, 96),
+                             "stream": (B.KERNEL_SKINNY_STREAM, 20), "popcount": (B.KERNEL_SKINNY_POPC, 2), "valu": (None, 96)})
+
+
+@pytest.mark.parametrize("M", [1024, 1028, 1027])      # eight, four and one element(s) a lane in the general kernel's store
+@pytest.mark.parametrize("kernel", list(KERNELS_FOR_SCALES))
+def test_scaled_and_bits_kinds_with_per_row_scales_from_denormal_to_overflow(oracle, kernel, M):
+    """`half(acc) * sw * sa (+ bias)` (tests/python/bgemm_linear.py:482-484) and the sign bits of its centred fp16 value
+    (the next layer's `(x - zpa).to(torch.half)`, :479-482) with per-row scales from fp16's denormal range (a layer of
+    M >= 13 000 output rows has sw = |W|_1 / numel there) to overflow: every kernel family, every scaled and bits kind,
+    against the oracle's step-by-step rounding, bit for bit (NaN for NaN)."""
+    kid, N = KERNELS_FOR_SCALES[kernel]
+    K = 1024
+    rng = np.random.default_rng(M * 7 + N)
+    w, x = pm1(rng, M, K), pm1(rng, N, K)
+    wp, xp = lk.pack_sign(to_dev(w)), lk.pack_sign(to_dev(x))
+    variant = VARIANT_VALU if kid is None else force_kernel(kid, VARIANT_MFMA_F4)
+    acc = dense(MODE_XOR, w, x)
+    for lo, hi in ((-24, -14), (-24, 6)):
+        for dtype in (np.float16, np.float32):
+            with np.errstate(over="ignore"):
+                sw = (np.exp2(rng.integers(lo, hi + 1, M)) * (1 + rng.random(M)) * rng.choice([-1.0, 1.0], M)).astype(dtype)
+                bias = (rng.standard_normal(M) * np.exp2(rng.integers(-24, 4, M))).astype(dtype)
+            for sa_v in (0.7371, 61.0):
+                sa = np.asarray(sa_v, dtype=dtype)
+                for b in (None, bias):
+                    sc = (to_dev(sw), to_dev(sa.reshape(1)), None if b is None else to_dev(b))
+                    y = oracle.np_scale_epilogue(acc, sw, sa, b)
+                    got = lk.bgemm_packed_forward(wp, xp, MODE_XOR, variant=variant, scale=sc)[0].cpu().numpy()
+                    same = (bits_of(got) == bits_of(y)) | (np.isnan(got) & np.isnan(y))
+                    assert got.dtype == y.dtype and same.all(), ("scaled", lo, hi, dtype, sa_v, b is not None, int((~same).sum()))
+                    # the bits kinds: zero points a few fp16 denormal steps either side of zero, and none
+                    for zp_steps in (None, 0, 3, -2, 40):
+                        zp = None if zp_steps is None else np.asarray(zp_steps * 2.0 ** -24, dtype=dtype)
+                        out = lk.bgemm_packed_forward(wp, xp, MODE_XOR, variant=variant, bits_out=lk.zeros_packed(N, M, 1, DEV),
+                                                      scale=sc, next_zero_point=None if zp is None else to_dev(zp.reshape(1)))
+                        with np.errstate(invalid="ignore", over="ignore"):
+                            c = oracle.np_center_to_f16(y, dtype(0) if zp is None else zp)
+                        want_bits = c.view(np.uint16) >> 15
+                        logical = lk.logical_from_tiled(out).cpu().numpy().view(np.uint32)
+                        got_bits = np.unpackbits(logical.byteswap().view(np.uint8), axis=1)[:, :M]
+                        ok = (got_bits == want_bits) | np.isnan(c)          # the sign of a NaN (inf - inf) is not defined
+                        assert ok.all(), ("bits", lo, hi, dtype, sa_v, b is not None, zp_steps, int((~ok).sum()))
