@@ -6,7 +6,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 SO = os.path.join(HERE, "libbgemm_mi355x.so")
-SOURCES = ["api.hip", "pack.hip", "gemm_mfma.hip", "gemm_valu.hip", "gemm_skinny.hip"]
+SOURCES = ["api.hip", "pack.hip", "gemm_mfma.hip", "gemm_valu.hip", "gemm_skinny.hip", "gemm_chain.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
          # keep the compiler from forming packed-fp32 VALU ops
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]

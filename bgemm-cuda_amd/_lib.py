@@ -9,11 +9,11 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 SO_PATH = os.path.join(_HERE, "libbgemm_mi355x.so")
 
-OK, EINVAL, ENULL, EWORKSPACE, ELAUNCH, EALIGN = 0, -1, -2, -3, -4, -5
+OK, EINVAL, ENULL, EWORKSPACE, ELAUNCH, EALIGN, ETIMEOUT = 0, -1, -2, -3, -4, -5, -6
 MODE_AND, MODE_XOR, MODE_ATTN, MODE_BWTA, MODE_ATTN_X = 0, 1, 2, 3, 4
 OUT_I32, OUT_F16, OUT_F32_SCALED, OUT_F16_SCALED, OUT_BITS_F32, OUT_BITS_F16 = 0, 1, 2, 3, 4, 5
 SRC_F16, SRC_F32 = 0, 1
-ABI_VERSION = 9
+ABI_VERSION = 10
 LAYOUT_VERSION = 6     # of the tiled operand layout, written into packed files; changes only when the layout does
 STATIC_SCRATCH_BYTES = 32 << 20      # BGEMM_STATIC_SCRATCH_BYTES
 VARIANT_AUTO, VARIANT_VALU, VARIANT_MFMA, VARIANT_MFMA_F4 = 0, 1, 2, 3
@@ -61,7 +61,16 @@ SIGNATURES = {
     "bgemm_f16_workspace_bytes": (_sz, [_i64, _i64, _i64, _int]),
     "bgemm_f16_forward": (_int, [_p, _p, _p, _i64, _i64, _i64, _p, _sz, _int, _int, _p]),
     "bgemm_f16_forward_static": (_int, [_p, _p, _p, _i64, _i64, _i64, _int, _int, _p]),
+    "bgemm_chain_workspace_bytes": (_sz, [_int, _p, _int, _i64]),
+    "bgemm_chain_forward": (_int, [_int, _p, _p, _int, _p, _p, _i64, _p, _int, _int, _p, _sz, _int, _p]),
+    "bgemm_chain_status": (_int, [_p, _p]),
 }
+
+
+class ChainLayer(ctypes.Structure):
+    """bgemm_chain_layer: one layer of a chain; every pointer is a device pointer."""
+    _fields_ = [("W_tiled", _p), ("sw", _p), ("bias", _p), ("sa", _p), ("next_zero_point", _p),
+                ("M", _i64), ("K", _i64), ("reserved", _i64)]
 
 _lib = None
 

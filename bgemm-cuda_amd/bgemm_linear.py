@@ -278,7 +278,8 @@ class BGEMMLinear(_ScaledBinaryLinear):
     """out = bgemm(x - zpa, w - zpw) * sw * sa (+ bias)  (bgemm_linear.py:460-486).
 
     Under ``torch.no_grad()`` the forward is fused (``fuse_inference``) and multiplies with a cached packed copy of
-    the weight.  The cache follows every update made through the parameter (optimizer steps, ``copy_``, ``+=``) and is
+    the weight.  The cache follows every update made through the parameter or the weight's zero point ``zpw``
+    (optimizer steps, ``copy_``, ``+=``) and is
     dropped by ``train()`` / ``eval()`` and ``load_state_dict``; after a write through ``weight.data`` call
     ``invalidate_packed_weight()``."""
     _fn = bgemm_linear
@@ -290,8 +291,14 @@ class BGEMMLinear(_ScaledBinaryLinear):
                 and x.dtype == dt and self.sw.dtype == dt and self.sa.dtype == dt
                 and (self.bias is None or self.bias.dtype == dt))
 
+    def _weight_key(self):
+        # the packed bits are those of (weight - zpw): an in-place update of the zero point alone (a calibration pass,
+        # an optimizer group of its own) must pack again as well
+        return (self.weight._version, self.weight.data_ptr(), self.weight.dtype, id(self.zpw), self.zpw._version,
+                self.zpw.data_ptr())
+
     def _packed_weight(self):
-        key = (self.weight._version, self.weight.data_ptr(), self.weight.dtype)
+        key = self._weight_key()
         if getattr(self, "_wp_key", None) != key:
             self._wp = lowbit_kernel.pack_sign(self.weight.detach(), zero_point=self.zpw)
             self._wp_key = key
@@ -302,7 +309,7 @@ class BGEMMLinear(_ScaledBinaryLinear):
         inference path; it is used until the float weight changes."""
         if (packed.rows, packed.K) != tuple(self.weight.shape):
             raise ValueError(f"packed weight is {packed.rows}x{packed.K} bits, the layer is {tuple(self.weight.shape)}")
-        self._wp, self._wp_key = packed, (self.weight._version, self.weight.data_ptr(), self.weight.dtype)
+        self._wp, self._wp_key = packed, self._weight_key()
 
     def _inference_state(self):
         """Detached views of the parameters for the inference path, rebuilt only when a parameter is replaced or

@@ -71,7 +71,7 @@ __global__ void clear_counters_kernel(uint32_t* c, int64_t n)
 using namespace bgemm;
 
 extern "C" const char* bgemm_last_error(void) { return g_err; }
-extern "C" int bgemm_abi_version(void) { return 9; }
+extern "C" int bgemm_abi_version(void) { return 10; }
 
 static bool ws_query(int mode, int64_t batch, int64_t M, int64_t N, int64_t K, int splitK, int variant,
                      size_t* part, size_t* counters)

@@ -63,6 +63,14 @@ __device__ __forceinline__ int dot_terms2(const ModeCoef& mc, const int d, const
     return (int)__umul24((unsigned)mc.cd2, (unsigned)d2) - (int)__umul24((unsigned)-mc.cd, (unsigned)d);
 }
 
+// Output of one (activation row, weight row) pair from the AND-dots d (and d2 of the second plane).
+__device__ __forceinline__ int skinny_value(const ModeCoef& mc, const bool two, const int kbits, const int pa,
+                                            const int pb, const int pb2, const int d, const int d2)
+{
+    const int val = mc.c0 * kbits + mc.ca * pa + mc.cb * pb;
+    return two ? val + mc.cb2 * pb2 + dot_terms2(mc, d, d2) : val + dot_term(mc, d);
+}
+
 struct GemmArgs {
     const uint4* W; const uint4* X; const uint4* X2;
     void* out; int out_kind;       // BGEMM_OUT_*

@@ -42,14 +42,6 @@ __device__ __forceinline__ const uint4* skinny_x_ptr(const GemmArgs& a, const in
     return (r >= 16 ? a.X2 : a.X) + (h * 32 + half * 16 + (r & 15)) + (int64_t)b * a.strideX;
 }
 
-// Output of one (activation row, weight row) pair from the AND-dots d (and d2 of the second plane).
-__device__ __forceinline__ int skinny_value(const ModeCoef& mc, const bool two, const int kbits, const int pa,
-                                            const int pb, const int pb2, const int d, const int d2)
-{
-    const int val = mc.c0 * kbits + mc.ca * pa + mc.cb * pb;
-    return two ? val + mc.cb2 * pb2 + dot_terms2(mc, d, d2) : val + dot_term(mc, d);
-}
-
 // ---- streaming kernel --------------------------------------------------------------------------
 template <typename Eng, int RT>
 __global__ __launch_bounds__(256, 2) void gemm_skinny_stream_kernel(const GemmArgs a, const int groups)

@@ -24,7 +24,7 @@ AND_POP, XOR_POP, ATTN_MM = 0, 1, 2   # lowbit_kernel/csrc/include/configs.h:70-
 
 __all__ = ["bgemm_linear_forward_cuda", "binary_weight_prepacking", "pack_sign", "pack_ternary",
            "pack_sign_transposed", "bgemm_packed_forward", "bgemm_packed_weight_forward", "PackedBits", "zeros_packed", "save_packed", "load_packed",
-           "set_weight_cache", "packed_kernel_id", "AND_POP", "XOR_POP", "ATTN_MM"]
+           "set_weight_cache", "packed_kernel_id", "DecodeChain", "AND_POP", "XOR_POP", "ATTN_MM"]
 
 
 _NULL_CTX = contextlib.nullcontext()
@@ -369,6 +369,94 @@ def bgemm_packed_forward(w, x, mode=MODE_XOR, out_dtype=torch.int32, splitK=1, v
             _b.check(L.bgemm_packed_forward_scaled(*args, sw.data_ptr(), sa.data_ptr(),
                                                    bias.data_ptr() if bias is not None else None, _stream()))
     return out
+
+
+class DecodeChain:
+    """A stack of dependent decode-shaped binary layers run as ONE launch (``bgemm_chain_forward``).
+
+    ``layers`` is a list of ``(w, sw, sa, bias, next_zero_point)``: ``w`` a binary PackedBits of M x K bits (batch 1),
+    ``sw`` [M], ``sa`` one element, ``bias`` [M] or None, ``next_zero_point`` one element or None, all of one dtype
+    (fp16 or fp32).  Layer l + 1 reads the bits of ``half(y_l - next_zero_point_l)``, ``y_l = half(acc_l) * sw * sa (+ bias)``
+    (tests/python/bgemm_linear.py:479-484): sign bits, or with ``mode=MODE_BWTA`` the ternary planes of its sign
+    (:222-241).  ``__call__(x)`` takes the first layer's packed operand (up to 32 rows, 16 with BWTA) and returns the
+    last layer's output: ``out_dtype`` torch.int32, torch.half (the rounded integer) or None for the scaled value
+    of the parameters' type.  Calls on one GPU must not overlap in time (each holds every compute unit)."""
+
+    def __init__(self, layers, mode=MODE_XOR, out_dtype=None, flags=0):
+        if not layers:
+            raise ValueError("a chain has at least one layer")
+        self.mode, self.flags, self.layers = mode, flags, list(layers)
+        w0, sw0 = layers[0][0], layers[0][1]
+        self.device, self.pdtype = w0.data.device, sw0.dtype
+        if self.pdtype not in (torch.float32, torch.half):
+            raise TypeError("scales must be fp32 or fp16")
+        self.out_dtype = self.pdtype if out_dtype is None else out_dtype
+        if self.out_dtype not in (torch.int32, torch.half, torch.float32):
+            raise ValueError("out_dtype must be torch.int32, torch.half or None (the parameters' type)")
+        if out_dtype is None:
+            self.kind = OUT_F32_SCALED if self.pdtype == torch.float32 else OUT_F16_SCALED
+        elif out_dtype == torch.int32:
+            self.kind = OUT_I32
+        elif out_dtype == torch.half:
+            self.kind = OUT_F16
+        else:
+            raise ValueError("a plain output is torch.int32 or torch.half")
+        arr = (_b.ChainLayer * len(layers))()
+        self._keep = []
+        for l, (w, sw, sa, bias, zp) in enumerate(layers):
+            if w.ternary or w.batch != 1:
+                raise ValueError("layer %d: the weight side is one binary matrix" % l)
+            _check_packed(w, "layer %d weights" % l)
+            for name, t, n in (("sw", sw, w.rows), ("sa", sa, 1), ("bias", bias, w.rows), ("next_zero_point", zp, 1)):
+                if t is None and name in ("bias", "next_zero_point"):
+                    continue
+                _need_cuda(t, name)
+                if t.dtype != self.pdtype or t.numel() != n or not t.is_contiguous() or t.device != self.device:
+                    raise ValueError("layer %d: %s must be a contiguous %s tensor of %d elements on %s" % (l, name, self.pdtype, n, self.device))
+            arr[l].W_tiled, arr[l].sw, arr[l].sa = w.data.data_ptr(), sw.data_ptr(), sa.data_ptr()
+            arr[l].bias = bias.data_ptr() if bias is not None else None
+            arr[l].next_zero_point = zp.data_ptr() if zp is not None else None
+            arr[l].M, arr[l].K = w.rows, w.K
+            self._keep.append((w, sw, sa, bias, zp))
+        self._host = arr
+        raw = torch.frombuffer(bytearray(bytes(arr)), dtype=torch.uint8)
+        self._dev = raw.to(self.device)
+        self._ws = {}
+
+    def workspace(self, N):
+        """The chain's workspace for N activation rows: zero-filled once, then left to the library."""
+        ws = self._ws.get(N)
+        if ws is None:
+            need = _b.lib().bgemm_chain_workspace_bytes(self.mode, self._host, len(self.layers), N)
+            if need == 0:
+                _b.check(_b.EINVAL if not _b.lib().bgemm_last_error() else _b.EINVAL)
+            ws = torch.zeros(need, dtype=torch.uint8, device=self.device)
+            self._ws[N] = ws
+        return ws
+
+    def __call__(self, x, out=None):
+        if (self.mode == MODE_BWTA) != x.ternary:
+            raise ValueError("MODE_BWTA needs a ternary activation operand, the other modes a binary one")
+        if x.batch != 1 or x.K != self.layers[0][0].K:
+            raise ValueError("the operand must be one matrix of K = %d bits a row" % self.layers[0][0].K)
+        _check_packed(x, "x")
+        N, M = x.rows, self.layers[-1][0].rows
+        ws = self.workspace(N)
+        if out is None:
+            out = torch.empty((N, M), dtype=self.out_dtype, device=self.device)
+        elif out.dtype != self.out_dtype or out.numel() != N * M or not out.is_contiguous() or out.device != self.device:
+            raise ValueError("out must be a contiguous %s tensor of %d x %d elements" % (self.out_dtype, N, M))
+        with _on(self.device):
+            _b.check(_b.lib().bgemm_chain_forward(self.mode, self._host, self._dev.data_ptr(), len(self.layers), x.data.data_ptr(),
+                                                  x.data2.data_ptr() if x.ternary else None, N, out.data_ptr(), self.kind,
+                                                  SRC_F32 if self.pdtype == torch.float32 else SRC_F16, ws.data_ptr(), ws.numel(),
+                                                  self.flags, _stream()))
+        return out
+
+    def check(self, N):
+        """Waits for the stream and raises if a launch of this chain gave up waiting (BGEMM_ETIMEOUT)."""
+        with _on(self.device):
+            _b.check(_b.lib().bgemm_chain_status(self.workspace(N).data_ptr(), _stream()))
 
 
 # Opt-in cache of packed weights for the drop-in call.  The reference's interface takes fp16 weights

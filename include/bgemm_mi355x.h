@@ -71,7 +71,8 @@ enum {
     BGEMM_ENULL = -2,       /* a required pointer is NULL                            */
     BGEMM_EWORKSPACE = -3,  /* workspace missing or smaller than *_workspace_bytes() */
     BGEMM_ELAUNCH = -4,     /* HIP reported an error at launch                       */
-    BGEMM_EALIGN = -5       /* a pointer is not 16-byte aligned                      */
+    BGEMM_EALIGN = -5,      /* a pointer is not 16-byte aligned                      */
+    BGEMM_ETIMEOUT = -6     /* a chain launch gave up waiting (bgemm_chain_status)   */
 };
 
 /* Message for the last error returned on the calling thread ("" if none). */
@@ -271,6 +272,45 @@ int bgemm_f16_forward(const void* W, const void* X, void* C, int64_t M, int64_t 
 #define BGEMM_STATIC_SCRATCH_BYTES (32u << 20)
 int bgemm_f16_forward_static(const void* W, const void* X, void* C, int64_t M, int64_t N, int64_t K,
                              int splitK, int INSTR, void* stream);
+
+/* ---- a chain of dependent decode-shaped layers in one launch ------------------------------------
+ * Layer l computes acc = MODE(W_l [M_l][K_l], x_l [N][K_l]) and hands layer l + 1 the bits of
+ * half_rn(y - *next_zero_point), y = half(acc) * sw * sa (+ bias) evaluated as in bgemm_packed_forward_scaled
+ * (tests/python/bgemm_linear.py:479-484: one BGEMMLinear feeding the next): sign bits for the modes of one
+ * plane, (nonzero, sign & nonzero) planes for BGEMM_MODE_BWTA (ternary = torch.sign, :222-241).  K_{l+1} = M_l.
+ * The last layer writes `out` [N][M_last] as out_dtype I32, F16 or a scaled kind.  The reference runs such a
+ * stack as one kernel launch (plus elementwise kernels) per layer and cannot run N < 32 at all
+ * (fp6_linear.cu:288-290); here one block per compute unit stays resident, requests a layer's weights
+ * while the layer before it is computed, and the layers exchange nothing but tagged bits.
+ *   layers      : HOST array of n_layers entries; every pointer in it is a DEVICE pointer of param_dtype
+ *                 (BGEMM_SRC_F16 / BGEMM_SRC_F32) elements: sw [M], bias [M] or NULL, sa one scalar,
+ *                 next_zero_point one scalar or NULL (0; unused in the last layer)
+ *   layers_dev  : the same array copied to the device by the caller (n_layers * 64 bytes)
+ *   X_tiled     : the first layer's operand (X2_tiled: its sign & nonzero plane for BWTA), N rows:
+ *                 N <= 32, with BWTA N <= 16
+ *   ws          : bgemm_chain_workspace_bytes() bytes, ZERO-FILLED ONCE before its first use and then left
+ *                 to the library; calls that share a workspace, or run on one GPU at the same time, must not
+ *                 overlap (each holds every compute unit until its last layer is done)
+ *   flags       : 0, or 1 / 2 to insist on the one-level / two-level exchange; bits 8.. = number of blocks
+ *                 (tests; 0 = one per compute unit)
+ * Layers of up to 3 row tiles a block with K <= 4096, 2 with K <= 12288, 1 with K <= 16384 (a row tile is
+ * 32 rows; blocks = compute units); others return BGEMM_EINVAL.  A block that waits longer than a quarter of
+ * a second for its predecessors gives up; bgemm_chain_status() (synchronises the stream) then returns
+ * BGEMM_ETIMEOUT and the output is undefined. */
+typedef struct bgemm_chain_layer {
+    const void* W_tiled;
+    const void* sw;
+    const void* bias;
+    const void* sa;
+    const void* next_zero_point;
+    int64_t M, K;
+    int64_t reserved;
+} bgemm_chain_layer;
+size_t bgemm_chain_workspace_bytes(int mode, const bgemm_chain_layer* layers, int n_layers, int64_t N);
+int bgemm_chain_forward(int mode, const bgemm_chain_layer* layers, const void* layers_dev, int n_layers,
+                        const void* X_tiled, const void* X2_tiled, int64_t N, void* out, int out_dtype,
+                        int param_dtype, void* ws, size_t ws_bytes, int flags, void* stream);
+int bgemm_chain_status(const void* ws, void* stream);
 
 #ifdef __cplusplus
 }

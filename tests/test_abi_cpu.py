@@ -29,7 +29,7 @@ def test_header_symbols_exported():
 
 def test_layout_sizes():
     L = _lib.lib()
-    assert L.bgemm_abi_version() == _lib.ABI_VERSION == 9
+    assert L.bgemm_abi_version() == _lib.ABI_VERSION == 10
     assert L.bgemm_tiled_words(1, 1) == 256
     assert L.bgemm_tiled_words(32, 256) == 256
     assert L.bgemm_tiled_words(33, 257) == 4 * 256

@@ -354,3 +354,18 @@ def test_packed_weight_cache_follows_the_parameter_and_can_be_dropped(cls):
         lin.weight.data.mul_(3.0)                    # (same signs: the bits would not change)
         lin.load_state_dict(sd)
         assert torch.equal(lin(x), y0)
+
+
+def test_packed_weight_cache_follows_the_weights_zero_point():
+    """The cached bits are those of (weight - zpw) (bgemm_linear.py:482): an in-place update of zpw alone packs again."""
+    torch.manual_seed(12)
+    lin = bl.BGEMMLinear(256, 64).to(DEV)
+    x = torch.randn(8, 256, device=DEV)
+    lin(x)
+    with torch.no_grad():
+        y0 = lin(x).clone()
+        lin.zpw.add_(0.5)                            # moves about two fifths of the signs
+        y1 = lin(x).clone()
+        lin.fuse_inference = False
+        want = lin(x)
+    assert not torch.equal(y0, y1) and torch.equal(y1, want)

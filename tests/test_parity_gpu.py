@@ -822,3 +822,25 @@ def test_scaled_fp16_matches_torchs_fp16_kernels_from_denormal_to_overflow(M, N,
                     want = want + bias
                 same = (got.view(torch.int16) == want.view(torch.int16)) | (got.isnan() & want.isnan())
                 assert bool(same.all()), (lo, hi, sa_v, bias is not None, int((~same).sum()))
+
+
+def test_bits_output_drops_row_popcounts_of_the_operand_it_overwrites(oracle):
+    """An operand that carried row popcounts and is then rewritten through bits_out must not feed the stale counts to
+    the counted kernel (XOR's rank-one terms would be those of the old bits)."""
+    rng = np.random.default_rng(5)
+    N, K, H, M = 256, 512, 1024, 512
+    x, w1, w2 = rand_f16(rng, N, K), rand_f16(rng, H, K), rand_f16(rng, M, H)
+    w1p, w2p, xp = lk.pack_sign(to_dev(w1)), lk.pack_sign(to_dev(w2)), lk.pack_sign(to_dev(x))
+    lk.row_popcounts(w2p)
+    hb = lk.zeros_packed(N, H, 1, DEV)
+    lk.row_popcounts(hb)                             # counts of the all-zero buffer
+    sw, sa = torch.ones(H, device=DEV), torch.ones(1, device=DEV)
+    lk.bgemm_packed_forward(w1p, xp, MODE_XOR, scale=(sw, sa, None), bits_out=hb)
+    assert hb.counts is None
+    got = lk.bgemm_packed_forward(w2p, hb, MODE_XOR, torch.int32)[0].cpu().numpy()
+    acc1 = oracle.c_bgemm_packed(1, oracle.c_pack_sign(w1), oracle.c_pack_sign(x), K)
+    h = oracle.np_center_to_f16(oracle.np_scale_epilogue(acc1, np.ones(H, np.float32), np.float32(1)), np.float32(0))
+    want = oracle.c_bgemm_packed(1, oracle.c_pack_sign(w2), oracle.c_pack_sign(h), H)
+    assert (got == want).all()
+    lk.row_popcounts(hb)                             # counted again: the counted kernel agrees
+    assert (lk.bgemm_packed_forward(w2p, hb, MODE_XOR, torch.int32)[0].cpu().numpy() == want).all()
