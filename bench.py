@@ -306,6 +306,7 @@ def probes():
     L.bench_probe_empty.argtypes = [ci, ci, p, p]
     L.bench_probe_read.argtypes = [p, i64, ci, ci, p, p]
     L.bench_probe_mfma.argtypes = [ci, ci, ci, ci, p, p]
+    L.bench_probe_exchange.argtypes = [p, ci, ci, ci, ci, ctypes.c_uint, p, ci, p]
     return L
 
 
@@ -354,6 +355,26 @@ def bench_floor(cold):
     res["sustained_read_361MB_us"] = round(best, 2)
     res["sustained_read_gbs"] = round(total / best / 1e3, 1)
     res["sustained_read_frac_of_8TBs"] = round(res["sustained_read_gbs"] / HBM_PEAK_GBS, 4)
+    # one all-to-all exchange among resident blocks (one per compute unit), the floor under a layer of the chain kernel:
+    # 3 units a block (a ternary row against two weight row tiles, less one), one replica and one replica per XCD
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    stride, rounds, epoch = cus * 8, 200, 1
+    buf = torch.zeros(2 * 8 * stride, dtype=torch.int64, device="cuda:0")
+    err = torch.zeros(2, dtype=torch.int64, device="cuda:0")
+    for copies in (1, 8):
+        best = None
+        for rep in range(3):
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            L.bench_probe_exchange(buf.data_ptr(), cus, 3, copies, rounds, epoch, err.data_ptr(), stride, st())
+            e1.record()
+            torch.cuda.synchronize()
+            epoch += rounds
+            us = 1e3 * e0.elapsed_time(e1) / rounds
+            best = us if best is None else min(best, us)
+        res["all_to_all_exchange_%d_blocks_%s_us" % (cus, "1_replica" if copies == 1 else "8_replicas")] = round(best, 3)
+    res["all_to_all_exchange_ok"] = bool((err == 0).all())
     return res
 
 

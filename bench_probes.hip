@@ -7,7 +7,9 @@
 //     the protocol of the reference's drivers (lowbit_kernel/csrc/kernel_test.h:10-11: warm-up launches, then
 //     timed launches between two events, which bench.py does around these entry points);
 //   * the same with a number of independent vector-ALU instructions after every MFMA, which is what the
-//     in-register bit expansion costs the matrix-core kernels.
+//     in-register bit expansion costs the matrix-core kernels;
+//   * what one all-to-all exchange of a few bytes per block costs blocks that stay resident (one per compute
+//     unit): the floor under a layer of the chain kernel, to be set against the cost of a kernel boundary.
 // Built into libbench_probes.so beside bench.py.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -83,6 +85,35 @@ __global__ __launch_bounds__(256) void probe_mfma_kernel(unsigned* out, const in
 }  // namespace
 
 // All return 0, -1 for bad arguments, or the hipError_t of the launch.
+// `rounds` all-to-all exchanges among the blocks of the grid: every round, every block stores `units` 8-byte
+// {tag, payload} units with device-scope stores into each of `copies` replicas and then polls every unit of replica
+// blockIdx % copies until it carries the round's tag.  Waits are bounded (0.2 s of the 100 MHz wall clock); a block
+// that runs out sets err[0] and leaves, a wrong payload counts in err[1].
+__global__ __launch_bounds__(512) void probe_exchange_kernel(unsigned long long* buf, const int units, const int copies, const int rounds,
+                                                            const unsigned epoch, unsigned long long* err, const int stride)
+{
+    const int G = gridDim.x, b = blockIdx.x, t = threadIdx.x, U = G * units;
+    const long long t0 = wall_clock64();
+    for (int r = 0; r < rounds; r++) {
+        unsigned long long* cur = buf + (size_t)(r & 1) * copies * stride;
+        const unsigned tag = epoch + r;
+        for (int i = t; i < units * copies; i += 512)
+            __hip_atomic_store(&cur[(size_t)(i / units) * stride + b * units + i % units],
+                               ((unsigned long long)tag << 32) | (unsigned)(b * 131 + i % units + r), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned long long* mine = cur + (size_t)(b % copies) * stride;
+        int bad = 0;
+        for (int i = t; i < U && !bad; i += 512) {
+            unsigned long long v = __hip_atomic_load(&mine[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for (unsigned tries = 1; (unsigned)(v >> 32) != tag; tries++) {
+                if ((tries & 63) == 0 && wall_clock64() - t0 > 20000000ll) { bad = 1; break; }
+                v = __hip_atomic_load(&mine[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            if (!bad && (unsigned)v != (unsigned)((i / units) * 131 + i % units + r)) atomicAdd(err + 1, 1ull);
+        }
+        if (__syncthreads_or(bad)) { if (t == 0) atomicAdd(err, 1ull); return; }
+    }
+}
+
 extern "C" int bench_probe_empty(int blocks, int threads, void* scratch, void* stream)
 {
     if (blocks <= 0 || threads <= 0 || threads > 1024) return -1;
@@ -95,6 +126,16 @@ extern "C" int bench_probe_read(const void* src, int64_t bytes, int blocks, int 
     if (!src || bytes < 16 || blocks <= 0 || threads <= 0 || threads > 512 || ((uintptr_t)src & 15)) return -1;
     hipLaunchKernelGGL(probe_read_kernel, dim3(blocks), dim3(threads), 0, (hipStream_t)stream, (const uint4*)src,
                        bytes / 16, (unsigned*)scratch);
+    return (int)hipGetLastError();
+}
+
+// buf: 2 * copies * stride units of 8 bytes, zero before the first call, stride >= blocks * units; epoch: a number that
+// is new for every call on the same buffer (advance it by `rounds`, starting at 1); err: two zeroed 8-byte counters.
+extern "C" int bench_probe_exchange(void* buf, int blocks, int units, int copies, int rounds, unsigned epoch, void* err, int stride, void* stream)
+{
+    if (!buf || !err || blocks <= 0 || units <= 0 || copies <= 0 || rounds <= 0 || stride < blocks * units) return -1;
+    hipLaunchKernelGGL(probe_exchange_kernel, dim3(blocks), dim3(512), 0, (hipStream_t)stream, (unsigned long long*)buf, units, copies, rounds,
+                       epoch, (unsigned long long*)err, stride);
     return (int)hipGetLastError();
 }
 

@@ -47,6 +47,8 @@ struct ChainArgs {
     unsigned long long* xg;                   // [2][u_max] units every block can see
     unsigned long long* xl;                   // [8][2][u_max] per-XCD replicas, or null: one level
     int u_max, kt_max;
+    long long* trace;                         // null, or [1 + 5 * n_layers] wall-clock stamps written by thread 0 of block 0: start; per layer
+                                              // operand in LDS, next layer requested, own K-tiles done, partial sums met, outputs published
     long long budget;                         // ticks of the 100 MHz wall clock a wait may take, from the kernel's start
     unsigned e_magic;                         // ceil(2^32 / E), E = planes * N units per word (unused for E = 1)
 };
@@ -72,15 +74,16 @@ __device__ __forceinline__ bool poll_units(const unsigned long long* src, const 
 #pragma unroll
         for (int c = 0; c < CHAIN_POLL_CH; c++) {
             const int u = base + c * stride;
-            v[c] = unit_load(src + (u < U ? u : u0));
+            v[c] = 0;
+            if (u < U) v[c] = unit_load(src + u);
         }
 #pragma unroll
         for (int c = 0; c < CHAIN_POLL_CH; c++) {
             const int u = base + c * stride;
             if (u >= U) continue;
-            while ((unsigned)(v[c] >> 32) != tag) {
-                if (wall_clock64() - t0 > budget) { ok = false; break; }
-                __builtin_amdgcn_s_sleep(1);
+            // (the wall clock is a slow read: looked at once in 64 tries)
+            for (unsigned tries = 1; (unsigned)(v[c] >> 32) != tag; tries++) {
+                if ((tries & 63u) == 0 && wall_clock64() - t0 > budget) { ok = false; break; }
                 v[c] = unit_load(src + u);
             }
             if (!ok) break;
@@ -124,7 +127,7 @@ __global__ __launch_bounds__(CHAIN_THREADS, 1) void gemm_chain_kernel(const Chai
     // layer's first tile instead, which is always there and stays in the cache; its registers are never used.
     // Parameters: thread i * 32 + c holds sw and bias of row c of tile i, thread NTM * 32 the two scalars; lanes
     // without a parameter read the tag base instead.
-    uint4 wq[2][NTM][KSM];
+    uint4 wq[NTM][KSM], wnext[NTM][KSM];      // this layer's tiles, the next layer's
     auto request_weights = [&](uint4 (&to)[NTM][KSM], const int l) {
         const ChainLayerDev& d = sL[l];
         const int MT = __builtin_amdgcn_readfirstlane((int)((d.M + 31) >> 5)), KT = __builtin_amdgcn_readfirstlane((int)((d.K + 255) >> 8));
@@ -179,7 +182,7 @@ __global__ __launch_bounds__(CHAIN_THREADS, 1) void gemm_chain_kernel(const Chai
     {
         P p0, p1;
         request_params(p0, p1, 0);
-        request_weights(wq[0], 0);
+        request_weights(wq, 0);
         const int KT0 = (int)((sL[0].K + 255) >> 8);
         for (int s = tid; s < a.kt_max * 64; s += CHAIN_THREADS) {
             const int kt = s >> 6, h = (s >> 5) & 1, prow = s & 31;
@@ -200,8 +203,13 @@ __global__ __launch_bounds__(CHAIN_THREADS, 1) void gemm_chain_kernel(const Chai
     }
 
     bool aborted = false;
-    auto body = [&](auto S_, const int l) -> bool {
-        constexpr int S = decltype(S_)::value;
+    const bool tracing = a.trace != nullptr && b == 0 && tid == 0;
+    const long long c0 = tracing ? clock64() : 0;
+    if (tracing) a.trace[0] = t0;
+    // One body for every layer (the LDS areas alternate by the layer's parity S, the registers are handed on at the end):
+    // a copy per parity would double the code, and the whole chain's code should stay in the instruction cache.
+    auto body = [&](const int l) -> bool {
+        const int S = l & 1;
         const ChainLayerDev& d = sL[l];
         const int M = __builtin_amdgcn_readfirstlane((int)d.M), K = __builtin_amdgcn_readfirstlane((int)d.K);
         const int MT = (M + 31) >> 5, KT = (K + 255) >> 8;
@@ -209,11 +217,13 @@ __global__ __launch_bounds__(CHAIN_THREADS, 1) void gemm_chain_kernel(const Chai
         const int ntb = MT > b ? (MT - b + G - 1) / G : 0;            // row tiles this block owns
         const bool has_bias = d.bias != nullptr;
 
+        if (tracing) a.trace[1 + 5 * l] = wall_clock64();
         // (1) the next layer's parameters and weights are requested before this layer is touched
         P np0, np1;
         request_params(np0, np1, last ? l : l + 1);
-        request_weights(wq[S ^ 1], last ? l : l + 1);
+        request_weights(wnext, last ? l : l + 1);
 
+        if (tracing) a.trace[2 + 5 * l] = wall_clock64();
         // (2) this wave's K-tiles of the block's row tiles against the operand in LDS
         typename Eng::Acc acc[NTM];
         int pa[NTM];
@@ -233,13 +243,14 @@ __global__ __launch_bounds__(CHAIN_THREADS, 1) void gemm_chain_kernel(const Chai
                 const typename Eng::Frag ax = Eng::expand_x(xq, s);
 #pragma unroll
                 for (int i = 0; i < NTM; i++)
-                    if (i < ntb) acc[i] = Eng::mma(ax, Eng::expand_w(wq[S][i][j], s), acc[i]);
+                    if (i < ntb) acc[i] = Eng::mma(ax, Eng::expand_w(wq[i][j], s), acc[i]);
             }
 #pragma unroll
             for (int i = 0; i < NTM; i++)
-                if (i < ntb) pa[i] += popc4(wq[S][i][j]);
+                if (i < ntb) pa[i] += popc4(wq[i][j]);
         }
 
+        if (tracing) a.trace[3 + 5 * l] = wall_clock64();
         // (3) the waves' partial sums meet in LDS (accumulator registers 4g .. 4g + 3 hold operand rows 8g .. 8g + 7)
         if (wave < KT) {
 #pragma unroll
@@ -257,6 +268,7 @@ __global__ __launch_bounds__(CHAIN_THREADS, 1) void gemm_chain_kernel(const Chai
             }
         }
         __syncthreads();
+        if (tracing) a.trace[4 + 5 * l] = wall_clock64();
 
         // (4) epilogue.  The areas of the other parity and the operand are cleared for the next layer, whose
         // parameters (requested in (1), before the weights, so they are here first) go to LDS.
@@ -318,6 +330,7 @@ __global__ __launch_bounds__(CHAIN_THREADS, 1) void gemm_chain_kernel(const Chai
             }
         }
         __syncthreads();
+        if (tracing) a.trace[5 + 5 * l] = wall_clock64();
         if (last) return true;
 
         // (5) the next layer's operand: MT words a row and plane, E units a word
@@ -343,15 +356,20 @@ __global__ __launch_bounds__(CHAIN_THREADS, 1) void gemm_chain_kernel(const Chai
         // Loads return in order, so the polls above have also seen the next layer's weights arrive; saying so keeps
         // the compiler from waiting for the requests of the NEXT body when this one's registers are first used.
         __builtin_amdgcn_s_waitcnt(0x0f70);          // vmcnt(0)
+#pragma unroll
+        for (int i = 0; i < NTM; i++)
+#pragma unroll
+            for (int j = 0; j < KSM; j++) wq[i][j] = wnext[i][j];
         __syncthreads();
         return sFlag[0] == 0;
     };
-    for (int l = 0; l < L; l += 2) {
-        if (!body(std::integral_constant<int, 0>{}, l)) { aborted = true; break; }
-        if (l + 1 >= L) break;
-        if (!body(std::integral_constant<int, 1>{}, l + 1)) { aborted = true; break; }
-    }
+    for (int l = 0; l < L; l++)
+        if (!body(l)) { aborted = true; break; }
 
+    if (tracing) {          // shader-clock ticks and wall-clock ticks of the whole launch: their ratio is the clock the launch ran at
+        a.trace[1 + 5 * CHAIN_MAX_LAYERS - 2] = clock64() - c0;
+        a.trace[1 + 5 * CHAIN_MAX_LAYERS - 1] = wall_clock64() - t0;
+    }
     // The last block to get here moves the tag base past this call's tags and re-arms the counter.
     if (tid == 0) {
         if (aborted) __hip_atomic_store(a.state + 2, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -389,7 +407,7 @@ static int chain_shape(int mode, const bgemm_chain_layer* layers, int n_layers, 
 {
     if (!mode_coef(mode, mc)) return fail(BGEMM_EINVAL, "bgemm_chain: unknown mode %d", mode);
     if (!layers) return fail(BGEMM_ENULL, "bgemm_chain: layers is NULL");
-    if (n_layers < 1 || n_layers > CHAIN_MAX_LAYERS) return fail(BGEMM_EINVAL, "bgemm_chain: 1 to %d layers, got %d", CHAIN_MAX_LAYERS, n_layers);
+    if (n_layers < 1 || n_layers > CHAIN_MAX_LAYERS - 1) return fail(BGEMM_EINVAL, "bgemm_chain: 1 to %d layers, got %d", CHAIN_MAX_LAYERS - 1, n_layers);
     if (N < 1 || N > (mc->planes == 2 ? 16 : 32))
         return fail(BGEMM_EINVAL, "bgemm_chain: N=%lld activation rows; one operand tile row holds up to %d", (long long)N, mc->planes == 2 ? 16 : 32);
     if (G < 1) return fail(BGEMM_ELAUNCH, "bgemm_chain: cannot read the number of compute units");
@@ -414,7 +432,8 @@ static int chain_shape(int mode, const bgemm_chain_layer* layers, int n_layers, 
     return BGEMM_OK;
 }
 
-static size_t chain_ws_bytes(const ChainShape& cs) { return 256 + (size_t)18 * cs.u_max * 8; }
+static size_t chain_trace_bytes() { return (1 + 5 * CHAIN_MAX_LAYERS) * 8; }
+static size_t chain_ws_bytes(const ChainShape& cs) { return 256 + (size_t)18 * cs.u_max * 8 + chain_trace_bytes(); }
 
 template <int NTM, int KSM, bool F32>
 static int chain_launch(const ChainArgs& a, int G, hipStream_t st)
@@ -461,7 +480,7 @@ extern "C" int bgemm_chain_forward(int mode, const bgemm_chain_layer* layers, co
         if (scaled && (!layers[l].sw || !layers[l].sa)) return fail(BGEMM_ENULL, "bgemm_chain_forward: layer %d has no sw or sa", l);
     }
     const int levels = flags & 3;
-    if (levels == 3) return fail(BGEMM_EINVAL, "bgemm_chain_forward: flags");
+    if (levels == 3 || (flags & 0xf8)) return fail(BGEMM_EINVAL, "bgemm_chain_forward: flags");
     ChainArgs a;
     memset(&a, 0, sizeof a);
     a.layers = (const ChainLayerDev*)layers_dev; a.n_layers = n_layers;
@@ -474,6 +493,7 @@ extern "C" int bgemm_chain_forward(int mode, const bgemm_chain_layer* layers, co
     const bool two_level = G % 8 == 0 && (levels == 2 || (levels == 0 && cs.u_max > 1024));
     a.xl = two_level ? a.xg + (size_t)2 * cs.u_max : nullptr;
     a.u_max = cs.u_max; a.kt_max = cs.kt_max;
+    a.trace = (flags & 4) ? (long long*)((char*)ws + 256 + (size_t)18 * cs.u_max * 8) : nullptr;
     a.budget = 25000000LL;          // a quarter of a second
     const unsigned E = (unsigned)(mc.planes * N);
     a.e_magic = E > 1 ? (unsigned)(((1ULL << 32) + E - 1) / E) : 0;

@@ -453,6 +453,14 @@ class DecodeChain:
                                                   self.flags, _stream()))
         return out
 
+    def trace(self, N):
+        """With flags & 4: microseconds since the launch's start at which block 0 (its first thread) had each layer's
+        operand in LDS, the next layer's weights requested, its own K-tiles multiplied, the block's partial sums met and
+        its outputs published, as an [n_layers, 5] tensor (of the last call with N rows)."""
+        ws = self.workspace(N)
+        t = ws[ws.numel() - (1 + 5 * 128) * 8:].view(torch.int64).cpu()
+        return (t[1:1 + 5 * len(self.layers)] - t[0]).reshape(-1, 5).double() / 100.0
+
     def check(self, N):
         """Waits for the stream and raises if a launch of this chain gave up waiting (BGEMM_ETIMEOUT)."""
         with _on(self.device):

@@ -291,8 +291,10 @@ int bgemm_f16_forward_static(const void* W, const void* X, void* C, int64_t M, i
  *   ws          : bgemm_chain_workspace_bytes() bytes, ZERO-FILLED ONCE before its first use and then left
  *                 to the library; calls that share a workspace, or run on one GPU at the same time, must not
  *                 overlap (each holds every compute unit until its last layer is done)
- *   flags       : 0, or 1 / 2 to insist on the one-level / two-level exchange; bits 8.. = number of blocks
- *                 (tests; 0 = one per compute unit)
+ *   flags       : 0, or 1 / 2 to insist on the one-level / two-level exchange; 4 = block 0 leaves wall-clock stamps
+ *                 (100 MHz ticks: start, then per layer operand ready / next layer requested / own K-tiles done /
+ *                 partial sums met / outputs published) in the last (1 + 5 * 128) * 8 bytes of the workspace; bits 8.. = number of blocks (tests;
+ *                 0 = one per compute unit)
  * Layers of up to 3 row tiles a block with K <= 4096, 2 with K <= 12288, 1 with K <= 16384 (a row tile is
  * 32 rows; blocks = compute units); others return BGEMM_EINVAL.  A block that waits longer than a quarter of
  * a second for its predecessors gives up; bgemm_chain_status() (synchronises the stream) then returns
