@@ -633,7 +633,25 @@ THRESHOLD_SHAPES = [
 ]
 
 
-def bench_thresholds(steps=60):
+# the shapes of the default run's `dispatch` block: the two sides of the most contested choices
+DISPATCH_SHAPES = [(1, 1, 8192, 8192, 2048), (1, 1, 8192, 2048, 4096), (1, 1, 11008, 768, 4096), (1, 1, 8192, 256, 4096), (1, 1, 8192, 256, 8192),
+                   (1, 1, 8192, 512, 8192), (1, 1, 8192, 768, 8192), (1, 1, 11008, 640, 8192), (1, 1, 2000, 4000, 1024), (1, 1, 4096, 256, 4096),
+                   (1, 1, 2048, 256, 16384), (2, 1, 11008, 128, 4096), (2, 1, 4096, 256, 11008), (2, 1, 8192, 256, 8192), (2, 1, 11008, 576, 8192),
+                   (1, 1, 12288, 160, 8192)]
+
+
+def dispatch_summary(rows):
+    """How far the library's own choice is from the fastest kernel that can take each shape (cold weights): the
+    largest and the 90th-percentile ratio and the three worst shapes."""
+    rs = sorted((r["auto_vs_fastest_cold"], r["shape"], r["auto"], r["fastest_cold"]) for r in rows if r.get("auto_vs_fastest_cold"))
+    if not rs:
+        return None
+    return {"shapes": len(rs), "regret_max": rs[-1][0], "regret_p90": rs[min(len(rs) - 1, int(0.9 * len(rs)))][0],
+            "worst": [{"shape": x[1], "auto": KERNEL_IDS.get(x[2], x[2]), "fastest": KERNEL_IDS.get(x[3], x[3]), "x": x[0]} for x in rs[-3:][::-1]],
+            "mismatch": [r["shape"] for r in rows if "mismatch" in r]}
+
+
+def bench_thresholds(steps=60, shapes=None, warm=True):
     """Every shape above under every kernel that can take it (BGEMM_FORCE_KERNEL), weights from HBM (rotating copies
     beyond the Infinity Cache) and from a warm cache: the timings the dispatch thresholds of the library rest on."""
     import torch
@@ -643,7 +661,7 @@ def bench_thresholds(steps=60):
     general = [B.KERNEL_MFMA_256x256, B.KERNEL_MFMA_256x128, B.KERNEL_MFMA_128x128, B.KERNEL_MFMA_64x128, B.KERNEL_MFMA_32x128,
                B.KERNEL_MFMA_32x256, B.KERNEL_MFMA_128x64, B.KERNEL_MFMA_64x64]
     rows = []
-    for planes, batch, M, N, K in THRESHOLD_SHAPES:
+    for planes, batch, M, N, K in (shapes or THRESHOLD_SHAPES):
         mode = lk.MODE_BWTA if planes == 2 else lk.MODE_XOR
         wbytes = batch * M * K // 8
         copies = max(2, min(40, int(300e6 // wbytes)))
@@ -680,11 +698,13 @@ def bench_thresholds(steps=60):
             elif not torch.equal(out, ref):
                 res["mismatch"] = KERNEL_NAMES[kid]
             res["us_cold"][KERNEL_NAMES[kid]] = round(1e3 * time_gpu_graph(fn, copies, 2, max(2, steps // copies)), 2)
-            res["us_warm"][KERNEL_NAMES[kid]] = round(1e3 * time_gpu_graph(lambda i: fn(0), 8, 2, max(2, steps // 8)), 2)
+            if warm:
+                res["us_warm"][KERNEL_NAMES[kid]] = round(1e3 * time_gpu_graph(lambda i: fn(0), 8, 2, max(2, steps // 8)), 2)
         res["fastest_cold"] = min(res["us_cold"], key=res["us_cold"].get)
         res["auto_vs_fastest_cold"] = round(res["us_cold"][res["auto"]] / res["us_cold"][res["fastest_cold"]], 3) if res["auto"] in res["us_cold"] else None
         rows.append(res)
-        log(json.dumps(res))
+        if shapes is None:
+            log(json.dumps(res))
         del pool, wps, xp, out
     return rows
 
@@ -804,10 +824,13 @@ def main():
         res = {"chain": lambda: bench_chain(cold), "c2": lambda: [bench_c2()], "c3": lambda: [bench_c3(), bench_qk()], "c4": lambda: section_decode(cold), "prefill": bench_prefill,
                "sweep": bench_sweep, "floor": lambda: bench_floor(cold), "peak": lambda: bench_mfma_peak(cold),
                "thresholds": bench_thresholds}[args.only]()
-        print(json.dumps({args.only: res}), flush=True)
+        out = {args.only: res}
+        if args.only == "thresholds":
+            out["dispatch"] = dispatch_summary(res)
+        print(json.dumps(out), flush=True)
         return
 
-    extra = floor = peak_measured = None
+    extra = floor = peak_measured = dispatch = None
     if not args.headline_only:
         cold = ColdRead()
         floor = bench_floor(cold)
@@ -815,6 +838,8 @@ def main():
         peak_measured = bench_mfma_peak(cold)
         log("mfma peak:", json.dumps(peak_measured))
         extra = all_configs(cold)
+        dispatch = dispatch_summary(bench_thresholds(40, DISPATCH_SHAPES, warm=False))
+        log("dispatch:", json.dumps(dispatch))
         del cold
         torch.cuda.empty_cache()
 
@@ -865,6 +890,7 @@ def main():
         line["config"]["c4_chain_frac_hbm"] = {r["id"].split(" N=")[1].split(",")[0]: r["frac"] for r in extra if r["id"].startswith("C4 chain")}
         line["config"]["c4_chain_us_per_layer"] = {r["id"].split(" N=")[1].split(",")[0]: r["us"] for r in extra if r["id"].startswith("C4 chain")}
         line["all_configs"] = extra
+        line["dispatch"] = dispatch
         line["floor"] = floor
         line["mfma_peak_measured"] = peak_measured
     print(json.dumps(line), flush=True)

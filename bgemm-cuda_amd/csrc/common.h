@@ -306,15 +306,12 @@ int launch_gemm_mfma(const GemmArgs& a, hipStream_t st, bool fp4);
 int gemm_mfma_kernel_id(int64_t batch, int64_t M, int64_t N, int64_t KT, int planes, int out_shift);     // BGEMM_KERNEL_MFMA_* by shape
 // A ternary operand's two planes on the general kernel's pipelined 128 x 128 tile (two resident blocks per CU): from two
 // thirds of a block per CU on 16 K-tiles or more, except between one block per CU and one and two thirds, which would
-// leave the launch waiting for the CUs that run two (11008 x 256 ternary rows x 8192, 172 blocks: 21.9 us against 28.8 on
-// four pieces a block; 4096 x 1024 x 11008, 256 blocks: 29.0 against 42.6; 11008 x 320 x 11008, 258 blocks: 48.5 against
-// 39.5; 8192 x 640 x 8192, 320 blocks: 37.2 against 31.6 on 32 x 256; 11008 x 512 x 16384, 344 blocks: 69.0 against 61.2;
-// 11008 x 576 x 8192, 430 blocks: 39.9 against 41.9).
+// leave the launch waiting for the CUs that run two, and only where most of the tiles land on real outputs.
 static inline bool two_plane_tile_128(int64_t batch, int64_t M, int64_t N, int64_t KT)
 {
     const int64_t b = batch * cdiv(N, 128) * cdiv(M, 128);
     const double filled = (double)(N * M) / (double)(cdiv(N, 128) * 128 * cdiv(M, 128) * 128);
-    return KT >= 16 && b >= 172 && !(b > 256 && b < 416) && filled >= 0.75;      // (11008 x 160 rows fill 0.63 of their tiles: 20.0 us against 17.5)
+    return KT >= 16 && b >= 172 && !(b > 256 && b < 416) && filled >= 0.75;
 }
 int gemm_skinny_kernel_id(const GemmArgs& a, bool fp4);                                   // BGEMM_KERNEL_SKINNY_* by shape
 int launch_gemm_valu(const GemmArgs& a, hipStream_t st);

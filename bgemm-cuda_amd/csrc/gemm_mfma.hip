@@ -16,7 +16,7 @@ namespace bgemm {
 
 // Block = WGN x WGM waves, each wave owns WN x WM tiles of 32x32 outputs, PL activation planes.
 // COUNTED (pipelined tiles only): the operands' row popcounts come with the call (GemmArgs::cntW / cntX) and the main
-// loop counts nothing: a sixth of its vector instructions on the 256 x 128 tile, 4 % of an 8192^3 launch.
+// loop counts nothing: a sixth of its vector instructions on the 256 x 128 tile.
 template <typename Eng, int WGN, int WGM, int WN, int WM, int PL, bool PIPE, bool COUNTED = false>
 // (Second launch bound: from two waves a SIMD on, a wave's register budget is the 256 architected registers, and the
 // compiler then keeps the accumulators there instead of in the accumulation registers, which the epilogue could
@@ -33,26 +33,19 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
     const int per_gemm = tiles_n * tiles_m;
     const int tile_id = bid % per_gemm, b = bid / per_gemm;
     // Tiles are walked in bands along n, so that the blocks in flight share their weight panels: eight tile rows, or two
-    // of the 128- and 256-row tiles on fewer than 32 K-tiles.  With two, blocks that run together write 16 KiB and more of
-    // every output row they touch instead of 4 KiB (8192^2 x 2048: 77.0 -> 68.4 us, 16384 x 8192 x 2048: 156.5 -> 140.6,
-    // 11008 x 8192 x 1024: 89.8 -> 76.4, 16384 x 8192 x 4096: 220.5 -> 205.4; two tile rows of the small tiles are up
-    // to a quarter slower).  From 32 K-tiles on the operands' reuse weighs as much: 8192^3 is 3 % faster on two with
-    // weights that rotate through HBM and 1.5 % slower with the same operands every launch; four there (rotating
-    // weights: 8192^3 176.0 -> 171.5 us, 16384 x 4096 x 8192 173.0 -> 169.9; the same operands every launch: level).
+    // of the 128- and 256-row tiles on fewer than 32 K-tiles (blocks that run together then write 16 KiB and more of every
+    // output row they touch instead of 4 KiB, which is what large outputs on a short K wait for; two tile rows of the small
+    // tiles are slower), four from 32 K-tiles on, where the operands' reuse in L2 weighs as much.
     const int band = WGN * WN * 32 >= 128 && a.KT < 128 ? (a.KT < 32 ? 2 : 4) : 8;
     int tn_block, tm;
     int sn = a.KT < 16 ? 4 : 2;
-    // (the other way round where only that divides, below 32 K-tiles: 11008 x 2048 x 4096, 16 x 86 tiles, 44.2 -> 41.5 us; on
-    // 32 K-tiles the same shape loses 3 % that way)
+    // (the other way round where only that divides, below 32 K-tiles)
     if (a.KT < 32 && (tiles_n % sn != 0 || tiles_m % (8 / sn) != 0)) sn = 8 / sn;
     const int sm = 8 / sn;
     if (WGN * WN * 32 >= 128 && gridDim.x == (unsigned)per_gemm && tiles_n % sn == 0 && tiles_m % sm == 0) {
         // One GEMM on the tall tiles whose tile grid splits evenly: XCD x (the hardware's block id modulo 8) takes a
         // sub-rectangle of the grid, 1/2 x 1/4 of it (1/4 x 1/2 on a short K), and walks that in bands: its L2 then
-        // needs a half and a quarter of the operands instead of an eighth of one and all of the other (weights
-        // rotating through HBM: 8192^3 170.3 -> 164.9 us, 16384 x 8192 x 4096 205.7 -> 197.2, 8192 x 4096 x 4096 53.5 ->
-        // 51.2, 8192^2 x 2048 67.9 -> 62.5; the same operands every launch: level, and the bytes the L2s fetch there
-        // stay what they were, 123 MiB a launch of 8192^3).
+        // needs a half and a quarter of the operands instead of an eighth of one and all of the other.
         const int x = blockIdx.x % 8, y = blockIdx.x / 8, sub_n = tiles_n / sn, sub_m = tiles_m / sm;
         const int bd = y / (band * sub_m), ib = y % (band * sub_m);
         const int n0 = bd * band, bh = min(band, sub_n - n0);
@@ -738,84 +731,51 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
 // ---- host side ---------------------------------------------------------------------------
 struct MfmaCfg { int id, bn, bm; };
 
-// Tile choice, from timings of every tile over a sweep of shapes (bench.py --only thresholds prints them): the
-// 256 x 256 tile (one block per CU, hand-pipelined loop, the fastest main loop) needs at least two rounds of
-// blocks and a long K (from 128 K-tiles) to pay for its epilogue, during which its CU computes nothing;
-// 256 x 128 (two resident blocks per CU that run half a tile apart, so one block's stores overlap the other's
-// main loop) from half a block per CU upwards on a long K (see below), from two below that, except on very
-// short K (under 4 K-tiles), where 128 x 128 keeps more waves in flight for what is then all prologue and
-// epilogue; below that the smaller tiles, down to 32 x 128, are
-// chosen so that every CU gets a block.  Narrow outputs (M <= 64) take 64-wide tiles: 128 rows from four
-// blocks per CU on, else 64 (192 x [512 x 512] x [512 x 64]: 7.0 against 7.3 us).
+// Tile choice.  Every rule below separates two tiles whose timings cross at that point; `bench.py --only thresholds`
+// re-times every tile on shapes either side of each rule and reports how far this function's choice is from the fastest
+// kernel (the default run carries a summary).  The terms: `blocks` of a tile shape, `filled` = the share of a tiling's
+// matrix-core work that lands on real outputs, K-tiles of 256 bits, 256 compute units holding one 256 x 256 block, two
+// 256 x 128 blocks or three 128 x 128 blocks each.
+//   * 256 x 256: one wave a SIMD and the cheapest loop per MFMA, but its epilogue is exposed: two rounds of blocks and a
+//     very long K (128 K-tiles).
+//   * 256 x 128: two resident blocks a unit, one storing while the other multiplies: from two blocks a unit; on 16 K-tiles
+//     or more already from half a block a unit, since its loop is so much cheaper per MFMA than the smaller tiles', except
+//     where a few units would run two blocks while the rest run one (257 to 384 blocks), or a last round would leave most
+//     of the GPU idle.
+//   * 128 x 128: runs the same hand-pipelined loop from 8 K-tiles on; from 192 blocks (144 on 16 K-tiles or more).
+//   * 32 x 256: a short K into 2-byte outputs or into int32 rows a power of two long (many small blocks drift apart and
+//     spread their stores over the memory channels), and two bit planes (one weight expansion feeds both planes).
+//   * 64 x 128, 32 x 128: whatever is left, so that every unit gets a block; 64-column tiles for outputs of at most 64
+//     columns.
 static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int planes, int out_shift)
 {
     auto blocks = [&](int bn, int bm) { return batch * cdiv(N, bn) * cdiv(M, bm); };
-    // the share of a tiling's MFMA work that lands on real outputs: a batch of [1024 x 64] outputs would fill a quarter
-    // of its 256-row tiles (74 us against 32 on a tile that fits, for 384 of them with K = 2048)
     auto filled = [&](int bn, int bm) { return (double)(N * M) / (double)(cdiv(N, bn) * bn * cdiv(M, bm) * bm); };
-    if (M <= 64) return blocks(128, 64) >= 1024 ? MfmaCfg{BGEMM_KERNEL_MFMA_128x64, 128, 64} : MfmaCfg{BGEMM_KERNEL_MFMA_64x64, 64, 64};   // narrow outputs
-    // a short K with a 2-byte output is all store path: rows of 512 bytes per block, many blocks in flight
-    // (192 x [512 x 512] x 64 -> fp16: 19.4 us against 20.4 on 128 x 128 and 25 to 29 on the tiles without paired
-    // columns; int32 output, 32 us for 201 MB, shows no preference)
-    // (one K-tile only: from two on, 128 x 128 is 15 % ahead: 48 x [1024 x 512] x 512 -> fp16 13.3 against 15.6 us)
-    // (from two such tiles a row on: 192 x [2048 x 256] x 256 -> fp16, one tile a row, 39.3 us against 35.5 on 128 x 128)
-    if (KT < 2 && out_shift == 1 && M >= 512 && blocks(32, 256) >= 512) return {BGEMM_KERNEL_MFMA_32x256, 32, 256};
-    // one K-tile into more int32 output than the 256 MiB memory-side cache holds: the same tile again (48 x [1024 x 2048] x
-    // 64, 403 MB: 70.4 us against 84.5 on 128 x 128; 192 x [512 x 1024] x 64: 71.9 against 76.3; at 201 MB no difference)
-    if (KT < 2 && out_shift == 2 && M >= 512 && batch * N * M > (64 << 20) && blocks(32, 256) >= 512)
-        return {BGEMM_KERNEL_MFMA_32x256, 32, 256};
-    // a short K with int32 rows of a power of two in bytes (4 to 64 KiB): the few large blocks of such a launch all
-    // run in step, and the rows they store at one moment lie a multiple of 1 MiB apart, on few memory channels;
-    // four times as many 32-row blocks drift apart (2048 x 4096 x 1024: 9.5 us against 12.6 on 128 x 128, 4096 x 2048 x
-    // 1024: 9.5 against 11.3, 16384 x 1024 x 1024: 17.7 against 21.9 on 256 x 128; 2000 x 4000 x 1024 shows no difference).
-    // From 1024 such blocks, up to 64 MiB of output; beyond, the larger tiles' rounds have drifted apart as well.
-    if (batch == 1 && planes == 1 && out_shift == 2 && KT <= 6 && M >= 1024 && M <= 16384 && (M & (M - 1)) == 0 &&
-        N * M <= (16 << 20) && blocks(32, 256) >= 1024)
-        return {BGEMM_KERNEL_MFMA_32x256, 32, 256};
-    // 256 x 256 (one wave a SIMD, the epilogue in the open) against 256 x 128 (two resident blocks a unit, one
-    // storing while the other multiplies, but half again as many expansions per MFMA).  With operands that come
-    // from HBM the smaller tile wins up to K = 16384 at least (8192^2 x 8192: 173 against 190 us, x 16384: 314 against
-    // 329); with operands that stay in the caches the two tie at K = 16384 and the larger one is 2 % ahead at 32768
-    if (planes == 1 && blocks(256, 256) >= 512 && KT >= 128 && filled(256, 256) >= 0.8) return {BGEMM_KERNEL_MFMA_256x256, 256, 256};
-    // from two blocks a unit; with 16 K-tiles or more from 132 blocks, i.e. as soon as the next tile down no longer has
-    // a unit to itself for every block (11008 x 512 x 8192, 172 blocks, 22.6 us against 29.6 to 33.2 on the smaller tiles;
-    // 8192 x 768 x 4096, 192 blocks, 14.9 against 17.1 to 18.9; 4352 x 1024 x 8192, 136 blocks, 21.1 against 23.9; but
-    // 2560 x 1536 x 8192, 120 blocks, 21.0 against 16.5 on 240 blocks of 128 x 128), except from a few blocks more than one
-    // a unit (11008 x 768 x 4096: 258, 11008 x 640 x 8192 likewise) to one and a half (6144 x 2048 x 16384: 384 blocks, 72.6
-    // against 71.3), which would leave the launch waiting for the units that run two blocks each while three blocks of
-    // the next tile down fit every unit at once: those go to the next tile down; so do 192 to 256 blocks on fewer than 24
-    // K-tiles (8192 x 768 x 4096: 14.7 us on 128 x 128 with three K-tiles in flight against 16.1)
-    const int64_t b21 = blocks(256, 128);
-    // a last round that leaves most of the GPU idle (576 blocks on 512 places: 6144 x 3072 x 4096 42.5 us against 34.9 on
-    // 128 x 128, whose 1152 blocks fill one and a half rounds of 768 places) goes to the smaller tile
     auto round_fill = [](int64_t b, int64_t places) { return (double)b / (double)(cdiv(b, places) * places); };
-    const bool last_round_idle = KT >= 8 && (KT <= 16 || b21 <= 600) && b21 > 256 &&      // (on a longer K the larger tile's cheaper loop makes up for it,
-                                                                                           //  but for a few blocks past one round: 9216 x 2048 x 8192, 576 blocks, 56.4 against 59.8 us)
-                                 round_fill(blocks(128, 128), 768) >= round_fill(b21, 512) + 0.15 &&
-                                 filled(128, 128) >= 0.6;
-    if (planes == 1 && !last_round_idle && (b21 >= 512 || (KT >= 16 && b21 >= 132 && (b21 < 192 || KT >= 24) && !(b21 > 256 && b21 <= 384))) &&
-        (KT >= 8 || (out_shift == 2 && KT >= 4 && batch * N * M >= (64 << 20)) || blocks(128, 128) < 512) &&      // (2-byte outputs leave 128 x 128 without staging in LDS:
-        filled(256, 128) >= 0.75)                                          //  48 x [2048 x 2048] x 1024 -> fp16 117 against 131 us; int32 on 4 to 7 K-tiles: the larger tile
-                                                                           //  from 256 MiB of output on, 8192^2 x 1024 58.7 against 69.9 us, below that the smaller one, 16384 x 2048 x 1024 27.7 against 32.8)
+    const int64_t out_elems = batch * N * M, b32 = blocks(32, 256), b21 = blocks(256, 128), b11 = blocks(128, 128);
+    if (M <= 64) return blocks(128, 64) >= 1024 ? MfmaCfg{BGEMM_KERNEL_MFMA_128x64, 128, 64} : MfmaCfg{BGEMM_KERNEL_MFMA_64x64, 64, 64};
+    // one K-tile: all store path.  2-byte outputs, or more int32 output than the memory-side cache holds
+    if (KT < 2 && M >= 512 && b32 >= 512 && (out_shift == 1 || out_elems > (64 << 20))) return {BGEMM_KERNEL_MFMA_32x256, 32, 256};
+    // up to six K-tiles into int32 rows of a power of two in bytes, up to 64 MiB of output
+    if (batch == 1 && planes == 1 && out_shift == 2 && KT <= 6 && M >= 1024 && M <= 16384 && (M & (M - 1)) == 0 &&
+        N * M <= (16 << 20) && b32 >= 1024)
+        return {BGEMM_KERNEL_MFMA_32x256, 32, 256};
+    if (planes == 1 && blocks(256, 256) >= 512 && KT >= 128 && filled(256, 256) >= 0.8) return {BGEMM_KERNEL_MFMA_256x256, 256, 256};
+    // 256 x 128 unless its last round would leave most of the GPU idle where 128 x 128 fills its own
+    const bool last_round_idle = KT >= 8 && (KT <= 16 || b21 <= 600) && b21 > 256 &&
+                                 round_fill(b11, 768) >= round_fill(b21, 512) + 0.15 && filled(128, 128) >= 0.6;
+    const bool few_blocks_ok = KT >= 16 && b21 >= 132 && (b21 < 192 || KT >= 24) && !(b21 > 256 && b21 <= 384);
+    const bool k_long_enough = KT >= 8 || (out_shift == 2 && KT >= 4 && out_elems >= (64 << 20)) || b11 < 512;
+    if (planes == 1 && !last_round_idle && (b21 >= 512 || few_blocks_ok) && k_long_enough && filled(256, 128) >= 0.75)
         return {BGEMM_KERNEL_MFMA_256x128, 256, 128};
-    // (with its pipelined loop, from eight K-tiles on, 192 blocks are enough: 3072 x 1024 x 8192 15.3 us against 17.3 to 20.1;
-    // from 16 K-tiles on 144: 6144 x 384 x 11008 16.9 against 18.9 to 22.9, 9216 x 256 x 4096 9.2 against 10.2 to 10.9,
-    // 11008 x 256 x 6144 12.0 against 14.5 to 17.5; level at eight K-tiles)
-    // (on 16 to 23 K-tiles and fewer than 192 blocks only where the tiles are full: 9216 x 160 x 4096, 0.63 of them, 9.0 against 8.1
-    // on 32 x 128)
-    if ((blocks(128, 128) >= 512 || (planes == 1 && KT >= 8 && blocks(128, 128) >= (KT >= 16 ? 144 : 192) &&
-                                     (blocks(128, 128) >= 192 || KT >= 24 || filled(128, 128) >= 0.85) &&
-                                     // (between one block per CU and one and two thirds on a short K the launch waits for the CUs
-                                     //  that run two: 8192 x 640 x 2048, 320 blocks, 10.4 us against 9.6 on 64 x 128; level from 16 K-tiles)
-                                     !(KT < 12 && blocks(128, 128) > 256 && blocks(128, 128) < 416))) && filled(128, 128) >= 0.6)
-        return {BGEMM_KERNEL_MFMA_128x128, 128, 128};
+    // 128 x 128: two rounds' worth of blocks, or (one plane, pipelined loop) from 192 / 144 blocks, not where some units
+    // would run two blocks and the rest one on a short K
+    const bool pipelined_ok = planes == 1 && KT >= 8 && b11 >= (KT >= 16 ? 144 : 192) &&
+                              (b11 >= 192 || KT >= 24 || filled(128, 128) >= 0.85) && !(KT < 12 && b11 > 256 && b11 < 416);
+    if ((b11 >= 512 || pipelined_ok) && filled(128, 128) >= 0.6) return {BGEMM_KERNEL_MFMA_128x128, 128, 128};
     if (planes == 2 && two_plane_tile_128(batch, M, N, KT)) return {BGEMM_KERNEL_MFMA_128x128, 128, 128};
-    // two bit planes: 32 x 256 shares every weight expansion between the planes of one row tile (W[11008,4096] x 128
-    // ternary rows 9.7 us against 10.9 / 11.3 on the next two; W[12288,11008] x 384 rows 47.4 against 55.7), once it
-    // has 160 blocks (96 from eight K-tiles on, where it runs the pipelined loop: W[11008,4096] x 96 ternary rows 8.4 us
-    // against 10.0 on 32 x 128)
-    if (planes == 2 && blocks(32, 256) >= (KT >= 8 ? 96 : 160)) return {BGEMM_KERNEL_MFMA_32x256, 32, 256};
-    if (blocks(64, 128) >= 512 && filled(64, 128) >= 0.6) return {BGEMM_KERNEL_MFMA_64x128, 64, 128};      // below two blocks a unit, twice as many 32-row tiles are faster
+    if (planes == 2 && b32 >= (KT >= 8 ? 96 : 160)) return {BGEMM_KERNEL_MFMA_32x256, 32, 256};
+    if (blocks(64, 128) >= 512 && filled(64, 128) >= 0.6) return {BGEMM_KERNEL_MFMA_64x128, 64, 128};
     return {BGEMM_KERNEL_MFMA_32x128, 32, 128};
 }
 

@@ -784,64 +784,41 @@ __global__ __launch_bounds__(KW * 64, 2) void gemm_skinny_splitk_quad_kernel(con
     }
 }
 
-// Shapes the four-pieces kernel takes: at least two tile rows on either side, enough blocks to give every
-// compute unit one, and a K long enough for the shared expansions to outweigh the larger meeting area (timed
-// against both neighbours, weights from HBM and from a warm cache, pieces = 32 x 32 outputs).  One bit plane:
-// up to 1024 pieces from 16 K-tiles on, 2048 from 24 (8192 x 256 x 16384: 18.7 us against 23.8 on the general kernel's
-// pipelined 128 x 128 tile; beyond that the tile is ahead: 6144 x 384 x 11008, 2304 pieces, 16.9 against 18.9 here; 8192 x
-// 512 x 12288, 4096 pieces, 21.3 against 24.9).  Two planes (twice the
-// matrix-core work per piece): from 24 K-tiles on, from 256 blocks (192 from 40 K-tiles on: W[4096,11008] x 96 ternary
-// rows 8.2 us against 9.3 on one piece a block) up to 512.  Beyond that the general kernel's tiles re-read less.
+// Shapes the four-pieces kernel takes (pieces = 32 x 32 outputs, blocks of 2 x 2 pieces, or of one tile row of both planes
+// x two weight tiles): at least two tile rows on either side, one round of blocks (192 / 256 to 512: fewer leave compute
+// units idle, more are a second round, where the general kernel's tiles re-read less), and a K long enough for the shared
+// expansions to outweigh the larger meeting area: one plane up to 1024 pieces from 16 K-tiles, 2048 from 24; two planes
+// from 24 K-tiles.  `bench.py --only thresholds` times it against both neighbours.
 static bool skinny_quad_shape(int planes, int64_t batch, int64_t M, int64_t N, int64_t KT)
 {
     const int64_t MT = row_tiles(M), NT = row_tiles(N);
-    // (two planes: one tile row of more than 16 rows as well: the block's two operands are its two planes; up to 16 rows
-    // both planes share ONE operand on the one-piece kernel, half the matrix-core work)
+    // (two planes of up to 16 rows share ONE operand on the one-piece kernel: half the matrix-core work)
     if (MT < 2 || (planes == 2 ? N <= 16 : NT < 2)) return false;
     if (batch > 1 && KT < 24) return false;      // (a batch of small products: operands that were just written, see gemm_skinny_shape)
-    const int64_t pieces = batch * MT * NT;
     if (planes == 2 && two_plane_tile_128(batch, M, N, KT)) return false;      // (the general kernel's pipelined tile is ahead there)
-    if (planes == 2)
-    {
-        // one round of blocks (up to 512: four K ways, two blocks a CU); with more, the general kernel's 32 x 256 tile,
-        // which runs two planes on its pipelined loop, is ahead (8192 x 160 ternary rows x 8192, 640 blocks: 13.2 us
-        // there against 16.0 here; 11008 x 96 x 8192, 516 blocks: 13.4 against 16.7; 8192 x 128 x 8192, 512 blocks: 13.3
-        // against 11.7)
-        const int64_t blocks2 = batch * cdiv(MT, 2) * NT;
-        return KT >= 24 && blocks2 >= (KT >= 40 ? 192 : 256) && blocks2 <= 512;
-    }
-    const int64_t blocks1 = batch * cdiv(MT, 2) * cdiv(NT, 2);
-    if (blocks1 < (KT >= 40 ? 192 : 256)) return false;      // (7168 x 128 x 11008, 224 blocks: 9.9 us against 11.8 on one piece a block)
-    // one round of blocks, as for two planes (odd tile counts make more blocks of the same pieces: 12288 x 160 x 8192, 576
-    // blocks, 16.2 us against 14.7 on 128 x 128; 10240 x 160 x 8192, 480 blocks: 12.7 against 14.1)
-    if (blocks1 > 512) return false;
-    return pieces <= (KT >= 24 ? 2048 : KT >= 16 ? 1024 : 0);
+    const int64_t blocks = batch * cdiv(MT, 2) * (planes == 2 ? NT : cdiv(NT, 2));
+    if (blocks < (KT >= 40 ? 192 : 256) || blocks > 512) return false;
+    if (planes == 2) return KT >= 24;
+    return batch * MT * NT <= (KT >= 24 ? 2048 : KT >= 16 ? 1024 : 0);
 }
 
-// Shapes the skinny kernels take: one group of activation rows always (32 rows, or 16 rows of two bit planes).
-// More groups where splitting K inside the block buys more than the general kernel's 32 x 128 tiles do (timed
-// over sweeps of shapes, pieces = 32 x 32 outputs): up to 1024 pieces from eight K-tiles on, one bit plane or two (two operands a block against one weight expansion); on four
-// to seven K-tiles up to 512 pieces of two bit planes, or up to two tile rows of activations.  The last bound is set by
-// weights that come from HBM rather than from a warm cache (a model's layers): there the general kernel's serial
-// K loop pays the full memory latency per step.  Beyond, the four-pieces kernel where that pays (see above),
-// else the general one (W[11008,4096] x 128 ternary rows, 1376 pieces: 9.7 us there against 12.5 here).
+// Shapes the skinny kernels take: one group of activation rows always (32 rows, or 16 rows of two bit planes).  More
+// groups where splitting K inside the block buys more than the general kernel's 32 x 128 tiles do (pieces = 32 x 32 outputs):
+// up to 1024 pieces from eight K-tiles on (512 for a batch of products: attention-shaped work on operands that were just
+// written and sit in the caches, where the general kernel keeps up); on four to seven K-tiles up to 512 pieces of two bit
+// planes, or few tile rows of activations.  The bounds are set by weights that come from HBM (a model's layers): there the
+// general kernel's serial K loop pays the full memory latency per step.  Beyond, the four-pieces kernel where that pays,
+// else the general one.
 bool gemm_skinny_shape(int planes, int64_t batch, int64_t M, int64_t N, int64_t K)
 {
     if (batch > 65535) return false;             // these kernels walk the batch in the grid's third dimension
     if (N <= (planes == 2 ? 16 : 32)) return true;
-    const int64_t pieces = batch * row_tiles(M) * row_tiles(N), KT = k_tiles(K);
+    const int64_t NT = row_tiles(N), pieces = batch * row_tiles(M) * NT, KT = k_tiles(K);
     if (skinny_quad_shape(planes, batch, M, N, KT)) return true;
-    // (a batch of products is attention-shaped work on operands that were just written and still sit in the caches:
-    // there the general kernel keeps up from 512 pieces on; 8 x [128 x 1024] x 2048, 1024 pieces: 4.3 us there, 5.1 here)
     if (KT >= 8) return pieces <= (batch > 1 ? 512 : 1024);
     if (KT < 4) return false;
-    if (planes == 2) return pieces <= 512 || (row_tiles(N) <= 2 && pieces <= 1024);      // (11008 x 48 ternary rows x 1792: 4.7 us here against 5.7)
-    // four to seven K-tiles, one bit plane: few tile rows of activations (1024 x 384 x 1024: 3.6 us here against 3.2
-    // on 32 x 128 tiles, 2048 x 192 x 1792: 4.1 against 3.7; 11008 x 40 x 1792: 4.3 here against 5.3, 16384 x 40 x 1024: 4.1
-    // against 4.5), and more than 384 pieces on four or five (6144 x 64 x 1024: 3.9 here against 3.3)
-    // (up to four tile rows and 512 pieces as well: the 784 -> 4096 layer of an MLP at batch 128, sign bits out, is
-    // 1.4 us faster here than on 32 x 128 tiles)
-    if (row_tiles(N) > 2) return row_tiles(N) <= 4 && pieces <= 512;
+    if (planes == 2) return pieces <= 512 || (NT <= 2 && pieces <= 1024);
+    if (NT > 2) return NT <= 4 && pieces <= 512;      // (an MLP's first layer at batch 128)
     return pieces <= 1024 && (KT >= 6 || pieces > 384);
 }
 
@@ -874,11 +851,9 @@ static int launch_splitk_quad(const GemmArgs& a, hipStream_t st)
     if (gy > 65535 || a.batch > 65535)
         return fail(BGEMM_EINVAL, "gemm_skinny: grid of %lld x %lld x %lld blocks", (long long)gx, (long long)gy, (long long)a.batch);
     // K ways per block.  The kernel's registers allow two waves a SIMD, eight a CU: eight ways are one block a CU, which is
-    // what up to 256 blocks want; beyond that every block more on a CU is a round more, and four ways (two blocks a CU,
-    // each wave on twice the K range, half as many meetings in LDS and store loops per unit of work) are 15 to 25 %
-    // faster (8192 x 160 ternary rows x 8192, 640 blocks: 15.9 against 19.0 us; 11008 x 192 x 8192, 1032 blocks: 24.5 against
-    // 31.3; 8192 x 384 x 16384 sign rows, 768 blocks: 26.9 against 33.5).  Two ways where four blocks a CU are one full round
-    // (769 to 1024 blocks: 8192 x 512 x 16384 31.9 against 33.8 on four ways).
+    // what up to 256 blocks want; beyond that every block more on a CU is a round more, and four ways (two blocks a CU, each
+    // wave on twice the K range, half as many meetings in LDS and store loops per unit of work) are faster; two ways where
+    // four blocks a CU are one full round (769 to 1024 blocks).
     const int64_t blocks = gx * gy * a.batch;
     int kw = blocks <= 256 ? 8 : blocks > 768 && blocks <= 1024 ? 2 : 4;
     while (kw > 1 && kw > a.KT) kw /= 2;
@@ -904,7 +879,7 @@ static int launch_splitk(const GemmArgs& a, hipStream_t st)
     while (kw < 8 && (kw < a.splitK || blocks * groups * kw < 4096) && kw * 2 <= a.KT) kw *= 2;
     const dim3 g((unsigned)a.MT, (unsigned)groups, (unsigned)a.batch);
     // few row tiles against a long K (W[4096,11008]: 128 blocks): eight ways leave under two waves a SIMD, each on
-    // a long serial range; sixteen ways are 5 % faster there (4.7 -> 4.5 us at one row, 5.2 -> 4.9 at sixteen)
+    // a long serial range; sixteen ways are faster there
     if (!pl2 && kw == 8 && blocks * groups * 8 < 2048 && a.KT >= 32) {
         hipLaunchKernelGGL((gemm_skinny_splitk_kernel<Eng, 16>), g, dim3(1024), 0, st, a);
         return check_launch("gemm_skinny");
@@ -943,8 +918,7 @@ static int launch_popc(const GemmArgs& a, hipStream_t st)
 
 // One or two vectors (rows x bit planes), packed or not.  From three on the matrix-core kernels are faster:
 // with unpacked activations every further row costs this kernel about a microsecond (all waves of the grid
-// fetch the same few lines of the row at once), timed on W[11008,4096], popcount / matrix cores: one sign row
-// 4.1 / 5.5 us, two 5.1 / 5.6, three 6.7 / 5.9; one ternary row 4.4 / 5.8, two 5.9 / 5.8.
+// fetch the same few lines of the row at once).
 template <bool FUSEX>
 static bool launch_popc_for(const GemmArgs& a, hipStream_t st, int* rc)
 {
