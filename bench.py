@@ -394,6 +394,9 @@ def bench_mfma_peak(cold):
             ops = 2.0 * 32 * 32 * (64 if fp4 else 32) * 8 * iters * 4 * blocks
             key = ("fp4" if fp4 else "int8") + ("_tops" if valu == 0 else "_tops_with_%d_valu_per_mfma" % valu)
             res[key] = round(ops / ms / 1e9, 1)
+    # expansions shared between the waves of a block through LDS: half the vector instructions, plus the LDS traffic
+    ms = time_gpu(lambda i: L.bench_probe_mfma(1, -1, blocks, iters, out.data_ptr(), st()), 20, 100)
+    res["fp4_tops_with_2_valu_and_shared_fragments_through_lds"] = round(2.0 * 32 * 32 * 64 * 8 * iters * 4 * blocks / ms / 1e9, 1)
     res["fp4_frac_of_datasheet"] = round(res["fp4_tops"] / FP4_MFMA_PEAK_TOPS, 4)
     res["int8_frac_of_datasheet"] = round(res["int8_tops"] / INT8_MFMA_PEAK_TOPS, 4)
     return res

@@ -85,6 +85,51 @@ __global__ __launch_bounds__(256) void probe_mfma_kernel(unsigned* out, const in
 }  // namespace
 
 // All return 0, -1 for bad arguments, or the hipError_t of the launch.
+// What sharing expanded fragments through LDS would make of the 256 x 128 tile's loop: per MFMA two vector-ALU
+// instructions (half of today's expansion: every fragment expanded once per block instead of once per wave that needs it)
+// plus the traffic that replaces the other half: of a K-tile's 32 MFMAs a wave, 24 ds_read_b128 (its six fragments x four
+// steps) and 12 ds_write_b128 (its quarter of the block's twelve fragments), i.e. three reads and one and a half writes per
+// four MFMAs.  Same accumulators, grid and launch bounds as the MFMA-only probe.
+__global__ __launch_bounds__(256) void probe_mfma_lds_kernel(unsigned* out, const int iters)
+{
+    __shared__ uint4 s[4][8][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    unsigned m[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) m[i] = threadIdx.x * 2654435761u + i;
+#pragma unroll
+    for (int i = 0; i < 8; i++) s[wave][i][lane] = make_uint4(m[0], m[1], m[2], m[3]);
+    __syncthreads();
+    v16f acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) acc[i][v] = 0;
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const v8i a = {(int)(m[0] & 0x22222222u), (int)(m[1] & 0x22222222u), (int)(m[2] & 0x22222222u), (int)(m[3] & 0x22222222u), 0, 0, 0, 0};
+            const v8i b = {(int)(m[4] & 0x22222222u), (int)(m[5] & 0x22222222u), (int)(m[6] & 0x22222222u), (int)(m[7] & 0x22222222u), 0, 0, 0, 0};
+            acc[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[i], 4, 4, 0, 0, 0, 0);
+            if ((i & 3) != 3) {                                  // three reads per four MFMAs: another wave's fragment
+                const uint4 r = s[(wave + 1) & 3][i][lane];
+                m[(i & 1) * 4 + 0] ^= r.x; m[(i & 1) * 4 + 1] ^= r.y; m[(i & 1) * 4 + 2] ^= r.z; m[(i & 1) * 4 + 3] ^= r.w;
+            }
+            if ((i & 3) == 1 || (i & 7) == 3)                    // one and a half writes per four MFMAs: this wave's own
+                s[wave][i][lane] = make_uint4(m[0] + it, m[1], m[2], m[3]);
+            m[i] = (m[i] >> 1) ^ (it + i);                       // the two vector-ALU instructions that stay
+            m[(i + 3) & 7] = (m[(i + 3) & 7] >> 1) ^ it;
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    unsigned sum = 0;
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) sum += (unsigned)acc[i][v];
+    out[(size_t)blockIdx.x * 256 + threadIdx.x] = sum;
+}
+
 // `rounds` all-to-all exchanges among the blocks of the grid: every round, every block stores `units` 8-byte
 // {tag, payload} units with device-scope stores into each of `copies` replicas and then polls every unit of replica
 // blockIdx % copies until it carries the round's tag.  Waits are bounded (0.2 s of the 100 MHz wall clock); a block
@@ -141,7 +186,8 @@ extern "C" int bench_probe_exchange(void* buf, int blocks, int units, int copies
 
 // One launch of `blocks` blocks of four waves, each wave issuing iters * 8 MFMAs (fp4 != 0:
 // v_mfma_f32_32x32x64_f8f6f4 with E2M1 operands, 2 * 32 * 32 * 64 ops each; else v_mfma_i32_32x32x32_i8,
-// 2 * 32 * 32 * 32 ops each) with `valu` in {0, 2, 4} vector-ALU instructions after every one.
+// 2 * 32 * 32 * 32 ops each) with `valu` in {0, 2, 4} vector-ALU instructions after every one; fp4 with valu = -1: two
+// vector-ALU instructions and the LDS traffic of fragments shared between the waves of a block (probe_mfma_lds_kernel).
 // out: blocks * 256 words.
 extern "C" int bench_probe_mfma(int fp4, int valu, int blocks, int iters, void* out, void* stream)
 {
@@ -149,7 +195,8 @@ extern "C" int bench_probe_mfma(int fp4, int valu, int blocks, int iters, void* 
     const dim3 g(blocks), b(256);
     hipStream_t st = (hipStream_t)stream;
     unsigned* o = (unsigned*)out;
-    if (fp4) {
+    if (fp4 && valu == -1) hipLaunchKernelGGL(probe_mfma_lds_kernel, g, b, 0, st, o, iters);      // fragments shared through LDS
+    else if (fp4) {
         if (valu == 0) hipLaunchKernelGGL((probe_mfma_kernel<true, 8, 0>), g, b, 0, st, o, iters);
         else if (valu == 2) hipLaunchKernelGGL((probe_mfma_kernel<true, 8, 2>), g, b, 0, st, o, iters);
         else if (valu == 4) hipLaunchKernelGGL((probe_mfma_kernel<true, 8, 4>), g, b, 0, st, o, iters);
