@@ -146,14 +146,29 @@ __global__ __launch_bounds__(512) void probe_exchange_kernel(unsigned long long*
             __hip_atomic_store(&cur[(size_t)(i / units) * stride + b * units + i % units],
                                ((unsigned long long)tag << 32) | (unsigned)(b * 131 + i % units + r), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         const unsigned long long* mine = cur + (size_t)(b % copies) * stride;
+        // a thread asks for all of its units that are still missing in every round of loads (up to four units a thread)
         int bad = 0;
-        for (int i = t; i < U && !bad; i += 512) {
-            unsigned long long v = __hip_atomic_load(&mine[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            for (unsigned tries = 1; (unsigned)(v >> 32) != tag; tries++) {
-                if ((tries & 63) == 0 && wall_clock64() - t0 > 20000000ll) { bad = 1; break; }
-                v = __hip_atomic_load(&mine[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int base = t; base < U && !bad; base += 4 * 512) {
+            unsigned pending = 0;
+#pragma unroll
+            for (int c = 0; c < 4; c++)
+                if (base + c * 512 < U) pending |= 1u << c;
+            for (unsigned tries = 1; pending; tries++) {
+                unsigned long long v[4];
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    v[c] = 0;
+                    if (pending >> c & 1) v[c] = __hip_atomic_load(&mine[base + c * 512], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+#pragma unroll
+                for (int c = 0; c < 4; c++)
+                    if ((pending >> c & 1) && (unsigned)(v[c] >> 32) == tag) {
+                        const int i = base + c * 512;
+                        if ((unsigned)v[c] != (unsigned)((i / units) * 131 + i % units + r)) atomicAdd(err + 1, 1ull);
+                        pending &= ~(1u << c);
+                    }
+                if (pending && (tries & 63) == 0 && wall_clock64() - t0 > 20000000ll) { bad = 1; break; }
             }
-            if (!bad && (unsigned)v != (unsigned)((i / units) * 131 + i % units + r)) atomicAdd(err + 1, 1ull);
         }
         if (__syncthreads_or(bad)) { if (t == 0) atomicAdd(err, 1ull); return; }
     }

@@ -62,35 +62,36 @@ __device__ __forceinline__ void unit_store(unsigned long long* p, const unsigned
     __hip_atomic_store(p, ((unsigned long long)tag << 32) | word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Polls units u0, u0 + stride, ... below U of `src` until each carries `tag` and hands (u, word) to `sink`.
-// CHAIN_POLL_CH loads are in flight per thread.  Returns false when the budget ran out.
+// Polls units u0, u0 + stride, ... below U of `src` until each carries `tag` and hands (u, word) to `sink`.  A thread
+// takes CHAIN_POLL_CH units at a time and asks for ALL of them that are still missing in every round of loads, so a round
+// trip through the memory fabric is paid once per round and not once per unit.  Returns false when the budget ran out (the
+// wall clock is a slow read: looked at once in 64 rounds).
 template <typename Sink>
 __device__ __forceinline__ bool poll_units(const unsigned long long* src, const int u0, const int stride, const int U, const unsigned tag,
                                            const long long t0, const long long budget, Sink sink)
 {
-    bool ok = true;
-    for (int base = u0; base < U && ok; base += CHAIN_POLL_CH * stride) {
-        unsigned long long v[CHAIN_POLL_CH];
+    for (int base = u0; base < U; base += CHAIN_POLL_CH * stride) {
+        unsigned pending = 0;
 #pragma unroll
-        for (int c = 0; c < CHAIN_POLL_CH; c++) {
-            const int u = base + c * stride;
-            v[c] = 0;
-            if (u < U) v[c] = unit_load(src + u);
-        }
+        for (int c = 0; c < CHAIN_POLL_CH; c++)
+            if (base + c * stride < U) pending |= 1u << c;
+        for (unsigned tries = 1; pending; tries++) {
+            unsigned long long v[CHAIN_POLL_CH];
 #pragma unroll
-        for (int c = 0; c < CHAIN_POLL_CH; c++) {
-            const int u = base + c * stride;
-            if (u >= U) continue;
-            // (the wall clock is a slow read: looked at once in 64 tries)
-            for (unsigned tries = 1; (unsigned)(v[c] >> 32) != tag; tries++) {
-                if ((tries & 63u) == 0 && wall_clock64() - t0 > budget) { ok = false; break; }
-                v[c] = unit_load(src + u);
+            for (int c = 0; c < CHAIN_POLL_CH; c++) {
+                v[c] = 0;
+                if (pending >> c & 1) v[c] = unit_load(src + base + c * stride);
             }
-            if (!ok) break;
-            sink(u, (unsigned)v[c]);
+#pragma unroll
+            for (int c = 0; c < CHAIN_POLL_CH; c++)
+                if ((pending >> c & 1) && (unsigned)(v[c] >> 32) == tag) {
+                    sink(base + c * stride, (unsigned)v[c]);
+                    pending &= ~(1u << c);
+                }
+            if (pending && (tries & 63u) == 0 && wall_clock64() - t0 > budget) return false;
         }
     }
-    return ok;
+    return true;
 }
 
 template <int NTM, int KSM, bool F32>
@@ -490,7 +491,7 @@ extern "C" int bgemm_chain_forward(int mode, const bgemm_chain_layer* layers, co
     a.state = (unsigned*)ws;
     a.xg = (unsigned long long*)((char*)ws + 256);
     // one level up to a few hundred units a layer (every block pulls every unit through the fabric), two beyond
-    const bool two_level = G % 8 == 0 && (levels == 2 || (levels == 0 && cs.u_max > 1024));
+    const bool two_level = G % 8 == 0 && (levels == 2 || (levels == 0 && cs.u_max > 4096));
     a.xl = two_level ? a.xg + (size_t)2 * cs.u_max : nullptr;
     a.u_max = cs.u_max; a.kt_max = cs.kt_max;
     a.trace = (flags & 4) ? (long long*)((char*)ws + 256 + (size_t)18 * cs.u_max * 8) : nullptr;
