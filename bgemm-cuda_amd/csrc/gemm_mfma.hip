@@ -765,7 +765,8 @@ static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int pla
     const bool last_round_idle = KT >= 8 && (KT <= 16 || b21 <= 600) && b21 > 256 &&
                                  round_fill(b11, 768) >= round_fill(b21, 512) + 0.15 && filled(128, 128) >= 0.6;
     const bool few_blocks_ok = KT >= 16 && b21 >= 132 && (b21 < 192 || KT >= 24) && !(b21 > 256 && b21 <= 384);
-    const bool k_long_enough = KT >= 8 || (out_shift == 2 && KT >= 4 && out_elems >= (64 << 20)) || b11 < 512;
+    // (on 8 to 11 K-tiles the smaller tile's extra blocks hide more of the stores than its dearer loop costs)
+    const bool k_long_enough = KT >= 12 || (out_shift == 2 && KT >= 4 && out_elems >= (64 << 20)) || b11 < 512;
     if (planes == 1 && !last_round_idle && (b21 >= 512 || few_blocks_ok) && k_long_enough && filled(256, 128) >= 0.75)
         return {BGEMM_KERNEL_MFMA_256x128, 256, 128};
     // 128 x 128: two rounds' worth of blocks, or (one plane, pipelined loop) from 192 / 144 blocks, not where some units
