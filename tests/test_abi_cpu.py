@@ -319,3 +319,21 @@ def test_shim_checks_buffers_before_the_kernel_sees_them(monkeypatch):
             lk.bgemm_packed_forward(bad, x)
     with pytest.raises(ValueError):
         lk.bgemm_packed_forward(w, lk.PackedBits(x.data, torch.zeros((1, 256), dtype=torch.int32), 1, 7, 300), _lib.MODE_BWTA)
+
+
+def test_chain_entry_point_rejects_bad_arguments_on_the_host():
+    """bgemm_chain_forward checks its arguments before anything touches a GPU (tests/python/bgemm_linear.py:474-486 is the
+    stack of layers it runs; the reference's own launcher asserts and aborts instead, fp6_linear.cu:288-290)."""
+    L = _lib.lib()
+    layers = (_lib.ChainLayer * 2)()
+    for l, (M, K) in enumerate(((512, 256), (64, 512))):
+        layers[l].W_tiled, layers[l].sw, layers[l].sa, layers[l].M, layers[l].K = 4096, 4096, 4096, M, K
+    call = lambda mode=1, lay=layers, n=2, N=4, out_dtype=0, param=0: L.bgemm_chain_forward(
+        mode, lay, 4096, n, 4096, 4096, N, 4096, out_dtype, param, 4096, 1 << 20, 0, None)
+    assert call(mode=9) == _lib.EINVAL
+    assert call(lay=None) == _lib.ENULL
+    assert call(n=0) == _lib.EINVAL and call(n=200) == _lib.EINVAL
+    assert call(N=0) == _lib.EINVAL and call(N=33) == _lib.EINVAL and call(mode=3, N=17) == _lib.EINVAL
+    assert b"activation rows" in L.bgemm_last_error()
+    assert L.bgemm_chain_workspace_bytes(9, layers, 2, 4) == 0
+    assert L.bgemm_chain_status(None, None) == _lib.ENULL
