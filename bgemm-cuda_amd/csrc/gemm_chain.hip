@@ -50,6 +50,7 @@ struct ChainArgs {
     long long* trace;                         // null, or [1 + 5 * n_layers] wall-clock stamps written by thread 0 of block 0: start; per layer
                                               // operand in LDS, next layer requested, own K-tiles done, partial sums met, outputs published
     long long budget;                         // ticks of the 100 MHz wall clock a wait may take, from the kernel's start
+    int mute_block0;                          // test hook: block 0 publishes nothing, so every wait for it runs out of budget
     unsigned e_magic;                         // ceil(2^32 / E), E = planes * N units per word (unused for E = 1)
 };
 
@@ -320,7 +321,7 @@ __global__ __launch_bounds__(CHAIN_THREADS, 1) void gemm_chain_kernel(const Chai
                 }
                 const unsigned long long bs = __ballot(sg != 0 && (!two || nz != 0)), bz = __ballot(nz != 0);
                 const unsigned ws = __brev((unsigned)(lane < 32 ? bs : bs >> 32)), wz = __brev((unsigned)(lane < 32 ? bz : bz >> 32));
-                if (c == 0 && valid) {
+                if (c == 0 && valid && !(a.mute_block0 && b == 0)) {
                     const int jw = b + i * G;
                     if (two) {
                         unit_store(pub + (jw * 2 + 0) * N + nl, tag, wz);
@@ -481,7 +482,7 @@ extern "C" int bgemm_chain_forward(int mode, const bgemm_chain_layer* layers, co
         if (scaled && (!layers[l].sw || !layers[l].sa)) return fail(BGEMM_ENULL, "bgemm_chain_forward: layer %d has no sw or sa", l);
     }
     const int levels = flags & 3;
-    if (levels == 3 || (flags & 0xf8)) return fail(BGEMM_EINVAL, "bgemm_chain_forward: flags");
+    if (levels == 3 || (flags & 0xf0)) return fail(BGEMM_EINVAL, "bgemm_chain_forward: flags");
     ChainArgs a;
     memset(&a, 0, sizeof a);
     a.layers = (const ChainLayerDev*)layers_dev; a.n_layers = n_layers;
@@ -496,6 +497,7 @@ extern "C" int bgemm_chain_forward(int mode, const bgemm_chain_layer* layers, co
     a.u_max = cs.u_max; a.kt_max = cs.kt_max;
     a.trace = (flags & 4) ? (long long*)((char*)ws + 256 + (size_t)18 * cs.u_max * 8) : nullptr;
     a.budget = 25000000LL;          // a quarter of a second
+    if (flags & 8) { a.mute_block0 = 1; a.budget = 100000LL; }      // (tests of the time-out path: a millisecond)
     const unsigned E = (unsigned)(mc.planes * N);
     a.e_magic = E > 1 ? (unsigned)(((1ULL << 32) + E - 1) / E) : 0;
     const bool f32 = param_dtype == BGEMM_SRC_F32;
@@ -505,7 +507,7 @@ extern "C" int bgemm_chain_forward(int mode, const bgemm_chain_layer* layers, co
     return f32 ? chain_launch<2, 6, true>(a, G, st) : chain_launch<2, 6, false>(a, G, st);
 }
 
-extern "C" int bgemm_chain_status(const void* ws, void* stream)
+extern "C" int bgemm_chain_status(void* ws, void* stream)
 {
     if (!ws) return fail(BGEMM_ENULL, "bgemm_chain_status: ws is NULL");
     unsigned st[4] = {0, 0, 0, 0};
@@ -513,7 +515,13 @@ extern "C" int bgemm_chain_status(const void* ws, void* stream)
         (void)hipGetLastError();
         return fail(BGEMM_ELAUNCH, "bgemm_chain_status: cannot read the workspace");
     }
-    if (st[2]) return fail(BGEMM_ETIMEOUT, "bgemm_chain: a block waited longer than its budget for the layer before it "
-                                          "(calls that share a GPU at the same time can starve each other of compute units)");
+    if (st[2]) {
+        // reported once: the word is cleared so that the workspace can be used again
+        const unsigned zero = 0;
+        if (hipMemcpyAsync((char*)ws + 8, &zero, 4, hipMemcpyHostToDevice, (hipStream_t)stream) != hipSuccess || hipStreamSynchronize((hipStream_t)stream) != hipSuccess)
+            (void)hipGetLastError();
+        return fail(BGEMM_ETIMEOUT, "bgemm_chain: a block waited longer than its budget for the layer before it "
+                                    "(calls that share a GPU at the same time can starve each other of compute units)");
+    }
     return BGEMM_OK;
 }

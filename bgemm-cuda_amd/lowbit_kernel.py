@@ -429,7 +429,7 @@ class DecodeChain:
         if ws is None:
             need = _b.lib().bgemm_chain_workspace_bytes(self.mode, self._host, len(self.layers), N)
             if need == 0:
-                _b.check(_b.EINVAL if not _b.lib().bgemm_last_error() else _b.EINVAL)
+                _b.check(_b.EINVAL)          # the library has recorded why the chain cannot run
             ws = torch.zeros(need, dtype=torch.uint8, device=self.device)
             self._ws[N] = ws
         return ws

@@ -298,7 +298,7 @@ int bgemm_f16_forward_static(const void* W, const void* X, void* C, int64_t M, i
  * Layers of up to 3 row tiles a block with K <= 4096, 2 with K <= 12288, 1 with K <= 16384 (a row tile is
  * 32 rows; blocks = compute units); others return BGEMM_EINVAL.  A block that waits longer than a quarter of
  * a second for its predecessors gives up; bgemm_chain_status() (synchronises the stream) then returns
- * BGEMM_ETIMEOUT and the output is undefined. */
+ * BGEMM_ETIMEOUT once (it clears the mark, the workspace stays usable) and that call's output is undefined. */
 typedef struct bgemm_chain_layer {
     const void* W_tiled;
     const void* sw;
@@ -312,7 +312,7 @@ size_t bgemm_chain_workspace_bytes(int mode, const bgemm_chain_layer* layers, in
 int bgemm_chain_forward(int mode, const bgemm_chain_layer* layers, const void* layers_dev, int n_layers,
                         const void* X_tiled, const void* X2_tiled, int64_t N, void* out, int out_dtype,
                         int param_dtype, void* ws, size_t ws_bytes, int flags, void* stream);
-int bgemm_chain_status(const void* ws, void* stream);
+int bgemm_chain_status(void* ws, void* stream);
 
 #ifdef __cplusplus
 }

@@ -145,3 +145,27 @@ def test_chain_rejects_what_it_cannot_run():
         device_chain(MODE_XOR, bad, None, 0)(lk.pack_sign(to_dev(rng.standard_normal((4, 256)).astype(np.float16))))
     with pytest.raises(ValueError):          # K beyond one block's LDS operand
         device_chain(MODE_XOR, make_chain(rng, [32768, 64], np.float16), None, 0)(lk.pack_sign(to_dev(rng.standard_normal((4, 32768)).astype(np.float16))))
+
+
+def test_a_wait_that_runs_out_of_budget_ends_the_launch_and_is_reported(oracle):
+    """The time-out path, forced from the host: with flags & 8 the first block publishes nothing and the budget is a
+    millisecond, so every block gives up waiting for it and leaves (no wave spins on); the status call reports it once,
+    and the same workspace then runs the chain correctly."""
+    import _lib
+    rng = np.random.default_rng(11)
+    layers = make_chain(rng, [512, 2048, 512], np.float16)
+    x = rng.standard_normal((4, 512)).astype(np.float16)
+    want = oracle_chain(oracle, MODE_XOR, layers, x, "i32")
+    chain = device_chain(MODE_XOR, layers, torch.int32, 0)
+    xp = lk.pack_sign(to_dev(x))
+    assert same(chain(xp), want)
+    chain.check(4)
+    chain.flags = 8
+    chain(xp)
+    with pytest.raises(_lib.BgemmError, match="budget"):
+        chain.check(4)
+    chain.flags = 0
+    chain.check(4)                      # reported once
+    for rep in range(2):
+        assert same(chain(xp), want)
+        chain.check(4)
