@@ -46,6 +46,11 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+def log_row(r):
+    """Progress on stderr: the row's id, time and whether it was bit-exact (the whole row is in the final line)."""
+    log("%s: %s us%s" % (r.get("id", r.get("shape", "")), r.get("us", ""), "" if r.get("ok", True) else "  NOT BIT-EXACT"))
+
+
 def measured_traffic_bytes():
     """HBM bytes per launch of the headline kernel as the tracked profile summary states them (a line
     `traffic_bytes_per_launch = N` under the FETCH_SIZE / WRITE_SIZE counter runs), or None."""
@@ -237,7 +242,7 @@ def bench_sweep(steps=40, warmup=5):
         r4, _ = bench_c5(steps, warmup, 8192, N, K, 4)
         rows.append(row("C5 sweep 8192x%dx%d" % (N, K), r1["ms"], r1["ops"], r1["bytes"],
                         r1["bit_exact"] and r4["bit_exact"], r1["kernel"], "mfma", us_splitK4=round(r4["ms"] * 1e3, 2)))
-        log(json.dumps(rows[-1]))
+        log_row(rows[-1])
     return rows
 
 
@@ -429,7 +434,7 @@ def bench_decode(cold, name, M, K, Ns, steps=640, total_mb=361):
         rows.append(row("%s W[%d,%d] N=%d 1 launch cold" % (name, M, K, N), ms, 2.0 * M * N * K, bytes_alg, ok,
                         kernel_of(wps[0], xt, lk.MODE_BWTA, 8), "hbm", cold_read_us=round(floor_us, 2),
                         x_cold_read=round(ms * 1e3 / floor_us, 2)))
-        log(json.dumps(rows[-1]))
+        log_row(rows[-1])
     return rows
 
 
@@ -518,7 +523,7 @@ def bench_chain(cold, Ns=(1, 4, 16), blocks=32, replays=6):
         floor_us = cold.us(wbytes)
         rows.append(row("C4 chain of %d dependent layers up/down W[11008,4096] N=%d, per layer" % (L, N), ms, 2.0 * 11008 * 4096 * N, bytes_alg, ok,
                         "chain", "hbm", cold_read_us=round(floor_us, 2), x_cold_read=round(ms * 1e3 / floor_us, 2), us_whole_chain=round(ms * L * 1e3, 1)))
-        log(json.dumps(rows[-1]))
+        log_row(rows[-1])
     return rows
 
 
@@ -717,14 +722,14 @@ def section_decode(cold):
     rows = bench_decode(cold, "C4", 11008, 4096, (1, 4, 16))
     for N in (1, 4, 16):
         rows.append(bench_decode_batched(N))
-        log(json.dumps(rows[-1]))
+        log_row(rows[-1])
     # the GEMMs a Llama-7B decode step issues against one set of activations: QKV fused, gate + up fused, down
     rows += bench_decode(cold, "QKV", 12288, 4096, (1, 4, 16))
     rows += bench_decode(cold, "gate+up", 22016, 4096, (1, 4, 16))
     rows += bench_decode(cold, "down", 4096, 11008, (1, 4, 16))
     for N in (1, 4):
         rows.append(bench_decode_from_fp16(N))
-        log(json.dumps(rows[-1]))
+        log_row(rows[-1])
     rows += bench_chain(cold)
     return rows
 
@@ -750,7 +755,7 @@ def bench_prefill(steps=20, warmup=5):
                 M * K / 8 + 2 * N * K / 8 + 4.0 * M * N, ok, kernel_of(wp, xt, lk.MODE_BWTA), "mfma")
         r["frac"] = round(2 * r["tops"] / FP4_MFMA_PEAK_TOPS, 4)       # matrix-core work is two products a weight expansion: 4*M*N*K
         rows.append(r)
-        log(json.dumps(r))
+        log_row(r)
         del w16, x16, wp, xt, out
     # batches of decode steps: a few hundred ternary rows against one layer, weights rotating through HBM as a model's do
     for name, M, N, K in (("up", 11008, 128, 4096), ("gate+up", 22016, 128, 4096), ("down", 4096, 128, 11008), ("up", 11008, 512, 4096)):
@@ -768,23 +773,23 @@ def bench_prefill(steps=20, warmup=5):
         r["frac"] = round(2 * r["tops"] / FP4_MFMA_PEAK_TOPS, 4)       # 4*M*N*K of matrix-core work, as above
         r["frac_hbm"] = round(r["gbs"] / HBM_PEAK_GBS, 4)
         rows.append(r)
-        log(json.dumps(r))
+        log_row(r)
         del w16, x16, wps, xt, out
     return rows
 
 
 def all_configs(cold):
     rows = [bench_c2()]
-    log(json.dumps(rows[-1]))
+    log_row(rows[-1])
     rows.append(bench_c3())
-    log(json.dumps(rows[-1]))
+    log_row(rows[-1])
     rows.append(bench_qk())
-    log(json.dumps(rows[-1]))
+    log_row(rows[-1])
     rows += section_decode(cold)
     rows += bench_sweep()
     rows += bench_prefill()
     rows.append(bench_c5_dropin(20, 3))
-    log(json.dumps(rows[-1]))
+    log_row(rows[-1])
     return rows
 
 
@@ -837,18 +842,18 @@ def main():
     if not args.headline_only:
         cold = ColdRead()
         floor = bench_floor(cold)
-        log("floor:", json.dumps(floor))
+        log("floor done")
         peak_measured = bench_mfma_peak(cold)
-        log("mfma peak:", json.dumps(peak_measured))
+        log("mfma peak done")
         extra = all_configs(cold)
         dispatch = dispatch_summary(bench_thresholds(40, DISPATCH_SHAPES, warm=False))
-        log("dispatch:", json.dumps(dispatch))
+        log("dispatch done")
         del cold
         torch.cuda.empty_cache()
 
     c5, (w16, x16) = bench_c5(args.steps, args.warmup, splitK=args.split_k, variant=args.variant, pre_roll=args.pre_roll,
                                   counted=args.counted)
-    log("C5:", json.dumps(c5))
+    log("C5: %.5f ms" % c5["ms"])
     cpu = None if args.no_cpu else cpu_baseline_c5(w16, x16)
     del w16, x16
     fp4 = args.variant in (0, 3)
