@@ -385,22 +385,33 @@ def bench_floor(cold):
 
 def bench_mfma_peak(cold):
     """The matrix cores alone: v_mfma_f32_32x32x64_f8f6f4 (E2M1 operands) and v_mfma_i32_32x32x32_i8 from two waves
-    per SIMD with eight independent accumulators each, no memory traffic; then with two and four independent vector-ALU
-    instructions after every MFMA (what the bit expansion adds to the issue stream).  20 warm-up + 100 timed launches."""
+    per SIMD with eight independent accumulators each, no memory traffic; then with a number of independent vector-ALU
+    instructions after every MFMA (what the bit expansion adds to the issue stream: the probe's loop holds exactly that
+    many v_and_b32 per MFMA).  20 warm-up + 100 timed launches."""
     import torch
     L = cold.L
     out = torch.empty(512 * 256, dtype=torch.int32, device="cuda:0")
     st = lambda: torch.cuda.current_stream().cuda_stream
     iters, blocks = 2000, 512
     res = {}
+
+    def probe(fp4, valu):
+        rc = L.bench_probe_mfma(fp4, valu, blocks, iters, out.data_ptr(), st())
+        if rc != 0:
+            raise RuntimeError("bench_probe_mfma(%d, %d) -> %d: libbench_probes.so is older than bench_probes.hip?" % (fp4, valu, rc))
+
     for fp4 in (1, 0):
-        for valu in (0, 2, 4):
-            ms = time_gpu(lambda i: L.bench_probe_mfma(fp4, valu, blocks, iters, out.data_ptr(), st()), 20, 100)
+        for valu in ((0, 1, 2, 3, 4, 5, 6, 8) if fp4 else (0, 4, 8)):
+            ms = time_gpu(lambda i: probe(fp4, valu), 20, 100)
             ops = 2.0 * 32 * 32 * (64 if fp4 else 32) * 8 * iters * 4 * blocks
             key = ("fp4" if fp4 else "int8") + ("_tops" if valu == 0 else "_tops_with_%d_valu_per_mfma" % valu)
             res[key] = round(ops / ms / 1e9, 1)
-    # expansions shared between the waves of a block through LDS: half the vector instructions, plus the LDS traffic
-    ms = time_gpu(lambda i: L.bench_probe_mfma(1, -1, blocks, iters, out.data_ptr(), st()), 20, 100)
+    # the same with an instruction that reads two vector registers (v_perm_b32) instead of one (v_and_b32)
+    for valu in (2, 4):
+        ms = time_gpu(lambda i: probe(1, 100 + valu), 20, 100)
+        res["fp4_tops_with_%d_two_register_valu_per_mfma" % valu] = round(2.0 * 32 * 32 * 64 * 8 * iters * 4 * blocks / ms / 1e9, 1)
+    # expansions shared between the waves of a block through LDS: the loop with two v_and_b32 per MFMA plus the LDS traffic
+    ms = time_gpu(lambda i: probe(1, -1), 20, 100)
     res["fp4_tops_with_2_valu_and_shared_fragments_through_lds"] = round(2.0 * 32 * 32 * 64 * 8 * iters * 4 * blocks / ms / 1e9, 1)
     res["fp4_frac_of_datasheet"] = round(res["fp4_tops"] / FP4_MFMA_PEAK_TOPS, 4)
     res["int8_frac_of_datasheet"] = round(res["int8_tops"] / INT8_MFMA_PEAK_TOPS, 4)

@@ -44,61 +44,78 @@ __global__ __launch_bounds__(512) void probe_read_kernel(const uint4* __restrict
     if (acc == 0x12345678u && out == reinterpret_cast<unsigned*>(1)) out[0] = acc;
 }
 
-// NACC independent accumulators per wave keep the matrix pipe full; VALU masks of live registers after
-// every MFMA stand in for the bit expansion (their results feed the next round's operands, so they stay).
-template <bool FP4, int NACC, int VALU>
-__global__ __launch_bounds__(256) void probe_mfma_kernel(unsigned* out, const int iters)
+// NACC independent accumulators per wave keep the matrix pipe full.  The MFMAs read two sets of eight operand
+// registers in turn, and after every MFMA exactly VALU vector-ALU instructions rewrite registers of the set it has just
+// read, which the MFMA after next reads: as in the software-pipelined bit expansion, no MFMA waits for a register
+// written just before it.  PERM: each is a v_perm_b32 (two vector registers and a scalar read); else a v_and_b32 of a
+// vector register with a scalar, the form of most of the expansion.  The count per MFMA in the generated loop is VALU.
+template <bool FP4, int NACC, int VALU, bool PERM>
+__global__ __launch_bounds__(256) void probe_mfma_kernel(unsigned* out, const int iters, const unsigned seed)
 {
-    unsigned m[8];
+    unsigned raw[8], op[16];
 #pragma unroll
-    for (int i = 0; i < 8; i++) m[i] = threadIdx.x * 2654435761u + i;
+    for (int i = 0; i < 16; i++) {
+        if (i < 8) raw[i] = threadIdx.x * 2654435761u + i * 0x9e3779b9u + seed;
+        op[i] = (threadIdx.x * 40503u + i) & (FP4 ? 0x22222222u : 0x01010101u);
+    }
     typename std::conditional<FP4, v16f, v16i>::type acc[NACC];
 #pragma unroll
     for (int i = 0; i < NACC; i++)
 #pragma unroll
         for (int v = 0; v < 16; v++) acc[i][v] = 0;
     for (int it = 0; it < iters; it++) {
+        const unsigned sel = 0x07020500u ^ ((seed + it) & 0x03030303u);           // scalar unit; bytes of either source
+        const unsigned msk = (FP4 ? 0x33333333u : 0x01010101u) ^ ((seed + it) & (FP4 ? 0x44444444u : 0x02020202u));
 #pragma unroll
         for (int i = 0; i < NACC; i++) {
+            const int s = (i & 1) * 8;
             if constexpr (FP4) {
-                const v8i a = {(int)(m[0] & 0x22222222u), (int)(m[1] & 0x22222222u), (int)(m[2] & 0x22222222u), (int)(m[3] & 0x22222222u), 0, 0, 0, 0};
-                const v8i b = {(int)(m[4] & 0x22222222u), (int)(m[5] & 0x22222222u), (int)(m[6] & 0x22222222u), (int)(m[7] & 0x22222222u), 0, 0, 0, 0};
+                const v8i a = {(int)op[s + 0], (int)op[s + 1], (int)op[s + 2], (int)op[s + 3], 0, 0, 0, 0};
+                const v8i b = {(int)op[s + 4], (int)op[s + 5], (int)op[s + 6], (int)op[s + 7], 0, 0, 0, 0};
                 acc[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[i], 4, 4, 0, 0, 0, 0);
             } else {
-                const v4i a = {(int)(m[0] & 0x01010101u), (int)(m[1] & 0x01010101u), (int)(m[2] & 0x01010101u), (int)(m[3] & 0x01010101u)};
-                const v4i b = {(int)(m[4] & 0x01010101u), (int)(m[5] & 0x01010101u), (int)(m[6] & 0x01010101u), (int)(m[7] & 0x01010101u)};
+                const v4i a = {(int)op[s + 0], (int)op[s + 1], (int)op[s + 2], (int)op[s + 3]};
+                const v4i b = {(int)op[s + 4], (int)op[s + 5], (int)op[s + 6], (int)op[s + 7]};
                 acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc[i], 0, 0, 0);
             }
 #pragma unroll
-            for (int u = 0; u < VALU; u++) m[(i * VALU + u) & 7] = (m[(i * VALU + u) & 7] >> 1) ^ (it + u);
+            for (int u = 0; u < VALU; u++) {
+                const int j = ((i >> 1) * VALU + u) & 7;
+                if constexpr (PERM) op[s + j] = __builtin_amdgcn_perm(op[s + j], raw[j], sel);
+                else op[s + j] = raw[j] & (msk * (unsigned)(2 * i + 1));                              // the mask: scalar unit
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
     }
-    unsigned s = 0;
+    unsigned sum = 0;
 #pragma unroll
     for (int i = 0; i < NACC; i++)
 #pragma unroll
-        for (int v = 0; v < 16; v++) s += (unsigned)acc[i][v];
-    out[(size_t)blockIdx.x * 256 + threadIdx.x] = s;
+        for (int v = 0; v < 16; v++) sum += (unsigned)acc[i][v];
+    out[(size_t)blockIdx.x * 256 + threadIdx.x] = sum;
 }
 
 }  // namespace
 
 // All return 0, -1 for bad arguments, or the hipError_t of the launch.
-// What sharing expanded fragments through LDS would make of the 256 x 128 tile's loop: per MFMA two vector-ALU
-// instructions (half of today's expansion: every fragment expanded once per block instead of once per wave that needs it)
-// plus the traffic that replaces the other half: of a K-tile's 32 MFMAs a wave, 24 ds_read_b128 (its six fragments x four
-// steps) and 12 ds_write_b128 (its quarter of the block's twelve fragments), i.e. three reads and one and a half writes per
-// four MFMAs.  Same accumulators, grid and launch bounds as the MFMA-only probe.
-__global__ __launch_bounds__(256) void probe_mfma_lds_kernel(unsigned* out, const int iters)
+// What sharing expanded fragments through LDS would make of the 256 x 128 tile's loop, at its most favourable: a wave
+// expands three of its six fragments itself (two vector-ALU instructions per MFMA, half of today's expansion), writes
+// them to LDS for the wave that needs the same ones and reads that wave's three: per step of eight MFMAs three
+// ds_write_b128 and three ds_read_b128 a wave, straight from and into operand registers, and no barrier or flag
+// between writer and reader (a real kernel needs one per K-tile).  Same accumulators, operand sets, grid and launch
+// bounds as probe_mfma_kernel<true, 8, 2, false>, whose loop this is plus the six LDS instructions.
+__global__ __launch_bounds__(256) void probe_mfma_lds_kernel(unsigned* out, const int iters, const unsigned seed)
 {
-    __shared__ uint4 s[4][8][64];
+    __shared__ uint4 sh[4][3][64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    unsigned m[8];
+    unsigned raw[8], op[16];
 #pragma unroll
-    for (int i = 0; i < 8; i++) m[i] = threadIdx.x * 2654435761u + i;
+    for (int i = 0; i < 16; i++) {
+        if (i < 8) raw[i] = threadIdx.x * 2654435761u + i * 0x9e3779b9u + seed;
+        op[i] = (threadIdx.x * 40503u + i) & 0x22222222u;
+    }
 #pragma unroll
-    for (int i = 0; i < 8; i++) s[wave][i][lane] = make_uint4(m[0], m[1], m[2], m[3]);
+    for (int i = 0; i < 3; i++) sh[wave][i][lane] = make_uint4(op[0], op[1], op[2], op[3]);
     __syncthreads();
     v16f acc[8];
 #pragma unroll
@@ -106,19 +123,24 @@ __global__ __launch_bounds__(256) void probe_mfma_lds_kernel(unsigned* out, cons
 #pragma unroll
         for (int v = 0; v < 16; v++) acc[i][v] = 0;
     for (int it = 0; it < iters; it++) {
+        const unsigned msk = 0x33333333u ^ ((seed + it) & 0x44444444u);                 // scalar unit
 #pragma unroll
         for (int i = 0; i < 8; i++) {
-            const v8i a = {(int)(m[0] & 0x22222222u), (int)(m[1] & 0x22222222u), (int)(m[2] & 0x22222222u), (int)(m[3] & 0x22222222u), 0, 0, 0, 0};
-            const v8i b = {(int)(m[4] & 0x22222222u), (int)(m[5] & 0x22222222u), (int)(m[6] & 0x22222222u), (int)(m[7] & 0x22222222u), 0, 0, 0, 0};
+            const int s = (i & 1) * 8;
+            const v8i a = {(int)op[s + 0], (int)op[s + 1], (int)op[s + 2], (int)op[s + 3], 0, 0, 0, 0};
+            const v8i b = {(int)op[s + 4], (int)op[s + 5], (int)op[s + 6], (int)op[s + 7], 0, 0, 0, 0};
             acc[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[i], 4, 4, 0, 0, 0, 0);
-            if ((i & 3) != 3) {                                  // three reads per four MFMAs: another wave's fragment
-                const uint4 r = s[(wave + 1) & 3][i][lane];
-                m[(i & 1) * 4 + 0] ^= r.x; m[(i & 1) * 4 + 1] ^= r.y; m[(i & 1) * 4 + 2] ^= r.z; m[(i & 1) * 4 + 3] ^= r.w;
+            if (i < 6 && (i & 1) == 0) {                          // own fragment: expanded in registers, then published
+#pragma unroll
+                for (int u = 0; u < 4; u++) op[s + u] = raw[u] & (msk * (unsigned)(2 * i + 1));
+                sh[wave][i >> 1][lane] = make_uint4(op[s + 0], op[s + 1], op[s + 2], op[s + 3]);
+            } else if (i < 6) {                                   // the other wave's fragment: read, not expanded
+                const uint4 r = sh[wave ^ 1][i >> 1][lane];
+                op[s + 4] = r.x; op[s + 5] = r.y; op[s + 6] = r.z; op[s + 7] = r.w;
+            } else {                                              // the remaining expansion of the step (16 in all)
+#pragma unroll
+                for (int u = 0; u < 2; u++) op[s + 4 * (i & 1) + u] = raw[4 + u] & (msk * (unsigned)(2 * i + 1));
             }
-            if ((i & 3) == 1 || (i & 7) == 3)                    // one and a half writes per four MFMAs: this wave's own
-                s[wave][i][lane] = make_uint4(m[0] + it, m[1], m[2], m[3]);
-            m[i] = (m[i] >> 1) ^ (it + i);                       // the two vector-ALU instructions that stay
-            m[(i + 3) & 7] = (m[(i + 3) & 7] >> 1) ^ it;
             __builtin_amdgcn_sched_barrier(0);
         }
     }
@@ -201,7 +223,7 @@ extern "C" int bench_probe_exchange(void* buf, int blocks, int units, int copies
 
 // One launch of `blocks` blocks of four waves, each wave issuing iters * 8 MFMAs (fp4 != 0:
 // v_mfma_f32_32x32x64_f8f6f4 with E2M1 operands, 2 * 32 * 32 * 64 ops each; else v_mfma_i32_32x32x32_i8,
-// 2 * 32 * 32 * 32 ops each) with `valu` in {0, 2, 4} vector-ALU instructions after every one; fp4 with valu = -1: two
+// 2 * 32 * 32 * 32 ops each) with `valu` in 0 .. 8 vector-ALU instructions after every one (v_and_b32; 100 + valu, fp4 only: v_perm_b32); fp4 with valu = -1: two
 // vector-ALU instructions and the LDS traffic of fragments shared between the waves of a block (probe_mfma_lds_kernel).
 // out: blocks * 256 words.
 extern "C" int bench_probe_mfma(int fp4, int valu, int blocks, int iters, void* out, void* stream)
@@ -210,17 +232,16 @@ extern "C" int bench_probe_mfma(int fp4, int valu, int blocks, int iters, void* 
     const dim3 g(blocks), b(256);
     hipStream_t st = (hipStream_t)stream;
     unsigned* o = (unsigned*)out;
-    if (fp4 && valu == -1) hipLaunchKernelGGL(probe_mfma_lds_kernel, g, b, 0, st, o, iters);      // fragments shared through LDS
-    else if (fp4) {
-        if (valu == 0) hipLaunchKernelGGL((probe_mfma_kernel<true, 8, 0>), g, b, 0, st, o, iters);
-        else if (valu == 2) hipLaunchKernelGGL((probe_mfma_kernel<true, 8, 2>), g, b, 0, st, o, iters);
-        else if (valu == 4) hipLaunchKernelGGL((probe_mfma_kernel<true, 8, 4>), g, b, 0, st, o, iters);
-        else return -1;
-    } else {
-        if (valu == 0) hipLaunchKernelGGL((probe_mfma_kernel<false, 8, 0>), g, b, 0, st, o, iters);
-        else if (valu == 2) hipLaunchKernelGGL((probe_mfma_kernel<false, 8, 2>), g, b, 0, st, o, iters);
-        else if (valu == 4) hipLaunchKernelGGL((probe_mfma_kernel<false, 8, 4>), g, b, 0, st, o, iters);
-        else return -1;
+    if (fp4 && valu == -1) hipLaunchKernelGGL(probe_mfma_lds_kernel, g, b, 0, st, o, iters, 1u);      // fragments shared through LDS
+    else {
+#define PROBE_CASE(V) case V: if (fp4) hipLaunchKernelGGL((probe_mfma_kernel<true, 8, V, false>), g, b, 0, st, o, iters, 1u); \
+                              else hipLaunchKernelGGL((probe_mfma_kernel<false, 8, V, false>), g, b, 0, st, o, iters, 1u); break; \
+                      case 100 + V: if (!fp4) return -1; hipLaunchKernelGGL((probe_mfma_kernel<true, 8, V, true>), g, b, 0, st, o, iters, 1u); break;
+        switch (valu) {
+            PROBE_CASE(0) PROBE_CASE(1) PROBE_CASE(2) PROBE_CASE(3) PROBE_CASE(4) PROBE_CASE(5) PROBE_CASE(6) PROBE_CASE(7) PROBE_CASE(8)
+            default: return -1;
+        }
+#undef PROBE_CASE
     }
     return (int)hipGetLastError();
 }
