@@ -645,7 +645,6 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
             const int* sp = st + row0 * ROW_I + c4 * 4;
             char* dst = out_base + (nrow0 + row0) * row_bytes + (m << esz_shift);
             const int64_t dstep = RSTEP * row_bytes;
-            const bool scaled = a.out_kind == BGEMM_OUT_F32_SCALED || a.out_kind == BGEMM_OUT_F16_SCALED;
             const bool has_bias = a.ep_bias != nullptr;
             const ColParams (&cp)[4] = cp4;
             const float saf = saf8;
