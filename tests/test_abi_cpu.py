@@ -3,6 +3,8 @@ rejects bad arguments from the host side (no kernel is launched by any call here
 import ctypes
 import os
 import re
+import shutil
+import subprocess
 
 import pytest
 
@@ -25,6 +27,26 @@ def test_header_symbols_exported():
         assert hasattr(L, n), "missing export: %s" % n
     # the binding table and the header list the same entry points
     assert sorted(_lib.SIGNATURES) == names
+
+
+def test_header_is_plain_c_and_a_c_program_links(tmp_path):
+    """The boundary is a C ABI: the header compiles as C99 and as C++11 with -pedantic, and a C program built against it
+    links with the library and calls a host-only entry point (what a cgo / JNI / FFI binding does first)."""
+    gcc = shutil.which("gcc")
+    if not gcc:
+        pytest.skip("no gcc")
+    src = tmp_path / "use_header.c"
+    src.write_text('#include <stdio.h>\n#include "bgemm_mi355x.h"\n'
+                   'int main(void) { printf("%d %lld\\n", bgemm_abi_version(), (long long)bgemm_tiled_words(33, 257)); return 0; }\n')
+    inc = os.path.dirname(HEADER)
+    for cc, std in ((gcc, ["-std=c99"]), (shutil.which("g++") or gcc, ["-std=c++11", "-x", "c++"])):
+        subprocess.check_call([cc] + std + ["-Wall", "-Wextra", "-Werror", "-pedantic", "-I", inc, "-fsyntax-only", str(src)])
+    exe = tmp_path / "use_header"
+    libdir = os.path.dirname(_lib.SO_PATH)
+    subprocess.check_call([gcc, "-std=c99", "-I", inc, str(src), "-o", str(exe), "-L", libdir, "-l:" + os.path.basename(_lib.SO_PATH),
+                           "-Wl,-rpath," + libdir, "-Wl,-rpath-link,/opt/rocm/lib"])
+    out = subprocess.check_output([str(exe)], env=dict(os.environ, LD_LIBRARY_PATH="/opt/rocm/lib:" + os.environ.get("LD_LIBRARY_PATH", "")))
+    assert out.split() == [str(_lib.ABI_VERSION).encode(), b"1024"]
 
 
 def test_layout_sizes():
