@@ -38,7 +38,7 @@ C5_PROFILE = os.path.join(ROOT, "profiles", "gemm_mfma_f4_bgemm_8192x8192x8192.t
 PROBES_SO = os.path.join(ROOT, "libbench_probes.so")
 
 KERNEL_NAMES = {0: "mfma 256x256", 1: "mfma 128x128", 2: "mfma 64x128", 3: "mfma 32x128", 4: "mfma 256x128", 5: "mfma 32x256",
-                6: "mfma 64x64", 7: "mfma 128x64", 16: "decode stream", 17: "decode split-K in the block",
+                6: "mfma 64x64", 7: "mfma 128x64", 8: "mfma 128x256 signed", 16: "decode stream", 17: "decode split-K in the block",
                 18: "decode four pieces a block", 19: "decode AND-popcount (vector ALU)", 32: "VALU popcount GEMM"}
 
 
@@ -171,6 +171,7 @@ def kernel_of(w, x, mode, splitK=1, variant=0, out_dtype=None):
 
 KERNEL_IDS = {"mfma 256x256": "m256x256", "mfma 128x128": "m128x128", "mfma 64x128": "m64x128", "mfma 32x128": "m32x128",
               "mfma 256x128": "m256x128", "mfma 32x256": "m32x256", "mfma 64x64": "m64x64", "mfma 128x64": "m128x64",
+              "mfma 128x256 signed": "m128x256t",
               "decode stream": "stream", "decode split-K in the block": "splitk", "decode four pieces a block": "quad",
               "decode AND-popcount (vector ALU)": "popc", "VALU popcount GEMM": "valu"}
 
@@ -699,8 +700,10 @@ def bench_thresholds(steps=60, shapes=None, warm=True):
         warm = lambda i: lk.bgemm_packed_forward(wps[i % copies], xp, mode, torch.int32, 8, 0, out=out)
         warm(0)
         time_gpu_graph(warm, copies, 2, 2)
-        for kid in general + [B.KERNEL_SKINNY_SPLITK, B.KERNEL_SKINNY_QUAD]:
+        for kid in general + [B.KERNEL_MFMA_128x256T, B.KERNEL_SKINNY_SPLITK, B.KERNEL_SKINNY_QUAD]:
             if planes == 2 and kid in (B.KERNEL_MFMA_256x256, B.KERNEL_MFMA_256x128):
+                continue
+            if planes == 1 and kid == B.KERNEL_MFMA_128x256T:
                 continue
             if kid in (B.KERNEL_MFMA_128x64, B.KERNEL_MFMA_64x64) and M > 64:
                 continue

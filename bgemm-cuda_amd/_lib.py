@@ -19,7 +19,7 @@ STATIC_SCRATCH_BYTES = 32 << 20      # BGEMM_STATIC_SCRATCH_BYTES
 VARIANT_AUTO, VARIANT_VALU, VARIANT_MFMA, VARIANT_MFMA_F4 = 0, 1, 2, 3
 # BGEMM_KERNEL_*: what bgemm_packed_kernel_id() returns and force_kernel() takes
 KERNEL_MFMA_256x256, KERNEL_MFMA_128x128, KERNEL_MFMA_64x128, KERNEL_MFMA_32x128, KERNEL_MFMA_256x128 = 0, 1, 2, 3, 4
-KERNEL_MFMA_32x256, KERNEL_MFMA_64x64, KERNEL_MFMA_128x64 = 5, 6, 7
+KERNEL_MFMA_32x256, KERNEL_MFMA_64x64, KERNEL_MFMA_128x64, KERNEL_MFMA_128x256T = 5, 6, 7, 8
 KERNEL_SKINNY_STREAM, KERNEL_SKINNY_SPLITK, KERNEL_SKINNY_QUAD, KERNEL_SKINNY_POPC, KERNEL_VALU = 16, 17, 18, 19, 32
 
 

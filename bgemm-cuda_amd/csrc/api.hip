@@ -44,7 +44,7 @@ static bool split_variant(int variant, int* family, int* force)
     switch (*force) {
     case BGEMM_KERNEL_MFMA_256x256: case BGEMM_KERNEL_MFMA_128x128: case BGEMM_KERNEL_MFMA_64x128:
     case BGEMM_KERNEL_MFMA_32x128: case BGEMM_KERNEL_MFMA_256x128: case BGEMM_KERNEL_MFMA_32x256: case BGEMM_KERNEL_MFMA_64x64:
-    case BGEMM_KERNEL_MFMA_128x64: case BGEMM_KERNEL_SKINNY_STREAM: case BGEMM_KERNEL_SKINNY_SPLITK:
+    case BGEMM_KERNEL_MFMA_128x64: case BGEMM_KERNEL_MFMA_128x256T: case BGEMM_KERNEL_SKINNY_STREAM: case BGEMM_KERNEL_SKINNY_SPLITK:
     case BGEMM_KERNEL_SKINNY_QUAD: case BGEMM_KERNEL_SKINNY_POPC: return true;
     default: return false;
     }
@@ -229,7 +229,7 @@ static int packed_forward(int mode, const void* W_tiled, const void* X_tiled, co
         return v == BGEMM_VARIANT_VALU ? BGEMM_KERNEL_VALU
                : force >= 0            ? force
                : skinny                ? gemm_skinny_kernel_id(a, fp4)
-                                       : gemm_mfma_kernel_id(batch, M, N, a.KT, a.mc.planes, out_elem_shift(a.out_kind));
+                                       : gemm_mfma_kernel_id(batch, M, N, a.KT, a.mc.planes, out_elem_shift(a.out_kind), fp4);
     if (splitK > 1 && v == BGEMM_VARIANT_VALU) {
         size_t part, cnt;
         ws_needs(v, a.mc.planes, batch, M, N, K, splitK, &part, &cnt);

@@ -303,7 +303,7 @@ int pack_sign_pair(const void* srcA, int64_t rowsA, void* dstA, const void* srcB
 
 // Kernel families (each in its own translation unit).
 int launch_gemm_mfma(const GemmArgs& a, hipStream_t st, bool fp4);
-int gemm_mfma_kernel_id(int64_t batch, int64_t M, int64_t N, int64_t KT, int planes, int out_shift);     // BGEMM_KERNEL_MFMA_* by shape
+int gemm_mfma_kernel_id(int64_t batch, int64_t M, int64_t N, int64_t KT, int planes, int out_shift, bool fp4);     // BGEMM_KERNEL_MFMA_* by shape
 // A ternary operand's two planes on the general kernel's pipelined 128 x 128 tile (two resident blocks per CU): from two
 // thirds of a block per CU on 16 K-tiles or more, except between one block per CU and one and two thirds, which would
 // leave the launch waiting for the CUs that run two, and only where most of the tiles land on real outputs.

@@ -17,7 +17,10 @@ namespace bgemm {
 // Block = WGN x WGM waves, each wave owns WN x WM tiles of 32x32 outputs, PL activation planes.
 // COUNTED (pipelined tiles only): the operands' row popcounts come with the call (GemmArgs::cntW / cntX) and the main
 // loop counts nothing: a sixth of its vector instructions on the 256 x 128 tile.
-template <typename Eng, int WGN, int WGM, int WN, int WM, int PL, bool PIPE, bool COUNTED = false>
+// TERN (pipelined, fp4 engine, PL = 1): binary weights x ternary activations with signed operands (EngF4::tern_x / tern_w):
+// a slot of the activation side is made of both planes' raw words, one MFMA does what takes the AND-dot two, and the
+// accumulators hold the output itself: no popcounts, no rank-one terms.
+template <typename Eng, int WGN, int WGM, int WN, int WM, int PL, bool PIPE, bool COUNTED = false, bool TERN = false>
 // (Second launch bound: from two waves a SIMD on, a wave's register budget is the 256 architected registers, and the
 // compiler then keeps the accumulators there instead of in the accumulation registers, which the epilogue could
 // only reach through one copy per value.)
@@ -66,7 +69,7 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
     const int mt0 = (tm * WGM + wm) * WM;
     const uint4* Wb = a.W + (int64_t)b * a.strideW;
     const uint4* Xb = a.X + (int64_t)b * a.strideX;
-    const uint4* X2b = PL == 2 ? a.X2 + (int64_t)b * a.strideX : nullptr;
+    const uint4* X2b = PL == 2 || TERN ? a.X2 + (int64_t)b * a.strideX : nullptr;
     constexpr int ROW_I = WM * 32 + 8;       // staged row stride in ints (+8 keeps the two lane halves on
                                              // different LDS banks)
     __shared__ __align__(16) int rowp[WGN * WGM * WN * 32];
@@ -80,7 +83,7 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
     // counts the bits of its first WN / 2 slots only, which are different rows for the two, and they swap the
     // counts through LDS before the epilogue (half the activation side's popcounts: 0.25 vector instructions a MFMA).
     static_assert(!PIPE || PL == 2 || (WGM == 2 && WN % 2 == 0), "the popcount split is laid out for two waves along M");
-    const int xs = PIPE && PL == 1 ? wm * (WN / 2) : 0;      // (two bit planes: every wave counts all its activation slots)
+    const int xs = PIPE && PL == 1 && !TERN ? wm * (WN / 2) : 0;      // (two bit planes: every wave counts all its activation slots)
     auto x_tile = [&](const int i) { return nt0 + (i ^ xs); };
 
     // per-fragment base pointers (row tile clamped so ragged edges re-read a valid tile)
@@ -155,8 +158,17 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
         // registers allow (two tiles ahead: the 256 x 128 tile's 32 MFMAs a K-tile are half a microsecond, less
         // than a trip to a far L2 takes under load; on the 128 x 128 tile likewise: 3072 x 1024 x 8192 17.0 -> 15.3 us,
         // 11008 x 640 x 8192 28.3 -> 25.8)
-        constexpr int NBUF = (NM == 8 || NM == 4) && STEPS == 4 ? 3 : 2;       // (the int8 engine's eight steps a tile leave no registers for it)
+        constexpr int NBUF = (NM == 8 || NM == 4) && STEPS == 4 && !TERN ? 3 : 2;       // (the int8 engine's eight steps a tile, and the second plane's raw words, leave no registers for it)
         unsigned rawA[NF][4], rawB[NF][4], rawC[NBUF == 3 ? NF : 1][4], buf[2][NF][4];
+        constexpr int XN2 = TERN ? XN : 1;                 // TERN: the sign plane's raw words of every activation slot
+        unsigned rawA2[XN2][4], rawB2[XN2][4];
+        __amdgpu_buffer_rsrc_t rs2[XN2];
+        if constexpr (TERN) {
+#pragma unroll
+            for (int f = 0; f < XN; f++)
+                rs2[f] = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint4*>(X2b + min((int64_t)x_tile(f), (int64_t)a.NT - 1) * a.KT * TILE_U4), 0,
+                                                           a.KT * (TILE_U4 * 16), 0x00020000);
+        }
         int pop[NF];
 #pragma unroll
         for (int f = 0; f < NF; f++) pop[f] = 0;
@@ -164,7 +176,16 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
             const v4i v = __builtin_amdgcn_raw_buffer_load_b128(rs[f], lane * 16 + kt * (TILE_U4 * 16), 0, 0);
             r[0] = v.x; r[1] = v.y; r[2] = v.z; r[3] = v.w;
         };
-        auto k_tile = [&](unsigned (&A)[NF][4], unsigned (&B)[NF][4], const int kt) {
+        auto load_frag2 = [&](unsigned (&r)[4], const int f, const int kt) {
+            const v4i v = __builtin_amdgcn_raw_buffer_load_b128(rs2[f], lane * 16 + kt * (TILE_U4 * 16), 0, 0);
+            r[0] = v.x; r[1] = v.y; r[2] = v.z; r[3] = v.w;
+        };
+        // register d of fragment f at step s, from the raw words of the K-tile it belongs to
+        auto expand_reg = [&](const unsigned (&R)[NF][4], const unsigned (&R2)[XN2][4], const int f, const int c, const int s) -> unsigned {
+            if constexpr (TERN) return f < XN ? Eng::tern_x(R[f][c], R2[f < XN2 ? f : 0][c], s) : Eng::tern_w(R[f][c], s);
+            else return (f < XN) == XS_FIRST ? Eng::expand1_x(R[f][c], s) : Eng::expand1_w(R[f][c], s);
+        };
+        auto k_tile = [&](unsigned (&A)[NF][4], unsigned (&B)[NF][4], unsigned (&A2)[XN2][4], unsigned (&B2)[XN2][4], const int kt) {
 #pragma unroll
             for (int s = 0; s < STEPS; s++) {
                 unsigned (&cur)[NF][4] = buf[s & 1];
@@ -174,15 +195,16 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
                     const int u = q / WM, j = q % WM;              // activation slot: plane u / WN, tile row u % WN
                     acc[u / WN][u % WN][j] = Eng::mma(Eng::make(cur[u]), Eng::make(cur[XN + j]), acc[u / WN][u % WN][j]);
 #pragma unroll
-                    for (int d = q * DPG; d < (q + 1) * DPG; d++)
-                        nxt[d / 4][d % 4] = (d / 4 < XN) == XS_FIRST      // fragments 0 .. XN-1 are the activation side
-                            ? (s + 1 < STEPS ? Eng::expand1_x(A[d / 4][d % 4], s + 1) : Eng::expand1_x(B[d / 4][d % 4], 0))
-                            : (s + 1 < STEPS ? Eng::expand1_w(A[d / 4][d % 4], s + 1) : Eng::expand1_w(B[d / 4][d % 4], 0));
-                    if (!COUNTED && s == 0 && (q < (PL == 1 ? WN / 2 : XN) || (q >= XN && q < NF))) {     // v_bcnt adds into its accumulator: four instructions a fragment, written out
+                    for (int d = q * DPG; d < (q + 1) * DPG; d++)      // fragments 0 .. XN-1 are the activation side
+                        nxt[d / 4][d % 4] = s + 1 < STEPS ? expand_reg(A, A2, d / 4, d % 4, s + 1) : expand_reg(B, B2, d / 4, d % 4, 0);
+                    if (!COUNTED && !TERN && s == 0 && (q < (PL == 1 ? WN / 2 : XN) || (q >= XN && q < NF))) {     // v_bcnt adds into its accumulator: four instructions a fragment, written out
 #pragma unroll                                  // because the compiler prefers four counts and two three-way adds
                         for (int c = 0; c < 4; c++) asm("v_bcnt_u32_b32 %0, %1, %0" : "+v"(pop[q]) : "v"(A[q][c]));
                     }
                     if (s == STEPS - 1 && q < NF) load_frag(A[q], q, kt + NBUF);   // A is dead after step STEPS-2
+                    if constexpr (TERN) {
+                        if (s == STEPS - 1 && q >= NM - XN) load_frag2(A2[q - (NM - XN)], q - (NM - XN), kt + NBUF);
+                    }
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
@@ -192,31 +214,39 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
             for (int f = 0; f < NF; f++) {
                 load_frag(rawA[f], f, kt0); load_frag(rawB[f], f, kt0 + 1);
                 if constexpr (NBUF == 3) load_frag(rawC[f], f, kt0 + 2);
+                if constexpr (TERN) {
+                    if (f < XN) { load_frag2(rawA2[f < XN ? f : 0], f, kt0); load_frag2(rawB2[f < XN ? f : 0], f, kt0 + 1); }
+                }
             }
 #pragma unroll
             for (int f = 0; f < NF; f++)
 #pragma unroll
-                for (int c = 0; c < 4; c++) buf[0][f][c] = (f < XN) == XS_FIRST ? Eng::expand1_x(rawA[f][c], 0) : Eng::expand1_w(rawA[f][c], 0);
+                for (int c = 0; c < 4; c++) buf[0][f][c] = expand_reg(rawA, rawA2, f, c, 0);
             if constexpr (NBUF == 3) {
                 // whole rounds of three, then what is left in the same rotation (a K-tile past the range multiplies zeros)
                 int kt = kt0;
                 for (; kt + 3 <= kt1; kt += 3) {
-                    k_tile(rawA, rawB, kt);
-                    k_tile(rawB, rawC, kt + 1);
-                    k_tile(rawC, rawA, kt + 2);
+                    k_tile(rawA, rawB, rawA2, rawB2, kt);
+                    k_tile(rawB, rawC, rawA2, rawB2, kt + 1);
+                    k_tile(rawC, rawA, rawA2, rawB2, kt + 2);
                 }
                 if (kt < kt1) {
-                    k_tile(rawA, rawB, kt);
-                    if (kt + 1 < kt1) k_tile(rawB, rawC, kt + 1);
+                    k_tile(rawA, rawB, rawA2, rawB2, kt);
+                    if (kt + 1 < kt1) k_tile(rawB, rawC, rawA2, rawB2, kt + 1);
                 }
             } else {
                 for (int kt = kt0; kt < kt1; kt += 2) {
-                    k_tile(rawA, rawB, kt);
-                    k_tile(rawB, rawA, kt + 1);
+                    k_tile(rawA, rawB, rawA2, rawB2, kt);
+                    k_tile(rawB, rawA, rawB2, rawA2, kt + 1);
                 }
             }
         }
-        if constexpr (COUNTED) {
+        if constexpr (TERN) {          // nothing was counted and nothing is needed
+#pragma unroll
+            for (int i = 0; i < WN; i++) pb[0][i] = 0;
+#pragma unroll
+            for (int j = 0; j < WM; j++) pa[j] = 0;
+        } else if constexpr (COUNTED) {
             // the lane's row of every fragment, read where the caller keeps the counts (rows past the end: any valid one,
             // their outputs are never stored); halved below by nothing: these are whole rows, not K-halves
             const int64_t cx = a.strideX ? (int64_t)b * a.N : 0, cw = a.strideW ? (int64_t)b * a.M : 0;
@@ -360,6 +390,8 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
             const int rowterm = (v & 3) == 0 ? q.x : (v & 3) == 1 ? q.y : (v & 3) == 2 ? q.z : q.w;
 #pragma unroll
             for (int j = 0; j < WM; j++) {
+                if constexpr (TERN) val[j][v] = Eng::to_int(acc[0][i][j], v);
+                else
                 val[j][v] = capa[j] + rowterm + (PL == 2 ? dot_terms2(mc, Eng::to_int(acc[0][i][j], v), Eng::to_int(acc[PL - 1][i][j], v))
                                                           : dot_term(mc, Eng::to_int(acc[0][i][j], v)));
             }
@@ -746,7 +778,9 @@ struct MfmaCfg { int id, bn, bm; };
 //     spread their stores over the memory channels), and two bit planes (one weight expansion feeds both planes).
 //   * 64 x 128, 32 x 128: whatever is left, so that every unit gets a block; 64-column tiles for outputs of at most 64
 //     columns.
-static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int planes, int out_shift)
+//   * 128 x 256 signed (a ternary operand on the fp4 engine): half the matrix-core work of the two-plane tiles; from more
+//     than half a block a unit on (129 blocks: 1.2 to 1.5 times the best two-plane kernel, level with it at 128 and below).
+static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int planes, int out_shift, bool fp4)
 {
     auto blocks = [&](int bn, int bm) { return batch * cdiv(N, bn) * cdiv(M, bm); };
     auto filled = [&](int bn, int bm) { return (double)(N * M) / (double)(cdiv(N, bn) * bn * cdiv(M, bm) * bm); };
@@ -772,6 +806,7 @@ static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int pla
     // would run two blocks and the rest one on a short K
     const bool pipelined_ok = planes == 1 && KT >= 8 && b11 >= (KT >= 16 ? 144 : 192) &&
                               (b11 >= 192 || KT >= 24 || filled(128, 128) >= 0.85) && !(KT < 12 && b11 > 256 && b11 < 416);
+    if (planes == 2 && fp4 && KT >= 4 && blocks(128, 256) > 128 && filled(128, 256) >= 0.7) return {BGEMM_KERNEL_MFMA_128x256T, 128, 256};
     if ((b11 >= 512 || pipelined_ok) && filled(128, 128) >= 0.6) return {BGEMM_KERNEL_MFMA_128x128, 128, 128};
     if (planes == 2 && two_plane_tile_128(batch, M, N, KT)) return {BGEMM_KERNEL_MFMA_128x128, 128, 128};
     if (planes == 2 && b32 >= (KT >= 8 ? 96 : 160)) return {BGEMM_KERNEL_MFMA_32x256, 32, 256};
@@ -828,15 +863,31 @@ static int launch_cfg(const GemmArgs& a, hipStream_t st)
     return check_launch("gemm_mfma");
 }
 
-int gemm_mfma_kernel_id(int64_t batch, int64_t M, int64_t N, int64_t KT, int planes, int out_shift)
+// Binary weights x ternary activations with signed operands on a 128 x 256 tile (a wave: two activation tile rows, the dearer
+// side to expand, against four weight tiles): fp4 engine only.
+template <typename Eng>
+static int launch_tern(const GemmArgs& a, hipStream_t st)
 {
-    return pick_cfg(batch, M, N, KT, planes, out_shift).id;
+    if constexpr (std::is_same<Eng, EngF4>::value) {
+        if (a.mc.planes != 2) return fail(BGEMM_EINVAL, "gemm_mfma: the signed tile takes a ternary activation operand");
+        const int tiles_n = (int)cdiv(a.N, 128), tiles_m = (int)cdiv(a.M, 256);
+        const int64_t grid = (int64_t)a.batch * tiles_n * tiles_m;
+        if (grid <= 0 || grid > 0x7fffffffLL) return fail(BGEMM_EINVAL, "gemm_mfma: grid of %lld blocks", (long long)grid);
+        hipLaunchKernelGGL((gemm_mfma_kernel<EngF4, 2, 2, 2, 4, 1, true, false, true>), dim3((unsigned)grid), dim3(256), 0, st, a, tiles_n, tiles_m);
+        return check_launch("gemm_mfma");
+    } else
+        return fail(BGEMM_EINVAL, "gemm_mfma: the signed ternary tile runs on the fp4 engine");
+}
+
+int gemm_mfma_kernel_id(int64_t batch, int64_t M, int64_t N, int64_t KT, int planes, int out_shift, bool fp4)
+{
+    return pick_cfg(batch, M, N, KT, planes, out_shift, fp4).id;
 }
 
 template <typename Eng>
 static int launch_eng(const GemmArgs& a, hipStream_t st)
 {
-    const int id = a.force >= 0 ? a.force : pick_cfg(a.batch, a.M, a.N, a.KT, a.mc.planes, out_elem_shift(a.out_kind)).id;
+    const int id = a.force >= 0 ? a.force : pick_cfg(a.batch, a.M, a.N, a.KT, a.mc.planes, out_elem_shift(a.out_kind), std::is_same<Eng, EngF4>::value).id;
     switch (id) {
     case BGEMM_KERNEL_MFMA_256x256: return launch_cfg<Eng, 2, 2, 4, 4>(a, st);
     case BGEMM_KERNEL_MFMA_256x128: return launch_cfg<Eng, 2, 2, 4, 2>(a, st);    // two blocks per CU
@@ -846,6 +897,7 @@ static int launch_eng(const GemmArgs& a, hipStream_t st)
     case BGEMM_KERNEL_MFMA_64x128: return launch_cfg<Eng, 1, 4, 2, 1>(a, st);
     case BGEMM_KERNEL_MFMA_32x128: return launch_cfg<Eng, 1, 4, 1, 1>(a, st);
     case BGEMM_KERNEL_MFMA_32x256: return launch_cfg<Eng, 1, 4, 1, 2>(a, st);
+    case BGEMM_KERNEL_MFMA_128x256T: return launch_tern<Eng>(a, st);
     default: return fail(BGEMM_EINVAL, "gemm_mfma: no kernel %d", id);
     }
 }

@@ -56,6 +56,7 @@ enum { BGEMM_KERNEL_MFMA_256x256 = 0, BGEMM_KERNEL_MFMA_128x128 = 1, BGEMM_KERNE
        BGEMM_KERNEL_MFMA_32x128 = 3, BGEMM_KERNEL_MFMA_256x128 = 4, BGEMM_KERNEL_MFMA_32x256 = 5,
        BGEMM_KERNEL_MFMA_64x64 = 6,
        BGEMM_KERNEL_MFMA_128x64 = 7,
+       BGEMM_KERNEL_MFMA_128x256T = 8,   /* ternary activations as signed operands: BGEMM_MODE_BWTA on the fp4 engine only */
        BGEMM_KERNEL_SKINNY_STREAM = 16, BGEMM_KERNEL_SKINNY_SPLITK = 17, BGEMM_KERNEL_SKINNY_QUAD = 18,
        BGEMM_KERNEL_SKINNY_POPC = 19,
        BGEMM_KERNEL_VALU = 32 };

@@ -78,7 +78,7 @@ def test_layout_sizes():
     (dict(mode=7), _lib.EINVAL),
     (dict(out_dtype=5), _lib.EINVAL),
     (dict(variant=4), _lib.EINVAL),
-    (dict(variant=_lib.force_kernel(8)), _lib.EINVAL),                                   # no such kernel
+    (dict(variant=_lib.force_kernel(9)), _lib.EINVAL),                                   # no such kernel
     (dict(variant=_lib.force_kernel(_lib.KERNEL_MFMA_64x64, _lib.VARIANT_VALU)), _lib.EINVAL),   # the VALU design has one kernel
     (dict(variant=_lib.force_kernel(_lib.KERNEL_SKINNY_STREAM), batch=70000, strideC=64 * 256), _lib.EINVAL),
     (dict(M=-1), _lib.EINVAL),
@@ -165,7 +165,12 @@ def test_dispatch_of_the_benchmark_configurations():
     assert kid(MODE_BWTA, 1, 8192, 160, 8192, 1, A) == B.KERNEL_MFMA_32x256      # 640
     assert kid(MODE_BWTA, 1, 11008, 96, 4096, 1, A) == B.KERNEL_MFMA_32x256      # 129 blocks of 32 x 256
     assert kid(MODE_BWTA, 1, 11008, 256, 8192, 1, A) == B.KERNEL_MFMA_128x128    # 172 blocks of 128 x 128
-    assert kid(MODE_BWTA, 1, 11008, 320, 11008, 1, A) == B.KERNEL_MFMA_32x256    # 258: between one block a unit and one and a quarter
+    # the signed tile takes a ternary operand from more than half a 128 x 256 block a unit on, on the fp4 engine only
+    assert kid(MODE_BWTA, 1, 11008, 320, 11008, 1, A) == B.KERNEL_MFMA_128x256T  # 129 blocks
+    assert kid(MODE_BWTA, 1, 11008, 320, 11008, 1, B.VARIANT_MFMA) == B.KERNEL_MFMA_32x256    # int8 engine: 258 blocks of 128 x 128, between one a unit and one and a quarter
+    assert kid(MODE_BWTA, 1, 22016, 2048, 4096, 1, A) == B.KERNEL_MFMA_128x256T
+    assert kid(MODE_BWTA, 1, 4096, 1024, 11008, 1, A) == B.KERNEL_MFMA_128x128   # 128 blocks of the signed tile: level, stays
+    assert kid(MODE_BWTA, 1, 8192, 8192, 512, 1, A) != B.KERNEL_MFMA_128x256T    # two K-tiles
     assert kid(MODE_ATTN_X, 24, 64, 512, 512, 1, A) == B.KERNEL_MFMA_64x64
     assert kid(MODE_BWTA, 1, 11008, 1, 4096, 8, A) == B.KERNEL_SKINNY_POPC
     assert kid(MODE_BWTA, 1, 11008, 16, 4096, 8, A) == B.KERNEL_SKINNY_SPLITK
@@ -173,7 +178,7 @@ def test_dispatch_of_the_benchmark_configurations():
     assert kid(MODE_XOR, 1, 4096, 128, 4096, 1, VARIANT_VALU) == B.KERNEL_VALU
     assert kid(MODE_XOR, 70000, 40, 8, 300, 1, A) in TILES        # a batch beyond the decode kernels' grid
     assert kid(MODE_XOR, 1, 64, 64, 64, 1, force_kernel(B.KERNEL_MFMA_256x256)) == B.KERNEL_MFMA_256x256
-    assert kid(MODE_XOR, 1, 64, 64, 64, 1, force_kernel(8)) == B.EINVAL    # no such kernel
+    assert kid(MODE_XOR, 1, 64, 64, 64, 1, force_kernel(9)) == B.EINVAL    # no such kernel
     assert kid(MODE_XOR, 1, 64, 64, 64, 1, force_kernel(B.KERNEL_MFMA_64x64, VARIANT_VALU)) == B.EINVAL
     assert kid(9, 1, 64, 64, 64, 1, A) == B.EINVAL and kid(MODE_XOR, 1, 64, 0, 64, 1, A) == B.EINVAL
 

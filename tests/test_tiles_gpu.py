@@ -69,7 +69,7 @@ def bits_of(a):
     return a.view(np.uint16 if a.dtype == np.float16 else np.uint32)
 
 
-def check_all_kinds(oracle, wp, xp, acc, M, N, variant, rng, rows=None, cols=None):
+def check_all_kinds(oracle, wp, xp, acc, M, N, variant, rng, rows=None, cols=None, mode=MODE_XOR):
     """Every output kind of one GEMM against `acc` (the exact int32 result, or its [rows][:, cols] sample)."""
     def sample(t):
         t = t[0]
@@ -77,9 +77,9 @@ def check_all_kinds(oracle, wp, xp, acc, M, N, variant, rng, rows=None, cols=Non
             t = t[torch.from_numpy(rows).to(DEV)][:, torch.from_numpy(cols).to(DEV)]
         return t.cpu().numpy()
 
-    got = sample(lk.bgemm_packed_forward(wp, xp, MODE_XOR, torch.int32, 1, variant))
+    got = sample(lk.bgemm_packed_forward(wp, xp, mode, torch.int32, 1, variant))
     assert (got == acc).all(), "int32"
-    got = sample(lk.bgemm_packed_forward(wp, xp, MODE_XOR, torch.half, 1, variant))
+    got = sample(lk.bgemm_packed_forward(wp, xp, mode, torch.half, 1, variant))
     assert (bits_of(got) == bits_of(f16_of(acc))).all(), "fp16"
     for dtype in (np.float32, np.float16):
         sw = rng.uniform(1e-4, 3e-3, M).astype(dtype)
@@ -88,13 +88,13 @@ def check_all_kinds(oracle, wp, xp, acc, M, N, variant, rng, rows=None, cols=Non
         swc, bc = (sw, bias) if cols is None else (sw[cols], bias[cols])
         for with_bias in (True, False):
             want = oracle.np_scale_epilogue(acc, swc, sa, bc if with_bias else None)
-            got = sample(lk.bgemm_packed_forward(wp, xp, MODE_XOR, variant=variant,
+            got = sample(lk.bgemm_packed_forward(wp, xp, mode, variant=variant,
                                                  scale=(to_dev(sw), to_dev(sa.reshape(1)), to_dev(bias) if with_bias else None)))
             assert got.dtype == want.dtype and (bits_of(got) == bits_of(want)).all(), ("scaled", dtype, with_bias)
         # bits kinds: the next layer's operand, the zero point at a value that splits the outputs
         zp = np.asarray(0.011, dtype=dtype)
         out = lk.zeros_packed(N, M, 1, DEV)
-        lk.bgemm_packed_forward(wp, xp, MODE_XOR, variant=variant, bits_out=out,
+        lk.bgemm_packed_forward(wp, xp, mode, variant=variant, bits_out=out,
                                 scale=(to_dev(sw), to_dev(sa.reshape(1)), to_dev(bias)), next_zero_point=to_dev(zp.reshape(1)))
         logical = lk.logical_from_tiled(out).cpu().numpy().view(np.uint32)               # [N][ceil(M/32)]
         y = oracle.np_scale_epilogue(acc, swc, sa, bc)
@@ -279,6 +279,79 @@ def test_row_popcounts_brought_by_the_caller(tile, engine):
         want[:, :, 7] -= 2
         want[1, 11, :] -= 2
     assert (got == want).all()
+
+
+def tern(rng, *shape):
+    """-1 / 0 / +1 fp16 with both zeros among the zeros."""
+    t = rng.integers(-1, 2, shape).astype(np.float16)
+    return np.where((t == 0) & (rng.random(shape) < 0.5), np.float16(-0.0), t).astype(np.float16)
+
+
+# The signed tile (binary weights x ternary activations as signed fp4 operands, one MFMA per 64 k where the two bit planes
+# take two): M picks the store path as above, N = 515 leaves a ragged strip, K = five K-tiles (odd: the loop runs whole pairs, the
+# last tile of the pair reads as zero bits) and eight, the last one ragged.
+@pytest.mark.parametrize("K", [1275, 2048 - 9])
+@pytest.mark.parametrize("M", [520, 516, 517])
+def test_signed_ternary_tile_every_output_kind(oracle, M, K):
+    N = 515
+    rng = np.random.default_rng(M * 37 + K)
+    w, t = pm1(rng, M, K), tern(rng, N, K)
+    wp, xt = lk.pack_sign(to_dev(w)), lk.pack_ternary(to_dev(t))
+    variant = force_kernel(B.KERNEL_MFMA_128x256T, VARIANT_MFMA_F4)
+    assert lk.packed_kernel_id(wp, xt, MODE_BWTA, 1, variant) == B.KERNEL_MFMA_128x256T
+    check_all_kinds(oracle, wp, xt, dense(MODE_BWTA, w, t), M, N, variant, rng, mode=MODE_BWTA)
+
+
+def test_signed_ternary_tile_batched_and_what_it_refuses():
+    """A batch of ragged matrices, one K-tile and several; every ternary value against every weight sign; the tile takes
+    nothing but a ternary operand on the fp4 engine."""
+    rng = np.random.default_rng(128256)
+    variant = force_kernel(B.KERNEL_MFMA_128x256T, VARIANT_MFMA_F4)
+    for Bn, M, N, K in ((3, 70, 300, 200), (2, 300, 70, 1000), (1, 257, 129, 256 * 3)):
+        w, t = pm1(rng, Bn, M, K), tern(rng, Bn, N, K)
+        wp, xt = lk.pack_sign(to_dev(w)), lk.pack_ternary(to_dev(t))
+        got = lk.bgemm_packed_forward(wp, xt, MODE_BWTA, torch.int32, 1, variant).cpu().numpy()
+        assert (got == dense(MODE_BWTA, w, t)).all()
+        got = lk.bgemm_packed_forward(wp, xt, MODE_BWTA, torch.half, 1, variant).cpu().numpy()
+        assert (bits_of(got) == bits_of(f16_of(dense(MODE_BWTA, w, t)))).all()
+    # all-equal operands: every product -1, 0 or +1 in all of K, whole rows at +-K
+    M, N, K = 256, 128, 1024
+    for wv in (1.0, -1.0):
+        for tv in (1.0, -1.0, 0.0):
+            wp = lk.pack_sign(torch.full((M, K), wv, dtype=torch.half, device=DEV))
+            xt = lk.pack_ternary(torch.full((N, K), tv, dtype=torch.half, device=DEV))
+            got = lk.bgemm_packed_forward(wp, xt, MODE_BWTA, torch.int32, 1, variant)
+            assert int(got.min()) == int(got.max()) == int(wv * tv * K)
+    xp = lk.pack_sign(to_dev(pm1(rng, N, K)))
+    with pytest.raises(ValueError):
+        lk.bgemm_packed_forward(wp, xp, MODE_XOR, torch.int32, 1, variant)                                    # one bit plane
+    with pytest.raises(ValueError):
+        lk.bgemm_packed_forward(wp, xt, MODE_BWTA, torch.int32, 1, force_kernel(B.KERNEL_MFMA_128x256T, VARIANT_MFMA))   # the int8 engine
+
+
+@pytest.mark.parametrize("M,N,K", [(4096 + 5, 2048 + 3, 17 * 256 - 7), (11008, 512, 4096)])
+def test_signed_ternary_tile_where_the_library_picks_it(oracle, M, N, K):
+    """No forcing: prefill-sized BWTA products go to the signed tile on the fp4 engine (the library's choice) and to the
+    two-plane tiles on the int8 engine; both agree with the dense product on sampled rows and columns, edges included, in
+    every output kind, and with each other everywhere."""
+    rng = np.random.default_rng(M + N)
+    g = torch.Generator(device=DEV).manual_seed(M * 7 + N)
+    w16 = (1 - 2 * torch.randint(0, 2, (M, K), generator=g, device=DEV, dtype=torch.int8)).to(torch.half)
+    t16 = torch.randint(-1, 2, (N, K), generator=g, device=DEV, dtype=torch.int8).to(torch.half)
+    wp, xt = lk.pack_sign(w16), lk.pack_ternary(t16)
+    assert lk.packed_kernel_id(wp, xt, MODE_BWTA) == B.KERNEL_MFMA_128x256T
+    assert lk.packed_kernel_id(wp, xt, MODE_BWTA, 1, VARIANT_MFMA_F4) == B.KERNEL_MFMA_128x256T
+    assert lk.packed_kernel_id(wp, xt, MODE_BWTA, 1, VARIANT_MFMA) != B.KERNEL_MFMA_128x256T
+    rows = np.unique(np.concatenate([rng.choice(N, 90, replace=False), [0, N - 1, N - 2, (N // 32) * 32, (N // 128) * 128]]))
+    cols = np.unique(np.concatenate([rng.choice(M, 120, replace=False), [0, M - 1, M - 2, (M // 32) * 32, (M // 256) * 256]]))
+    rows, cols = rows[rows < N], cols[cols < M]
+    wsub = w16[torch.from_numpy(cols).to(DEV)].float().cpu()
+    xsub = t16[torch.from_numpy(rows).to(DEV)].float().cpu()
+    acc = (xsub @ wsub.T).to(torch.int32).numpy()
+    check_all_kinds(oracle, wp, xt, acc, M, N, VARIANT_AUTO, rng, rows, cols, mode=MODE_BWTA)
+    out = lk.bgemm_packed_forward(wp, xt, MODE_BWTA, torch.int32)[0]
+    assert torch.equal(out, lk.bgemm_packed_forward(wp, xt, MODE_BWTA, torch.int32, 1, VARIANT_MFMA)[0])
+    assert int(out.to(torch.int64).sum()) == int((w16.double().sum(0) * t16.double().sum(0)).sum().item())
 
 
 @pytest.mark.parametrize("engine", list(ENGINES))
