@@ -749,9 +749,10 @@ def section_decode(cold):
 
 
 def bench_prefill(steps=20, warmup=5):
-    """Binary weights x a batch of ternary rows (a prefill step, or a batch of decode steps): the two bit planes of the
-    activations are two matrix-core products against one expansion of the weights, so the matrix cores do 4*M*N*K of work
-    for the 2*M*N*K effective operations that `tops` counts; `frac` is the matrix-core work against the fp4 peak."""
+    """Binary weights x a batch of ternary rows (a prefill step, or a batch of decode steps).  On the signed tile (fp4 operands
+    that carry the ternary values themselves) the matrix cores do the 2*M*N*K operations that `tops` counts; on the two-plane
+    kernels the activations' bit planes are two products against one expansion of the weights, 4*M*N*K of matrix-core work;
+    `frac` is the matrix-core work against the fp4 peak either way."""
     import torch
     import lowbit_kernel as lk
     dev = torch.device("cuda:0")
@@ -767,7 +768,7 @@ def bench_prefill(steps=20, warmup=5):
         ok = check_sampled(out[0], w16, x16)
         r = row("BWTA %s W[%d,%d] x %d rows" % (name, M, K, N), ms, 2.0 * M * N * K,
                 M * K / 8 + 2 * N * K / 8 + 4.0 * M * N, ok, kernel_of(wp, xt, lk.MODE_BWTA), "mfma")
-        r["frac"] = round(2 * r["tops"] / FP4_MFMA_PEAK_TOPS, 4)       # matrix-core work is two products a weight expansion: 4*M*N*K
+        r["frac"] = round((1 if r["k"] == "m128x256t" else 2) * r["tops"] / FP4_MFMA_PEAK_TOPS, 4)
         rows.append(r)
         log_row(r)
         del w16, x16, wp, xt, out
@@ -784,7 +785,7 @@ def bench_prefill(steps=20, warmup=5):
         ms = min(time_gpu_graph(fn, copies, 2, 5) for _ in range(3))
         r = row("BWTA %s W[%d,%d] x %d rows cold" % (name, M, K, N), ms, 2.0 * M * N * K,
                 M * K / 8 + 2 * N * K / 8 + 4.0 * M * N, ok, kernel_of(wps[0], xt, lk.MODE_BWTA), "mfma")
-        r["frac"] = round(2 * r["tops"] / FP4_MFMA_PEAK_TOPS, 4)       # 4*M*N*K of matrix-core work, as above
+        r["frac"] = round((1 if r["k"] == "m128x256t" else 2) * r["tops"] / FP4_MFMA_PEAK_TOPS, 4)
         r["frac_hbm"] = round(r["gbs"] / HBM_PEAK_GBS, 4)
         rows.append(r)
         log_row(r)

@@ -180,9 +180,11 @@ __global__ __launch_bounds__(WGN* WGM * 64, (WN * WM * PL <= 8 ? 2 : 1)) void ge
             const v4i v = __builtin_amdgcn_raw_buffer_load_b128(rs2[f], lane * 16 + kt * (TILE_U4 * 16), 0, 0);
             r[0] = v.x; r[1] = v.y; r[2] = v.z; r[3] = v.w;
         };
+        unsigned tern_c1 = 0;
+        if constexpr (TERN) tern_c1 = Eng::tern_const();
         // register d of fragment f at step s, from the raw words of the K-tile it belongs to
         auto expand_reg = [&](const unsigned (&R)[NF][4], const unsigned (&R2)[XN2][4], const int f, const int c, const int s) -> unsigned {
-            if constexpr (TERN) return f < XN ? Eng::tern_x(R[f][c], R2[f < XN2 ? f : 0][c], s) : Eng::tern_w(R[f][c], s);
+            if constexpr (TERN) return f < XN ? Eng::tern_x(R[f][c], R2[f < XN2 ? f : 0][c], s) : Eng::tern_w(R[f][c], s, tern_c1);
             else return (f < XN) == XS_FIRST ? Eng::expand1_x(R[f][c], s) : Eng::expand1_w(R[f][c], s);
         };
         auto k_tile = [&](unsigned (&A)[NF][4], unsigned (&B)[NF][4], unsigned (&A2)[XN2][4], unsigned (&B2)[XN2][4], const int kt) {
@@ -779,7 +781,8 @@ struct MfmaCfg { int id, bn, bm; };
 //   * 64 x 128, 32 x 128: whatever is left, so that every unit gets a block; 64-column tiles for outputs of at most 64
 //     columns.
 //   * 128 x 256 signed (a ternary operand on the fp4 engine): half the matrix-core work of the two-plane tiles; from more
-//     than half a block a unit on (129 blocks: 1.2 to 1.5 times the best two-plane kernel, level with it at 128 and below).
+//     than half a block a unit on (129 blocks: 1.2 to 1.5 times the best two-plane kernel, level with it at 128 and below),
+//     two K-tiles or more (its loop runs whole pairs of them).
 static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int planes, int out_shift, bool fp4)
 {
     auto blocks = [&](int bn, int bm) { return batch * cdiv(N, bn) * cdiv(M, bm); };
@@ -806,7 +809,7 @@ static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int pla
     // would run two blocks and the rest one on a short K
     const bool pipelined_ok = planes == 1 && KT >= 8 && b11 >= (KT >= 16 ? 144 : 192) &&
                               (b11 >= 192 || KT >= 24 || filled(128, 128) >= 0.85) && !(KT < 12 && b11 > 256 && b11 < 416);
-    if (planes == 2 && fp4 && KT >= 4 && blocks(128, 256) > 128 && filled(128, 256) >= 0.7) return {BGEMM_KERNEL_MFMA_128x256T, 128, 256};
+    if (planes == 2 && fp4 && KT >= 2 && blocks(128, 256) > 128 && filled(128, 256) >= 0.7) return {BGEMM_KERNEL_MFMA_128x256T, 128, 256};
     if ((b11 >= 512 || pipelined_ok) && filled(128, 128) >= 0.6) return {BGEMM_KERNEL_MFMA_128x128, 128, 128};
     if (planes == 2 && two_plane_tile_128(batch, M, N, KT)) return {BGEMM_KERNEL_MFMA_128x128, 128, 128};
     if (planes == 2 && b32 >= (KT >= 8 ? 96 : 160)) return {BGEMM_KERNEL_MFMA_32x256, 32, 256};

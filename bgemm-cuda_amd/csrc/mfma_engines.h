@@ -100,22 +100,32 @@ struct EngF4 {
     // the activations) and rank-one terms.  A nibble is a sign (bit 3) and one value bit.  Activation: the nonzero plane's
     // bit stays where it is at steps 0..2 (0.5, 1, 2; at step 3 it moves to 1.0) under the bit of the sign plane (a sign
     // over a zero value adds nothing); weight: its sign bit over the reciprocal value (2, 1, 0.5, 1), so a product is -1, 0
-    // or +1 and the accumulator holds the layer's output itself.  Three VALU ops per activation register, two per weight
-    // register.
+    // or +1 and the accumulator holds the layer's output itself.  Three VALU ops per activation register, seven per four
+    // weight registers.
     __device__ static __forceinline__ unsigned tern_x(const unsigned z, const unsigned zs, const int s)
     {
         return s == 3 ? (zs & 0x88888888u) | ((z >> 2) & 0x22222222u) : ((zs << (3 - s)) & 0x88888888u) | (z & (0x11111111u << s));
     }
     // (mask in place, then one v_lshl_or_b32 with the value constant in a scalar register: written as the instruction,
-    // because the compiler turns the expression into shift, AND and OR, a literal each, which this ISA cannot fold)
-    __device__ static __forceinline__ unsigned tern_w(const unsigned w, const int s)
+    // because the compiler turns the expression into shift, AND and OR, a literal each, which this ISA cannot fold.  Step 3
+    // needs no shift: one v_and_or_b32, whose second constant has to sit in a vector register, `c1` = tern_const().)
+    __device__ static __forceinline__ unsigned tern_const()
     {
-        const unsigned m = w & (0x11111111u << s), c = s == 3 ? 0x22222222u : 0x44444444u >> s;
+        unsigned c = 0x22222222u;
+        asm volatile("" : "+v"(c));          // kept in a register: as a literal it would be a second constant operand
+        return c;
+    }
+    __device__ static __forceinline__ unsigned tern_w(const unsigned w, const int s, const unsigned c1)
+    {
         unsigned r;
+        if (s == 3) {
+            asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(w), "s"(0x88888888u), "v"(c1));
+            return r;
+        }
+        const unsigned m = w & (0x11111111u << s), c = 0x44444444u >> s;
         if (s == 0) asm("v_lshl_or_b32 %0, %1, 3, %2" : "=v"(r) : "v"(m), "s"(c));
         else if (s == 1) asm("v_lshl_or_b32 %0, %1, 2, %2" : "=v"(r) : "v"(m), "s"(c));
-        else if (s == 2) asm("v_lshl_or_b32 %0, %1, 1, %2" : "=v"(r) : "v"(m), "s"(c));
-        else asm("v_or_b32 %0, %2, %1" : "=v"(r) : "v"(m), "s"(c));
+        else asm("v_lshl_or_b32 %0, %1, 1, %2" : "=v"(r) : "v"(m), "s"(c));
         return r;
     }
     // a = activation-side fragment, b = weight-side fragment

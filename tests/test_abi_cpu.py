@@ -170,7 +170,7 @@ def test_dispatch_of_the_benchmark_configurations():
     assert kid(MODE_BWTA, 1, 11008, 320, 11008, 1, B.VARIANT_MFMA) == B.KERNEL_MFMA_32x256    # int8 engine: 258 blocks of 128 x 128, between one a unit and one and a quarter
     assert kid(MODE_BWTA, 1, 22016, 2048, 4096, 1, A) == B.KERNEL_MFMA_128x256T
     assert kid(MODE_BWTA, 1, 4096, 1024, 11008, 1, A) == B.KERNEL_MFMA_128x128   # 128 blocks of the signed tile: level, stays
-    assert kid(MODE_BWTA, 1, 8192, 8192, 512, 1, A) != B.KERNEL_MFMA_128x256T    # two K-tiles
+    assert kid(MODE_BWTA, 1, 8192, 8192, 256, 1, A) != B.KERNEL_MFMA_128x256T    # one K-tile
     assert kid(MODE_ATTN_X, 24, 64, 512, 512, 1, A) == B.KERNEL_MFMA_64x64
     assert kid(MODE_BWTA, 1, 11008, 1, 4096, 8, A) == B.KERNEL_SKINNY_POPC
     assert kid(MODE_BWTA, 1, 11008, 16, 4096, 8, A) == B.KERNEL_SKINNY_SPLITK
