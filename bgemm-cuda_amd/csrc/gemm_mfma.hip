@@ -781,7 +781,7 @@ struct MfmaCfg { int id, bn, bm; };
 //   * 64 x 128, 32 x 128: whatever is left, so that every unit gets a block; 64-column tiles for outputs of at most 64
 //     columns.
 //   * 128 x 256 signed (a ternary operand on the fp4 engine): half the matrix-core work of the two-plane tiles; from more
-//     than half a block a unit on (129 blocks: 1.2 to 1.5 times the best two-plane kernel, level with it at 128 and below),
+//     than half a block a unit on (ahead of every two-plane kernel from there, level with the best of them at 128 blocks),
 //     two K-tiles or more (its loop runs whole pairs of them).
 static MfmaCfg pick_cfg(int64_t batch, int64_t M, int64_t N, int64_t KT, int planes, int out_shift, bool fp4)
 {
