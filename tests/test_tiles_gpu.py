@@ -511,6 +511,33 @@ def test_k_just_under_2_to_24_every_term_at_its_maximum(kernel):
             assert run(w1, tern(xh), MODE_BWTA) == pb
 
 
+def test_signed_ternary_tile_k_just_under_2_to_24():
+    """K = 2^24 - 32 on the signed tile: sums of +1 or -1 over all of K reach +-K, the last integers the fp32
+    accumulator holds exactly; all-zero activations give 0, and rows whose nonzero entries are every other word (all
+    negative) give the count of those entries with the weight's sign."""
+    K = (1 << 24) - 32
+    W = K // 32
+    ones = torch.full((32, W), -1, dtype=torch.int32, device=DEV)
+    zeros = torch.zeros((32, W), dtype=torch.int32, device=DEV)
+    half = ones.clone()
+    half[:, ::2] = 0
+    pb = (W // 2) * 32
+    w_neg, w_pos = lk.tile_from_logical(ones, K), lk.tile_from_logical(zeros, K)
+    p1, p0, ph = lk.tile_from_logical(ones, K), lk.tile_from_logical(zeros, K), lk.tile_from_logical(half, K)
+    tern = lambda nz, sg: lk.PackedBits(nz.data, sg.data.clone(), 1, nz.rows, nz.K)      # planes: nonzero, sign & nonzero
+    variant = force_kernel(B.KERNEL_MFMA_128x256T, VARIANT_MFMA_F4)
+
+    def run(w, x):
+        out = lk.bgemm_packed_forward(w, x, MODE_BWTA, torch.int32, 1, variant)
+        lo, hi = int(out.min()), int(out.max())
+        assert lo == hi, (lo, hi)
+        return lo
+    assert run(w_neg, tern(p1, p1)) == K and run(w_pos, tern(p1, p1)) == -K          # t = -1 everywhere
+    assert run(w_neg, tern(p1, p0)) == -K and run(w_pos, tern(p1, p0)) == K          # t = +1 everywhere
+    assert run(w_neg, tern(p0, p0)) == 0
+    assert run(w_neg, tern(ph, ph)) == pb and run(w_pos, tern(ph, p0)) == pb
+
+
 KERNELS_FOR_SCALES = dict({"mfma " + t: (TILES[t], 96) for t in TILES},
                           **{"split-K in the block": (B.KERNEL_SKINNY_SPLITK, 96), "four pieces": (B.KERNEL_SKINNY_QUAD, 96),
                              "stream": (B.KERNEL_SKINNY_STREAM, 20), "popcount": (B.KERNEL_SKINNY_POPC, 2), "valu": (None, 96)})
