@@ -329,6 +329,25 @@ def test_signed_ternary_tile_batched_and_what_it_refuses():
         lk.bgemm_packed_forward(wp, xt, MODE_BWTA, torch.int32, 1, force_kernel(B.KERNEL_MFMA_128x256T, VARIANT_MFMA))   # the int8 engine
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_signed_ternary_tile_random_shapes(seed):
+    """Seeded random shapes, ragged in every dimension (K from one bit to a dozen K-tiles, batches of one to three), sparse
+    and dense ternary rows: the forced signed tile against the dense product, int32 and fp16."""
+    rng = np.random.default_rng(9100 + seed)
+    variant = force_kernel(B.KERNEL_MFMA_128x256T, VARIANT_MFMA_F4)
+    for _ in range(4):
+        Bn, M, N = int(rng.integers(1, 4)), int(rng.integers(1, 700)), int(rng.integers(1, 400))
+        K = int(rng.choice([1, 31, 64, 255, 256, 257, int(rng.integers(1, 3000))]))
+        w, t = pm1(rng, Bn, M, K), tern(rng, Bn, N, K)
+        t[rng.random(t.shape) < rng.random()] = 0                      # from almost dense to almost empty
+        wp, xt = lk.pack_sign(to_dev(w)), lk.pack_ternary(to_dev(t))
+        want = dense(MODE_BWTA, w, t)
+        got = lk.bgemm_packed_forward(wp, xt, MODE_BWTA, torch.int32, 1, variant).cpu().numpy()
+        assert (got == want).all(), (Bn, M, N, K)
+        got = lk.bgemm_packed_forward(wp, xt, MODE_BWTA, torch.half, 1, variant).cpu().numpy()
+        assert (bits_of(got) == bits_of(f16_of(want))).all(), (Bn, M, N, K)
+
+
 @pytest.mark.parametrize("M,N,K", [(4096 + 5, 2048 + 3, 17 * 256 - 7), (11008, 512, 4096)])
 def test_signed_ternary_tile_where_the_library_picks_it(oracle, M, N, K):
     """No forcing: prefill-sized BWTA products go to the signed tile on the fp4 engine (the library's choice) and to the
